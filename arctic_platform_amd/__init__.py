@@ -1,0 +1,32 @@
+"""MI355X-native forest cascade decode attention (ZoRRo inference path)."""
+
+from .config import ModelConfig, build_model_config, parse_arctic_inference_rollout, validate_fca_support
+from .kv_layout import BLOCK_SIZE, convert_cache, kv_cache_shape, pack_blocks, unpack_blocks
+
+__all__ = [
+    "BLOCK_SIZE",
+    "ModelConfig",
+    "build_model_config",
+    "parse_arctic_inference_rollout",
+    "validate_fca_support",
+    "kv_cache_shape",
+    "pack_blocks",
+    "unpack_blocks",
+    "convert_cache",
+    "build_forest_metadata",
+    "forest_cascade_decode",
+]
+
+
+def __getattr__(name):
+    # operators need the HIP library; resolve them lazily so the flag parser and layout
+    # helpers stay importable in a process that only builds or inspects
+    if name in ("build_forest_metadata", "ForestMetadata"):
+        from . import forest
+
+        return getattr(forest, name)
+    if name in ("forest_cascade_decode", "prefix_pass", "suffix_pass", "merge_partials"):
+        from . import ops
+
+        return getattr(ops, name)
+    raise AttributeError(name)

@@ -1,0 +1,221 @@
+// C ABI of libzorro_fca.so (declared in include/zorro_fca.h): argument checks and launches.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "fca_common.h"
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail(FCA_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+int check_plan(const fca_plan* p) {
+  if (!p) return fail(FCA_ERR_INVALID_ARG, "plan is NULL");
+  if (p->num_seqs < 1) return fail(FCA_ERR_INVALID_ARG, "num_seqs must be >= 1, got %d", p->num_seqs);
+  if (p->max_blocks < 1) return fail(FCA_ERR_INVALID_ARG, "max_blocks must be >= 1, got %d", p->max_blocks);
+  if (p->block_size != FCA_BLOCK_SIZE)
+    return fail(FCA_ERR_UNSUPPORTED, "block_size %d is not supported (only %d)", p->block_size, FCA_BLOCK_SIZE);
+  if (p->head_dim != 64 && p->head_dim != 128)
+    return fail(FCA_ERR_UNSUPPORTED, "head_dim %d is not supported (64 or 128)", p->head_dim);
+  if (p->num_kv_heads < 1 || p->num_q_heads < p->num_kv_heads || p->num_q_heads % p->num_kv_heads)
+    return fail(FCA_ERR_INVALID_ARG, "num_q_heads %d must be a positive multiple of num_kv_heads %d", p->num_q_heads,
+                p->num_kv_heads);
+  if (p->rows_per_item != 32 && p->rows_per_item != 64)
+    return fail(FCA_ERR_UNSUPPORTED, "rows_per_item %d is not supported (32 or 64)", p->rows_per_item);
+  if (p->num_q_heads / p->num_kv_heads > p->rows_per_item)
+    return fail(FCA_ERR_UNSUPPORTED, "GQA group %d exceeds rows_per_item %d", p->num_q_heads / p->num_kv_heads,
+                p->rows_per_item);
+  if (p->chunk_tokens < fca::kTile || p->chunk_tokens > fca::kMaxChunk || p->chunk_tokens % fca::kTile)
+    return fail(FCA_ERR_INVALID_ARG, "chunk_tokens %d must be a multiple of %d in [%d, %d]", p->chunk_tokens, fca::kTile,
+                fca::kTile, fca::kMaxChunk);
+  if (p->max_levels < 0 || p->max_levels > FCA_MAX_LEVELS)
+    return fail(FCA_ERR_INVALID_ARG, "max_levels %d must be in [0, %d]", p->max_levels, FCA_MAX_LEVELS);
+  const fca::MetaLayout L = fca::make_layout(*p);
+  if (L.max_items * p->num_kv_heads > 0x7fffffffLL || L.total > 0x7fffffffLL)
+    return fail(FCA_ERR_UNSUPPORTED, "batch too large for 32-bit work indices");
+  return FCA_OK;
+}
+
+int check_tensors(const fca_plan* p, const fca_tensors* t) {
+  if (!t) return fail(FCA_ERR_INVALID_ARG, "tensors is NULL");
+  if (!t->q_dev || !t->k_cache_dev || !t->v_cache_dev || !t->block_table_dev)
+    return fail(FCA_ERR_INVALID_ARG, "q, k_cache, v_cache and block_table must be non-NULL");
+  if (t->kv_dtype != FCA_BF16 && t->kv_dtype != FCA_FP8_E4M3)
+    return fail(FCA_ERR_UNSUPPORTED, "kv_dtype %d is not supported (bf16 or fp8 e4m3)", t->kv_dtype);
+  const int esz = t->kv_dtype == FCA_FP8_E4M3 ? 1 : 2;
+  if ((reinterpret_cast<uintptr_t>(t->q_dev) & 15) || (t->q_seq_stride % 8) || (t->q_head_stride % 8))
+    return fail(FCA_ERR_INVALID_ARG, "q must be 16-byte aligned with strides that are multiples of 8 elements");
+  if ((reinterpret_cast<uintptr_t>(t->k_cache_dev) & 15) || (reinterpret_cast<uintptr_t>(t->v_cache_dev) & 15) ||
+      (t->kv_block_stride * esz) % 16 || (t->kv_head_stride * esz) % 16)
+    return fail(FCA_ERR_INVALID_ARG, "KV cache planes must be 16-byte aligned with 16-byte-multiple strides");
+  if (t->kv_head_stride < (int64_t)FCA_BLOCK_SIZE * p->head_dim)
+    return fail(FCA_ERR_INVALID_ARG, "kv_head_stride %lld is smaller than one tile (%d elements)",
+                (long long)t->kv_head_stride, FCA_BLOCK_SIZE * p->head_dim);
+  if (t->block_table_stride < p->max_blocks)
+    return fail(FCA_ERR_INVALID_ARG, "block_table_stride %lld is smaller than max_blocks %d",
+                (long long)t->block_table_stride, p->max_blocks);
+  return FCA_OK;
+}
+
+fca::AttendParams attend_params(const fca_plan* p, const fca_tensors* t, void* meta, float* po, float* pl, int select) {
+  const fca::MetaLayout L = fca::make_layout(*p);
+  const int esz = t->kv_dtype == FCA_FP8_E4M3 ? 1 : 2;
+  fca::AttendParams a{};
+  a.q = t->q_dev;
+  a.q_seq_stride = t->q_seq_stride;
+  a.q_head_stride = t->q_head_stride;
+  a.k_cache = static_cast<const char*>(t->k_cache_dev);
+  a.v_cache = static_cast<const char*>(t->v_cache_dev);
+  a.kv_block_bytes = t->kv_block_stride * esz;
+  a.kv_head_bytes = t->kv_head_stride * esz;
+  a.block_table = t->block_table_dev;
+  a.bt_stride = t->block_table_stride;
+  a.k_scale = t->k_scale_dev;
+  a.v_scale = t->v_scale_dev;
+  a.scale = t->softmax_scale;
+  a.meta = static_cast<int32_t*>(meta);
+  a.off_header = L.header;
+  a.off_items = L.items;
+  a.off_members = L.members;
+  a.partial_out = po;
+  a.partial_lse = pl;
+  a.num_q_heads = p->num_q_heads;
+  a.num_kv_heads = p->num_kv_heads;
+  a.group = p->num_q_heads / p->num_kv_heads;
+  a.max_partials = (int32_t)L.max_partials;
+  a.select = select;
+  return a;
+}
+
+int run_attend(const fca_plan* p, const fca_tensors* t, void* meta, float* po, float* pl, int select, void* stream) {
+  if (int rc = check_plan(p)) return rc;
+  if (int rc = check_tensors(p, t)) return rc;
+  if (!meta || !po || !pl) return fail(FCA_ERR_INVALID_ARG, "metadata and partial workspaces must be non-NULL");
+  const fca::AttendParams a = attend_params(p, t, meta, po, pl, select);
+  hipError_t e = fca::launch_attend(a, *p, t->kv_dtype, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? FCA_OK : hip_fail(e, "attention pass launch");
+}
+
+int run_merge(const fca_plan* p, const void* meta, const float* po, const float* pl, void* out, int64_t oss, int64_t ohs,
+              int32_t out_dtype, float* lse, void* stream) {
+  if (int rc = check_plan(p)) return rc;
+  if (!meta || !po || !pl || !out) return fail(FCA_ERR_INVALID_ARG, "metadata, partials and out must be non-NULL");
+  if (out_dtype != FCA_BF16 && out_dtype != FCA_F32)
+    return fail(FCA_ERR_UNSUPPORTED, "out dtype %d is not supported (bf16 or f32)", out_dtype);
+  const fca::MetaLayout L = fca::make_layout(*p);
+  fca::MergeParams m{};
+  m.seq_npart = static_cast<const int32_t*>(meta) + L.seq_npart;
+  m.partial_out = po;
+  m.partial_lse = pl;
+  m.out = out;
+  m.out_seq_stride = oss;
+  m.out_head_stride = ohs;
+  m.lse = lse;
+  m.num_seqs = p->num_seqs;
+  m.num_q_heads = p->num_q_heads;
+  m.head_dim = p->head_dim;
+  m.max_partials = (int32_t)L.max_partials;
+  m.out_dtype = out_dtype;
+  hipError_t e = fca::launch_merge(m, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? FCA_OK : hip_fail(e, "merge launch");
+}
+
+}  // namespace
+
+extern "C" {
+
+int fca_version(void) { return FCA_VERSION; }
+
+const char* fca_last_error(void) { return g_error; }
+
+int fca_workspace_bytes(const fca_plan* plan, size_t* meta_bytes, size_t* partial_out_bytes, size_t* partial_lse_bytes) {
+  if (int rc = check_plan(plan)) return rc;
+  const fca::MetaLayout L = fca::make_layout(*plan);
+  const size_t slots = (size_t)plan->num_seqs * (size_t)L.max_partials;
+  if (meta_bytes) *meta_bytes = (size_t)L.total * sizeof(int32_t);
+  if (partial_out_bytes) *partial_out_bytes = slots * plan->num_q_heads * plan->head_dim * sizeof(float);
+  if (partial_lse_bytes) *partial_lse_bytes = slots * plan->num_q_heads * sizeof(float);
+  return FCA_OK;
+}
+
+int fca_meta_describe(const fca_plan* plan, fca_meta_layout* out) {
+  if (int rc = check_plan(plan)) return rc;
+  if (!out) return fail(FCA_ERR_INVALID_ARG, "layout is NULL");
+  const fca::MetaLayout L = fca::make_layout(*plan);
+  out->header = L.header;
+  out->seq_npart = L.seq_npart;
+  out->seq_leaf_blk = L.seq_leaf_blk;
+  out->node_rep = L.node_rep;
+  out->node_blk = L.node_blk;
+  out->node_nblk = L.node_nblk;
+  out->node_level = L.node_level;
+  out->node_moff = L.node_moff;
+  out->node_mcnt = L.node_mcnt;
+  out->node_ord = L.node_ord;
+  out->members = L.members;
+  out->items = L.items;
+  out->max_items = L.max_items;
+  out->max_partials = L.max_partials;
+  out->total_int32 = L.total;
+  return FCA_OK;
+}
+
+int fca_build_metadata(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,
+                       const int32_t* seq_lens_dev, void* meta_dev, void* stream) {
+  if (int rc = check_plan(plan)) return rc;
+  if (!block_table_dev || !seq_lens_dev || !meta_dev)
+    return fail(FCA_ERR_INVALID_ARG, "block_table, seq_lens and metadata workspace must be non-NULL");
+  if (block_table_stride < plan->max_blocks)
+    return fail(FCA_ERR_INVALID_ARG, "block_table_stride %lld is smaller than max_blocks %d",
+                (long long)block_table_stride, plan->max_blocks);
+  if (reinterpret_cast<uintptr_t>(meta_dev) & 15)
+    return fail(FCA_ERR_INVALID_ARG, "metadata workspace must be 16-byte aligned");
+  fca::BuildParams b{};
+  b.plan = *plan;
+  b.block_table = block_table_dev;
+  b.bt_stride = block_table_stride;
+  b.seq_lens = seq_lens_dev;
+  b.meta = static_cast<int32_t*>(meta_dev);
+  b.L = fca::make_layout(*plan);
+  hipError_t e = fca::launch_build(b, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? FCA_OK : hip_fail(e, "metadata builder launch");
+}
+
+int fca_prefix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev, float* partial_out_dev,
+                    float* partial_lse_dev, void* stream) {
+  return run_attend(plan, t, meta_dev, partial_out_dev, partial_lse_dev, 1, stream);
+}
+
+int fca_suffix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev, float* partial_out_dev,
+                    float* partial_lse_dev, void* stream) {
+  return run_attend(plan, t, meta_dev, partial_out_dev, partial_lse_dev, 2, stream);
+}
+
+int fca_merge(const fca_plan* plan, const void* meta_dev, const float* partial_out_dev, const float* partial_lse_dev,
+              void* out_dev, int64_t out_seq_stride, int64_t out_head_stride, int32_t out_dtype, float* lse_dev,
+              void* stream) {
+  return run_merge(plan, meta_dev, partial_out_dev, partial_lse_dev, out_dev, out_seq_stride, out_head_stride, out_dtype,
+                   lse_dev, stream);
+}
+
+int fca_decode_step(const fca_plan* plan, const fca_tensors* t, void* meta_dev, float* partial_out_dev,
+                    float* partial_lse_dev, void* out_dev, int64_t out_seq_stride, int64_t out_head_stride,
+                    int32_t out_dtype, float* lse_dev, void* stream) {
+  if (int rc = run_attend(plan, t, meta_dev, partial_out_dev, partial_lse_dev, 0, stream)) return rc;
+  return run_merge(plan, meta_dev, partial_out_dev, partial_lse_dev, out_dev, out_seq_stride, out_head_stride, out_dtype,
+                   lse_dev, stream);
+}
+
+}  // extern "C"

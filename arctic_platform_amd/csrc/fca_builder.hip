@@ -1,0 +1,320 @@
+// Forest metadata builder: one workgroup turns (block_table, seq_lens) into shared
+// nodes, member lists and a size-ordered work list, with no host round trip.
+//
+// Discovery is a level-by-level radix-tree construction.  At each level every still
+// active sequence is keyed by (parent node, physical block id at its current position);
+// sequences with equal keys elect the smallest index as leader, compare their rows
+// against the leader's to find the common run, and the minimum run over the group
+// becomes a shared node.  Members advance past the node and the next level regroups
+// them; sequences left alone become private leaves.  Grouping semantics (compare with
+// the group's first member, members ascending) follow the trainer's host-side discovery,
+// arctic_platform/rl/zorro_train/zorro_train.py:242-285.
+#include "fca_common.h"
+
+namespace fca {
+
+constexpr int kBuildThreads = 1024;
+constexpr unsigned long long kEmptyKey = ~0ull;
+
+// Exclusive prefix sum of in[0..n) into out[0..n) by the whole workgroup; returns the
+// total to every thread.  `in` may alias `out`.
+__device__ int block_exclusive_scan(const int* in, int* out, int n, int* lds) {
+  const int tid = threadIdx.x;
+  const int per = (n + kBuildThreads - 1) / kBuildThreads;
+  const int lo = min(tid * per, n), hi = min(lo + per, n);
+  int sum = 0;
+  for (int i = lo; i < hi; ++i) sum += in[i];
+  lds[tid] = sum;
+  __syncthreads();
+  for (int off = 1; off < kBuildThreads; off <<= 1) {
+    int v = tid >= off ? lds[tid - off] : 0;
+    __syncthreads();
+    lds[tid] += v;
+    __syncthreads();
+  }
+  int run = tid ? lds[tid - 1] : 0;
+  const int total = lds[kBuildThreads - 1];
+  for (int i = lo; i < hi; ++i) {
+    int v = in[i];
+    out[i] = run;
+    run += v;
+  }
+  __syncthreads();
+  return total;
+}
+
+__device__ inline unsigned hash_key(unsigned long long k) {
+  k ^= k >> 33;
+  k *= 0xff51afd7ed558ccdull;
+  k ^= k >> 29;
+  return (unsigned)k;
+}
+
+__global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p) {
+  __shared__ int lds_scan[kBuildThreads];
+  __shared__ int lds_hist[2 * kSizeBuckets];
+  __shared__ int lds_cursor[2 * kSizeBuckets];
+  __shared__ unsigned long long lds_tokens;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int nwaves = kBuildThreads / 64;
+  const int S = p.plan.num_seqs;
+  const int chunk = p.plan.chunk_tokens;
+  const int group = p.plan.num_q_heads / p.plan.num_kv_heads;
+  const int members_per_item = p.plan.rows_per_item / group;
+  const MetaLayout& L = p.L;
+  int32_t* meta = p.meta;
+  int32_t* hdr = meta + L.header;
+  int* pos = meta + L.s_pos;
+  int* par = meta + L.s_par;
+  int* ord = meta + L.s_ord;
+  int* nfull = meta + L.s_nfull;
+  int* leader = meta + L.s_leader;
+  int* lcp = meta + L.s_lcp;
+  int* run = meta + L.s_run;
+  int* cnt = meta + L.s_cnt;
+  int* nodeof = meta + L.s_node;
+  int* slot = meta + L.s_slot;
+  int* tmp0 = meta + L.s_tmp0;
+  int* tmp1 = meta + L.s_tmp1;
+  unsigned long long* hkeys = reinterpret_cast<unsigned long long*>(meta + L.hash_keys);
+  int* hmin = meta + L.hash_min;
+  const int hsize = (int)L.hash_size;
+  int* members = meta + L.members;
+
+  if (tid < kHeaderInts) hdr[tid] = 0;
+  if (tid == 0) lds_tokens = 0;
+  for (int s = tid; s < S; s += kBuildThreads) {
+    int len = p.seq_lens[s];
+    if (len < 0 || len > p.plan.max_blocks * kBlock) {
+      atomicOr(&hdr[H_ERROR], 1);
+      len = max(0, min(len, p.plan.max_blocks * kBlock));
+    }
+    tmp1[s] = len;  // validated length, kept for the leaf pass
+    nfull[s] = p.plan.max_levels > 0 ? len / kBlock : 0;
+    pos[s] = 0;
+    par[s] = -1;
+    ord[s] = 0;
+  }
+  __syncthreads();
+
+  int node_base = 0, member_base = 0, levels = 0;
+  for (int level = 0; level < p.plan.max_levels; ++level) {
+    for (int i = tid; i < hsize; i += kBuildThreads) {
+      hkeys[i] = kEmptyKey;
+      hmin[i] = 0x7fffffff;
+    }
+    for (int s = tid; s < S; s += kBuildThreads) {
+      run[s] = 0x7fffffff;
+      cnt[s] = 0;
+      leader[s] = -1;
+      slot[s] = -1;
+    }
+    __syncthreads();
+    // Key every sequence that still has a full block at its position.  A sequence whose
+    // parent is -2 dropped out of sharing at an earlier level.
+    for (int s = tid; s < S; s += kBuildThreads) {
+      if (par[s] == -2 || pos[s] >= nfull[s]) continue;
+      unsigned blk = (unsigned)p.block_table[s * p.bt_stride + pos[s]];
+      unsigned long long key = ((unsigned long long)(unsigned)(par[s] + 1) << 32) | blk;
+      int h = hash_key(key) & (hsize - 1);
+      for (int probe = 0; probe < hsize; ++probe) {
+        unsigned long long prev = atomicCAS(&hkeys[h], kEmptyKey, key);
+        if (prev == kEmptyKey || prev == key) break;
+        h = (h + 1) & (hsize - 1);
+      }
+      slot[s] = h;
+      atomicMin(&hmin[h], s);
+    }
+    __syncthreads();
+    for (int s = tid; s < S; s += kBuildThreads) {
+      if (slot[s] >= 0) {
+        leader[s] = hmin[slot[s]];
+        lcp[s] = nfull[s] - pos[s];
+      }
+    }
+    __syncthreads();
+    // Common run with the leader: one wave per sequence, 256 positions per round.
+    for (int s = wave; s < S; s += nwaves) {
+      const int t = leader[s];
+      if (t < 0 || t == s) continue;
+      const int lim = min(nfull[s], nfull[t]) - pos[s];
+      const int32_t* row_s = p.block_table + s * p.bt_stride + pos[s];
+      const int32_t* row_t = p.block_table + t * p.bt_stride + pos[s];
+      int first = lim;
+      for (int j0 = 0; j0 < lim && first == lim; j0 += 256) {
+        int mine = lim;
+#pragma unroll
+        for (int u = 3; u >= 0; --u) {
+          int j = j0 + u * 64 + lane;
+          if (j < lim && row_s[j] != row_t[j]) mine = j;
+        }
+        for (int off = 32; off; off >>= 1) mine = min(mine, __shfl_xor(mine, off));
+        first = mine;
+      }
+      if (lane == 0) lcp[s] = min(lcp[s], first);
+    }
+    __syncthreads();
+    for (int s = tid; s < S; s += kBuildThreads) {
+      if (leader[s] >= 0) {
+        atomicMin(&run[leader[s]], lcp[s]);
+        atomicAdd(&cnt[leader[s]], 1);
+      }
+    }
+    __syncthreads();
+    for (int s = tid; s < S; s += kBuildThreads) {
+      const bool is_node = leader[s] == s && cnt[s] >= 2;
+      tmp0[s] = is_node ? 1 : 0;
+      nodeof[s] = is_node ? cnt[s] : 0;
+    }
+    __syncthreads();
+    const int new_nodes = block_exclusive_scan(tmp0, tmp0, S, lds_scan);
+    if (new_nodes == 0) break;
+    const int new_members = block_exclusive_scan(nodeof, nodeof, S, lds_scan);
+    ++levels;
+    for (int s = tid; s < S; s += kBuildThreads) {
+      if (leader[s] == s && cnt[s] >= 2) {
+        const int id = node_base + tmp0[s];
+        meta[L.node_rep + id] = s;
+        meta[L.node_blk + id] = pos[s];
+        meta[L.node_nblk + id] = run[s];
+        meta[L.node_level + id] = level;
+        meta[L.node_moff + id] = member_base + nodeof[s];
+        meta[L.node_mcnt + id] = cnt[s];
+        meta[L.node_ord + id] = ord[s];
+        tmp0[s] = id;
+        atomicAdd(&lds_tokens, (unsigned long long)run[s] * kBlock);
+      }
+    }
+    __syncthreads();
+    // Member lists in ascending sequence order: rank = members of the same leader below s.
+    for (int s = wave; s < S; s += nwaves) {
+      const int t = leader[s];
+      if (t < 0 || cnt[t] < 2) continue;
+      int below = 0;
+      for (int j0 = t; j0 < s; j0 += 64) {
+        int j = j0 + lane;
+        below += __popcll(__ballot(j < s && leader[j] == t));
+      }
+      if (lane == 0) members[meta[L.node_moff + tmp0[t]] + below] = s;
+    }
+    __syncthreads();
+    for (int s = tid; s < S; s += kBuildThreads) {
+      const int t = leader[s];
+      if (t >= 0 && cnt[t] >= 2) {
+        lcp[s] = run[t];  // advance amount, applied after the barrier (pos[t] is read by others)
+        par[s] = tmp0[t];
+      } else {
+        lcp[s] = 0;
+        par[s] = -2;
+      }
+    }
+    __syncthreads();
+    for (int s = tid; s < S; s += kBuildThreads) {
+      pos[s] += lcp[s];
+      ord[s] += num_chunks_for(lcp[s] * kBlock, chunk);
+    }
+    node_base += new_nodes;
+    member_base += new_members;
+    __syncthreads();
+  }
+
+  // Private leaves and per-sequence partial counts.  Node index space for the work list:
+  // shared nodes [0, node_base), then leaf of sequence s at node_base + s.
+  const int leaf_members = member_base;
+  for (int s = tid; s < S; s += kBuildThreads) {
+    const int tokens = tmp1[s] - pos[s] * kBlock;
+    meta[L.seq_leaf_blk + s] = pos[s];
+    meta[L.seq_npart + s] = ord[s] + num_chunks_for(tokens, chunk);
+    members[leaf_members + s] = s;
+    atomicAdd(&lds_tokens, (unsigned long long)tokens);
+  }
+  if (tid < 2 * kSizeBuckets) {
+    lds_hist[tid] = 0;
+    lds_cursor[tid] = 0;
+  }
+  __syncthreads();
+
+  // Work list: one item per (node chunk, tile of members), shared items first, each
+  // class in descending size order so the dynamic queue ends on the small ones.
+  const int total_nodes = node_base + S;
+  auto node_fields = [&](int n, int& rep, int& blk, int& tokens, int& moff, int& mcnt, int& o) {
+    if (n < node_base) {
+      rep = meta[L.node_rep + n];
+      blk = meta[L.node_blk + n];
+      tokens = meta[L.node_nblk + n] * kBlock;
+      moff = meta[L.node_moff + n];
+      mcnt = meta[L.node_mcnt + n];
+      o = meta[L.node_ord + n];
+    } else {
+      const int s = n - node_base;
+      rep = s;
+      blk = pos[s];
+      tokens = tmp1[s] - pos[s] * kBlock;
+      moff = leaf_members + s;
+      mcnt = 1;
+      o = ord[s];
+    }
+  };
+  auto bucket_of = [&](int cls, int tok_len) {
+    int sb = min(kSizeBuckets - 1, (tok_len * kSizeBuckets - 1) / chunk);
+    return cls * kSizeBuckets + (kSizeBuckets - 1 - sb);
+  };
+  for (int n = tid; n < total_nodes; n += kBuildThreads) {
+    int rep, blk, tokens, moff, mcnt, o;
+    node_fields(n, rep, blk, tokens, moff, mcnt, o);
+    const int clen = chunk_len_for(tokens, chunk);
+    const int nch = num_chunks_for(tokens, chunk);
+    const int ntile = (mcnt + members_per_item - 1) / members_per_item;
+    const int cls = n < node_base ? 0 : 1;
+    for (int c = 0; c < nch; ++c) {
+      const int tl = min(clen, tokens - c * clen);
+      atomicAdd(&lds_hist[bucket_of(cls, tl)], ntile);
+    }
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int acc = 0, shared_items = 0;
+    for (int b = 0; b < 2 * kSizeBuckets; ++b) {
+      if (b == kSizeBuckets) shared_items = acc;
+      int v = lds_hist[b];
+      lds_hist[b] = acc;
+      acc += v;
+    }
+    hdr[H_ITEMS] = acc;
+    hdr[H_SHARED_ITEMS] = shared_items;
+    hdr[H_NODES] = node_base;
+    hdr[H_LEVELS] = levels;
+    hdr[H_TOKENS_LO] = (int)(lds_tokens & 0xffffffffull);
+    hdr[H_TOKENS_HI] = (int)(lds_tokens >> 32);
+    if (acc > (int)L.max_items) atomicOr(&hdr[H_ERROR], 2);
+  }
+  __syncthreads();
+  int32_t* items = meta + L.items;
+  for (int n = tid; n < total_nodes; n += kBuildThreads) {
+    int rep, blk, tokens, moff, mcnt, o;
+    node_fields(n, rep, blk, tokens, moff, mcnt, o);
+    const int clen = chunk_len_for(tokens, chunk);
+    const int nch = num_chunks_for(tokens, chunk);
+    const int ntile = (mcnt + members_per_item - 1) / members_per_item;
+    const int cls = n < node_base ? 0 : 1;
+    for (int c = 0; c < nch; ++c) {
+      const int tl = min(clen, tokens - c * clen);
+      const int b = bucket_of(cls, tl);
+      const int at = lds_hist[b] + atomicAdd(&lds_cursor[b], ntile);
+      for (int r = 0; r < ntile; ++r) {
+        if (at + r >= (int)L.max_items) break;
+        int4* rec = reinterpret_cast<int4*>(items + (int64_t)(at + r) * kItemInts);
+        rec[0] = make_int4(rep, blk + c * (clen / kBlock), tl, moff + r * members_per_item);
+        rec[1] = make_int4(min(members_per_item, mcnt - r * members_per_item), o + c, n, 0);
+      }
+    }
+  }
+}
+
+hipError_t launch_build(const BuildParams& p, hipStream_t stream) {
+  hipLaunchKernelGGL(fca_build_kernel, dim3(1), dim3(kBuildThreads), 0, stream, p);
+  return hipGetLastError();
+}
+
+}  // namespace fca

@@ -1,0 +1,152 @@
+// Shared definitions of the forest-cascade kernels: metadata workspace layout and
+// launch parameter blocks.  Internal to libzorro_fca.so; the public ABI is zorro_fca.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/zorro_fca.h"
+
+namespace fca {
+
+constexpr int kBlock = FCA_BLOCK_SIZE;   // tokens per physical KV block
+constexpr int kTile = 32;                // tokens per MFMA tile (two blocks)
+constexpr int kMaxChunk = 1024;          // one lane of a wave holds one block id of a chunk
+constexpr int kItemInts = 8;             // int32 per work-item record
+constexpr int kSizeBuckets = 32;         // size classes for the descending work-list order
+constexpr int kHeaderInts = 16;
+
+enum HeaderSlot {
+  H_ITEMS = 0,
+  H_SHARED_ITEMS = 1,
+  H_NODES = 2,
+  H_TICKET = 3,
+  H_DONE = 4,
+  H_ERROR = 5,
+  H_TOKENS_LO = 6,
+  H_TOKENS_HI = 7,
+  H_LEVELS = 8
+};
+
+// Offsets in int32 units from the start of the metadata workspace.
+struct MetaLayout {
+  int64_t header;
+  int64_t seq_npart, seq_leaf_blk;
+  int64_t node_rep, node_blk, node_nblk, node_level, node_moff, node_mcnt, node_ord;
+  int64_t members;
+  int64_t items;
+  // builder scratch
+  int64_t s_pos, s_par, s_ord, s_nfull, s_leader, s_lcp, s_run, s_cnt, s_node, s_slot, s_tmp0, s_tmp1, s_nitems;
+  int64_t hash_keys;  // 64-bit keys, 2 int32 each
+  int64_t hash_min;
+  int64_t hash_size;  // entries (power of two)
+  int64_t max_items;
+  int64_t max_partials;
+  int64_t total;
+};
+
+inline __host__ __device__ int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+inline __host__ MetaLayout make_layout(const fca_plan& p) {
+  MetaLayout L{};
+  const int64_t S = p.num_seqs;
+  int64_t off = 0;
+  auto take = [&](int64_t n) {
+    int64_t at = off;
+    off = align_up(off + n, 4);  // keep every array 16-byte aligned
+    return at;
+  };
+  L.max_partials = (int64_t)p.max_blocks * kBlock / p.chunk_tokens + p.max_levels + 1;
+  L.max_items = S * L.max_partials;
+  L.header = take(kHeaderInts);
+  L.seq_npart = take(S);
+  L.seq_leaf_blk = take(S);
+  L.node_rep = take(S);
+  L.node_blk = take(S);
+  L.node_nblk = take(S);
+  L.node_level = take(S);
+  L.node_moff = take(S);
+  L.node_mcnt = take(S);
+  L.node_ord = take(S);
+  L.members = take(S * (FCA_MAX_LEVELS + 1));
+  L.items = take(L.max_items * kItemInts);
+  L.s_pos = take(S);
+  L.s_par = take(S);
+  L.s_ord = take(S);
+  L.s_nfull = take(S);
+  L.s_leader = take(S);
+  L.s_lcp = take(S);
+  L.s_run = take(S);
+  L.s_cnt = take(S);
+  L.s_node = take(S);
+  L.s_slot = take(S);
+  L.s_tmp0 = take(S);
+  L.s_tmp1 = take(S);
+  L.s_nitems = take(2 * S);
+  int64_t hs = 64;
+  while (hs < 4 * S) hs <<= 1;
+  L.hash_size = hs;
+  L.hash_keys = take(2 * hs);
+  L.hash_min = take(hs);
+  L.total = off;
+  return L;
+}
+
+// Chunks a node of `tokens` KV tokens is split into, and their common length: an even
+// split rounded up to whole MFMA tiles, so no chunk is a sliver.
+inline __host__ __device__ int chunk_len_for(int tokens, int chunk_tokens) {
+  if (tokens <= 0) return 0;
+  int n = (tokens + chunk_tokens - 1) / chunk_tokens;
+  int len = (tokens + n - 1) / n;
+  return (len + kTile - 1) / kTile * kTile;
+}
+inline __host__ __device__ int num_chunks_for(int tokens, int chunk_tokens) {
+  if (tokens <= 0) return 0;
+  int len = chunk_len_for(tokens, chunk_tokens);
+  return (tokens + len - 1) / len;
+}
+
+struct BuildParams {
+  fca_plan plan;
+  const int32_t* block_table;
+  int64_t bt_stride;
+  const int32_t* seq_lens;
+  int32_t* meta;
+  MetaLayout L;
+};
+
+struct AttendParams {
+  const void* q;
+  int64_t q_seq_stride, q_head_stride;  // elements
+  const char* k_cache;
+  const char* v_cache;
+  int64_t kv_block_bytes, kv_head_bytes;
+  const int32_t* block_table;
+  int64_t bt_stride;
+  const float* k_scale;
+  const float* v_scale;
+  float scale;
+  int32_t* meta;
+  int64_t off_header, off_items, off_members;
+  float* partial_out;
+  float* partial_lse;
+  int32_t num_q_heads, num_kv_heads, group;  // group = Hq / Hkv
+  int32_t max_partials;
+  int32_t select;  // 0 all items, 1 shared only, 2 leaves only
+};
+
+struct MergeParams {
+  const int32_t* seq_npart;
+  const float* partial_out;
+  const float* partial_lse;
+  void* out;
+  int64_t out_seq_stride, out_head_stride;
+  float* lse;
+  int32_t num_seqs, num_q_heads, head_dim, max_partials, out_dtype;
+};
+
+hipError_t launch_build(const BuildParams& p, hipStream_t stream);
+hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, hipStream_t stream);
+hipError_t launch_merge(const MergeParams& p, hipStream_t stream);
+
+}  // namespace fca

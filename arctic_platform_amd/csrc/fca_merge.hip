@@ -1,0 +1,68 @@
+// Log-sum-exp merge of the per-sequence partial results (tree levels x split-K chunks).
+// Running-max formulation with guards for empty partials, as the online log-sum-exp of
+// arctic_platform/model/implementations/qwen35/models/layers/lm_head.py:190-202.
+#include <hip/hip_bf16.h>
+
+#include "fca_common.h"
+
+namespace fca {
+
+constexpr int kMergeThreads = 256;
+constexpr int kLanesPerRow = 32;
+
+// 32 lanes per (sequence, query head) row; each lane owns D / 32 adjacent channels.
+template <int D>
+__global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p) {
+  constexpr int V = D / kLanesPerRow;
+  const int row = blockIdx.x * (kMergeThreads / kLanesPerRow) + threadIdx.x / kLanesPerRow;
+  const int sub = threadIdx.x % kLanesPerRow;
+  if (row >= p.num_seqs * p.num_q_heads) return;
+  const int s = row / p.num_q_heads, hq = row - s * p.num_q_heads;
+  const int np = p.seq_npart[s];
+  const int64_t base = (int64_t)s * p.max_partials;
+
+  float m = -INFINITY;
+  for (int i = 0; i < np; ++i) m = fmaxf(m, p.partial_lse[(base + i) * p.num_q_heads + hq]);
+  float acc[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) acc[e] = 0.f;
+  float wsum = 0.f;
+  if (m > -INFINITY) {
+    for (int i = 0; i < np; ++i) {
+      const int64_t pr = (base + i) * p.num_q_heads + hq;
+      const float l = p.partial_lse[pr];
+      if (!(l > -INFINITY)) continue;  // empty partial: weight 0, its output is not read
+      const float w = __expf(l - m);
+      wsum += w;
+      const float* src = p.partial_out + pr * D + sub * V;
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] += w * src[e];
+    }
+  }
+  const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
+  const int64_t o = (int64_t)s * p.out_seq_stride + (int64_t)hq * p.out_head_stride + sub * V;
+  if (p.out_dtype == FCA_F32) {
+    float* dst = reinterpret_cast<float*>(p.out) + o;
+#pragma unroll
+    for (int e = 0; e < V; ++e) dst[e] = acc[e] * inv;
+  } else {
+    __hip_bfloat16* dst = reinterpret_cast<__hip_bfloat16*>(p.out) + o;
+#pragma unroll
+    for (int e = 0; e < V; ++e) dst[e] = __float2bfloat16(acc[e] * inv);
+  }
+  if (p.lse && sub == 0) p.lse[row] = wsum > 0.f ? m + __logf(wsum) : -INFINITY;
+}
+
+hipError_t launch_merge(const MergeParams& p, hipStream_t stream) {
+  const int rows = p.num_seqs * p.num_q_heads;
+  const int per_block = kMergeThreads / kLanesPerRow;
+  const int grid = (rows + per_block - 1) / per_block;
+  if (grid == 0) return hipSuccess;
+  if (p.head_dim == 128)
+    hipLaunchKernelGGL(fca_merge_kernel<128>, dim3(grid), dim3(kMergeThreads), 0, stream, p);
+  else
+    hipLaunchKernelGGL(fca_merge_kernel<64>, dim3(grid), dim3(kMergeThreads), 0, stream, p);
+  return hipGetLastError();
+}
+
+}  // namespace fca

@@ -1,0 +1,189 @@
+"""Forest metadata: block tables -> shared nodes, member lists and the work list.
+
+Host-side face of ``fca_build_metadata``.  The discovery runs on the device with no
+host synchronisation; this module only sizes the workspaces and, for inspection and
+tests, decodes a built workspace back into Python lists.
+
+The grouping rule mirrors the trainer's prompt-group discovery
+(arctic_platform/rl/zorro_train/zorro_train.py:242-285): rows are compared with the first
+member of a group, groups come out in first-seen order, members ascending.  Here the rows
+are leading runs of physical block ids and the rule is applied level by level.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import dataclasses
+
+import torch
+
+from . import _lib
+from .kv_layout import BLOCK_SIZE
+
+ITEM_INTS = 8
+
+
+def _stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+@dataclasses.dataclass
+class ForestMetadata:
+    plan: _lib.FcaPlan
+    layout: _lib.FcaMetaLayout
+    meta: torch.Tensor  # int32 workspace on the device
+    partial_out: torch.Tensor  # fp32 [S * max_partials, Hq, D]
+    partial_lse: torch.Tensor  # fp32 [S * max_partials, Hq]
+    block_table: torch.Tensor
+    seq_lens: torch.Tensor
+
+    # ---- inspection (synchronises; not for the decode loop) -------------------------
+    def header(self) -> dict:
+        h = self.meta[self.layout.header : self.layout.header + 16].tolist()
+        return dict(
+            items=h[0],
+            shared_items=h[1],
+            shared_nodes=h[2],
+            ticket=h[3],
+            done=h[4],
+            error=h[5],
+            unique_tokens=(h[6] & 0xFFFFFFFF) | (h[7] << 32),
+            levels=h[8],
+        )
+
+    def check(self) -> None:
+        err = self.header()["error"]
+        if err & 1:
+            raise ValueError("a sequence length is negative or exceeds max_blocks * block_size")
+        if err & 2:
+            raise RuntimeError("work list overflowed its reserved size")
+
+    def nodes(self) -> list:
+        L, m = self.layout, self.meta.cpu()
+        n = int(m[L.header + 2])
+        members = m[L.members :]
+        out = []
+        for i in range(n):
+            off, cnt = int(m[L.node_moff + i]), int(m[L.node_mcnt + i])
+            out.append(
+                dict(
+                    members=members[off : off + cnt].tolist(),
+                    rep=int(m[L.node_rep + i]),
+                    blk_start=int(m[L.node_blk + i]),
+                    num_blocks=int(m[L.node_nblk + i]),
+                    level=int(m[L.node_level + i]),
+                    ord=int(m[L.node_ord + i]),
+                )
+            )
+        return out
+
+    def leaves(self) -> list:
+        L, m = self.layout, self.meta.cpu()
+        s = self.plan.num_seqs
+        lens = self.seq_lens.cpu().tolist()
+        blk = m[L.seq_leaf_blk : L.seq_leaf_blk + s].tolist()
+        return [dict(blk_start=blk[i], tokens=lens[i] - blk[i] * BLOCK_SIZE) for i in range(s)]
+
+    def seq_num_partials(self) -> list:
+        L = self.layout
+        return self.meta[L.seq_npart : L.seq_npart + self.plan.num_seqs].tolist()
+
+    def items(self) -> list:
+        L, m = self.layout, self.meta.cpu()
+        n = int(m[L.header])
+        shared = int(m[L.header + 1])
+        rec = m[L.items : L.items + n * ITEM_INTS].view(n, ITEM_INTS).tolist()
+        members = m[L.members :]
+        out = []
+        for i, r in enumerate(rec):
+            out.append(
+                dict(
+                    rep=r[0],
+                    blk_start=r[1],
+                    tok_len=r[2],
+                    members=members[r[3] : r[3] + r[4]].tolist(),
+                    ord=r[5],
+                    node=r[6],
+                    shared=i < shared,
+                )
+            )
+        return out
+
+
+def make_plan(
+    num_seqs, max_blocks, num_q_heads, num_kv_heads, head_dim, *, chunk_tokens=512, rows_per_item=32, max_levels=4
+) -> _lib.FcaPlan:
+    return _lib.FcaPlan(
+        num_seqs, max_blocks, num_q_heads, num_kv_heads, head_dim, BLOCK_SIZE, chunk_tokens, rows_per_item, max_levels
+    )
+
+
+def build_forest_metadata(
+    block_table: torch.Tensor,
+    seq_lens: torch.Tensor,
+    *,
+    num_q_heads: int,
+    num_kv_heads: int,
+    head_dim: int,
+    block_size: int = BLOCK_SIZE,
+    chunk_tokens: int = 512,
+    rows_per_item: int = 32,
+    cascade: bool = True,
+    max_levels: int = 4,
+    out: ForestMetadata | None = None,
+) -> ForestMetadata:
+    """Discover the shared-prefix forest of a decode batch on the device.
+
+    ``cascade=False`` turns sharing off: every sequence becomes one private node over its
+    whole block-table row, which makes the same kernels a plain paged decode attention.
+    Pass a previous result as ``out`` to rebuild into the same workspaces (no allocation).
+    """
+    if block_size != BLOCK_SIZE:
+        raise ValueError(f"block_size must be {BLOCK_SIZE}")
+    if block_table.dtype != torch.int32 or seq_lens.dtype != torch.int32:
+        raise TypeError("block_table and seq_lens must be int32")
+    if block_table.dim() != 2 or block_table.stride(1) != 1 or seq_lens.shape != (block_table.shape[0],):
+        raise ValueError("block_table must be [num_seqs, max_blocks] with contiguous rows and seq_lens [num_seqs]")
+    if not block_table.is_cuda:
+        raise RuntimeError("forest metadata is built on the GPU; block_table must be a device tensor")
+    lib = _lib.load_library()
+    plan = make_plan(
+        block_table.shape[0],
+        block_table.shape[1],
+        num_q_heads,
+        num_kv_heads,
+        head_dim,
+        chunk_tokens=chunk_tokens,
+        rows_per_item=rows_per_item,
+        max_levels=max_levels if cascade else 0,
+    )
+    if out is not None and bytes(out.plan) == bytes(plan):
+        md = dataclasses.replace(out, block_table=block_table, seq_lens=seq_lens)
+    else:
+        layout = _lib.FcaMetaLayout()
+        _lib.check(lib.fca_meta_describe(ctypes.byref(plan), ctypes.byref(layout)))
+        nm, no, nl = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+        _lib.check(lib.fca_workspace_bytes(ctypes.byref(plan), ctypes.byref(nm), ctypes.byref(no), ctypes.byref(nl)))
+        dev = block_table.device
+        slots = plan.num_seqs * layout.max_partials
+        md = ForestMetadata(
+            plan=plan,
+            layout=layout,
+            meta=torch.empty(nm.value // 4, dtype=torch.int32, device=dev),
+            partial_out=torch.empty(slots, num_q_heads, head_dim, dtype=torch.float32, device=dev),
+            partial_lse=torch.empty(slots, num_q_heads, dtype=torch.float32, device=dev),
+            block_table=block_table,
+            seq_lens=seq_lens,
+        )
+        assert md.partial_out.numel() * 4 == no.value and md.partial_lse.numel() * 4 == nl.value
+    _lib.check(
+        lib.fca_build_metadata(
+            ctypes.byref(md.plan),
+            block_table.data_ptr(),
+            block_table.stride(0),
+            seq_lens.data_ptr(),
+            md.meta.data_ptr(),
+            _stream_ptr(block_table.device),
+        )
+    )
+    return md

@@ -1,0 +1,147 @@
+"""Forest cascade decode attention operator.
+
+``forest_cascade_decode`` is what an attention backend's per-layer ``forward`` calls for a
+decode batch: one query token per sequence against the paged KV cache, using metadata
+built once per scheduler step by ``build_forest_metadata``.  It sits where the platform's
+sampling engine runs attention after ``ReplicaPool.generate``
+(arctic_platform/common/ray_server.py:921-933) when the job was started with
+``zorro_inference.enable`` (arctic_platform/common/utils/server_models.py:123-140).
+
+Semantics: plain softmax attention with grouped KV heads, scale passed in, no mask
+(arctic_platform/model/implementations/qwen35/models/qwen3_5_moe/modeling_qwen3_5_moe.py:
+368-373, :385, :440-454); ``lse`` is the natural-log sum of exponentiated scaled scores.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _lib
+from .forest import ForestMetadata, _stream_ptr
+from .kv_layout import BLOCK_SIZE
+
+
+def _tensors(q, kv_cache, meta: ForestMetadata, scale, k_scale, v_scale) -> _lib.FcaTensors:
+    plan = meta.plan
+    if q.dtype != torch.bfloat16:
+        raise TypeError("q must be bfloat16")
+    if q.shape != (plan.num_seqs, plan.num_q_heads, plan.head_dim) or q.stride(2) != 1:
+        raise ValueError(f"q must be [{plan.num_seqs}, {plan.num_q_heads}, {plan.head_dim}] with contiguous head_dim")
+    if kv_cache.dtype == torch.bfloat16:
+        kv_dtype = _lib.FCA_BF16
+    elif kv_cache.dtype == torch.float8_e4m3fn:
+        kv_dtype = _lib.FCA_FP8_E4M3
+    else:
+        raise TypeError(f"unsupported KV cache dtype {kv_cache.dtype} (bfloat16 or float8_e4m3fn)")
+    if (
+        kv_cache.dim() != 4
+        or kv_cache.shape[0] != 2
+        or kv_cache.shape[2] != plan.num_kv_heads
+        or kv_cache.shape[3] != BLOCK_SIZE * plan.head_dim
+        or kv_cache.stride(3) != 1
+    ):
+        raise ValueError("kv_cache must be [2, num_blocks, num_kv_heads, 16 * head_dim] (see kv_layout)")
+    if not (q.is_cuda and kv_cache.is_cuda):
+        raise RuntimeError("forest cascade attention runs on the GPU only; q and kv_cache must be device tensors")
+    for name, sc in (("k_scale", k_scale), ("v_scale", v_scale)):
+        if sc is not None and (sc.dtype != torch.float32 or sc.shape != (plan.num_kv_heads,) or not sc.is_contiguous()):
+            raise ValueError(f"{name} must be a contiguous fp32 tensor of shape [{plan.num_kv_heads}]")
+    esz = kv_cache.element_size()
+    return _lib.FcaTensors(
+        q.data_ptr(),
+        q.stride(0),
+        q.stride(1),
+        kv_cache.data_ptr(),
+        kv_cache.data_ptr() + kv_cache.stride(0) * esz,
+        kv_cache.stride(1),
+        kv_cache.stride(2),
+        kv_dtype,
+        0,
+        meta.block_table.data_ptr(),
+        meta.block_table.stride(0),
+        k_scale.data_ptr() if k_scale is not None else None,
+        v_scale.data_ptr() if v_scale is not None else None,
+        float(scale),
+    )
+
+
+def _out_args(q, meta, out, out_dtype):
+    plan = meta.plan
+    if out is None:
+        out = torch.empty(plan.num_seqs, plan.num_q_heads, plan.head_dim, dtype=out_dtype or torch.bfloat16, device=q.device)
+    if out.dtype == torch.bfloat16:
+        code = _lib.FCA_BF16
+    elif out.dtype == torch.float32:
+        code = _lib.FCA_F32
+    else:
+        raise TypeError("out must be bfloat16 or float32")
+    if out.shape != (plan.num_seqs, plan.num_q_heads, plan.head_dim) or out.stride(2) != 1:
+        raise ValueError("out must be [num_seqs, num_q_heads, head_dim] with contiguous head_dim")
+    return out, code
+
+
+def forest_cascade_decode(
+    q, kv_cache, meta: ForestMetadata, scale, k_scale=None, v_scale=None, out=None, return_lse=True, out_dtype=None
+):
+    """One layer's decode attention.  Returns ``out`` or ``(out, lse)``."""
+    lib = _lib.load_library()
+    t = _tensors(q, kv_cache, meta, scale, k_scale, v_scale)
+    out, code = _out_args(q, meta, out, out_dtype)
+    lse = torch.empty(meta.plan.num_seqs, meta.plan.num_q_heads, dtype=torch.float32, device=q.device) if return_lse else None
+    _lib.check(
+        lib.fca_decode_step(
+            ctypes.byref(meta.plan),
+            ctypes.byref(t),
+            meta.meta.data_ptr(),
+            meta.partial_out.data_ptr(),
+            meta.partial_lse.data_ptr(),
+            out.data_ptr(),
+            out.stride(0),
+            out.stride(1),
+            code,
+            lse.data_ptr() if lse is not None else None,
+            _stream_ptr(q.device),
+        )
+    )
+    return (out, lse) if return_lse else out
+
+
+def prefix_pass(q, kv_cache, meta: ForestMetadata, scale, k_scale=None, v_scale=None):
+    """Shared-node work items only; fills their slots of the partial buffers."""
+    lib = _lib.load_library()
+    t = _tensors(q, kv_cache, meta, scale, k_scale, v_scale)
+    _lib.check(
+        lib.fca_prefix_pass(
+            ctypes.byref(meta.plan), ctypes.byref(t), meta.meta.data_ptr(), meta.partial_out.data_ptr(),
+            meta.partial_lse.data_ptr(), _stream_ptr(q.device),
+        )
+    )
+
+
+def suffix_pass(q, kv_cache, meta: ForestMetadata, scale, k_scale=None, v_scale=None):
+    """Private-leaf work items only; fills their slots of the partial buffers."""
+    lib = _lib.load_library()
+    t = _tensors(q, kv_cache, meta, scale, k_scale, v_scale)
+    _lib.check(
+        lib.fca_suffix_pass(
+            ctypes.byref(meta.plan), ctypes.byref(t), meta.meta.data_ptr(), meta.partial_out.data_ptr(),
+            meta.partial_lse.data_ptr(), _stream_ptr(q.device),
+        )
+    )
+
+
+def merge_partials(meta: ForestMetadata, q_like, out=None, return_lse=True, out_dtype=None):
+    """Log-sum-exp merge of the partial buffers into ``out`` (and ``lse``)."""
+    lib = _lib.load_library()
+    out, code = _out_args(q_like, meta, out, out_dtype)
+    lse = torch.empty(meta.plan.num_seqs, meta.plan.num_q_heads, dtype=torch.float32, device=out.device) if return_lse else None
+    _lib.check(
+        lib.fca_merge(
+            ctypes.byref(meta.plan), meta.meta.data_ptr(), meta.partial_out.data_ptr(), meta.partial_lse.data_ptr(),
+            out.data_ptr(), out.stride(0), out.stride(1), code, lse.data_ptr() if lse is not None else None,
+            _stream_ptr(out.device),
+        )
+    )
+    return (out, lse) if return_lse else out

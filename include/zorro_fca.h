@@ -1,0 +1,142 @@
+/*
+ * zorro_fca.h - C ABI of libzorro_fca.so: forest cascade decode attention for gfx950.
+ *
+ * The platform switches this path on per sampling job with
+ * arctic_inference_config = {"zorro_inference": {"enable": true}}
+ * (arctic_platform/common/utils/server_models.py:123-140) and the engine it starts
+ * (arctic_platform/common/ray_server.py:395-404, :921-933) runs it once per attention
+ * layer per decode step.  The reference binds the path through an external Python
+ * package, not through an in-tree FFI, so the entry points below are what a ctypes /
+ * nanobind stub of that package's attention backend binds:
+ *
+ *   metadata build   <- the backend's per-scheduler-step metadata builder
+ *   prefix / suffix / merge / decode_step <- the backend's per-layer forward()
+ *
+ * Conventions
+ *   - every function returns 0 on success or a negative fca_status; fca_last_error()
+ *     returns a thread-local message for the last failure on the calling thread;
+ *   - all pointers named *_dev are device pointers; strides are in ELEMENTS;
+ *   - `stream` is a hipStream_t passed as void*; every call is asynchronous on it,
+ *     performs no host<->device synchronisation and allocates nothing;
+ *   - the caller owns every buffer, including the metadata and partial workspaces whose
+ *     sizes fca_workspace_bytes() reports;
+ *   - one metadata workspace must not be used by two streams at the same time (it holds
+ *     the work-queue ticket of the attention kernel).
+ */
+#ifndef ZORRO_FCA_H
+#define ZORRO_FCA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FCA_VERSION 100
+#define FCA_BLOCK_SIZE 16
+#define FCA_MAX_LEVELS 8
+
+typedef enum fca_status {
+  FCA_OK = 0,
+  FCA_ERR_INVALID_ARG = -1,
+  FCA_ERR_UNSUPPORTED = -2,
+  FCA_ERR_HIP = -3
+} fca_status;
+
+typedef enum fca_dtype {
+  FCA_BF16 = 0,     /* q, out, KV cache */
+  FCA_FP8_E4M3 = 1, /* KV cache only (OCP e4m3fn) */
+  FCA_F32 = 2       /* out only */
+} fca_dtype;
+
+/* Shape of one decode batch and the tiling the metadata is built for. */
+typedef struct fca_plan {
+  int32_t num_seqs;      /* S: rows of q and of the block table */
+  int32_t max_blocks;    /* columns of the block table */
+  int32_t num_q_heads;   /* Hq, multiple of num_kv_heads, Hq / Hkv <= 32 */
+  int32_t num_kv_heads;  /* Hkv */
+  int32_t head_dim;      /* 64 or 128 */
+  int32_t block_size;    /* must be FCA_BLOCK_SIZE */
+  int32_t chunk_tokens;  /* split-K chunk, multiple of 32 in [32, 1024] */
+  int32_t rows_per_item; /* query rows stacked per work item: 32 or 64 */
+  int32_t max_levels;    /* shared tree levels to discover, 0 = non-cascade, <= FCA_MAX_LEVELS */
+} fca_plan;
+
+/* Tensors of one attention layer. */
+typedef struct fca_tensors {
+  const void* q_dev;           /* bf16 [S, Hq, D], D contiguous */
+  int64_t q_seq_stride;
+  int64_t q_head_stride;
+  const void* k_cache_dev;     /* K plane: [num_blocks, Hkv, D/x, 16, x], x = 16 bytes / elem size */
+  const void* v_cache_dev;     /* V plane: [num_blocks, Hkv, D, 16] */
+  int64_t kv_block_stride;     /* elements between blocks of one plane */
+  int64_t kv_head_stride;      /* elements between KV heads of one block */
+  int32_t kv_dtype;            /* FCA_BF16 or FCA_FP8_E4M3 */
+  int32_t reserved;
+  const int32_t* block_table_dev; /* [S, max_blocks] physical block ids */
+  int64_t block_table_stride;
+  const float* k_scale_dev;    /* [Hkv] dequant scales for fp8 caches, or NULL (= 1) */
+  const float* v_scale_dev;
+  float softmax_scale;         /* usually head_dim ** -0.5 */
+} fca_tensors;
+
+/* Offsets (in int32 units) of the arrays inside a built metadata workspace, for
+ * inspection and tests.  Item records are 8 x int32:
+ * {rep_seq, blk_start, tok_len, member_off, member_cnt, ord, node, 0}. */
+typedef struct fca_meta_layout {
+  int64_t header;        /* [16]: 0 items, 1 shared items, 2 nodes (shared), 3 ticket, 4 done,
+                            5 error flag, 6/7 unique tokens lo/hi, 8 levels found */
+  int64_t seq_npart;     /* [S] partial slots used per sequence */
+  int64_t seq_leaf_blk;  /* [S] first block position of the private leaf */
+  int64_t node_rep;      /* [S] shared nodes: representative sequence */
+  int64_t node_blk;      /* [S] first block position */
+  int64_t node_nblk;     /* [S] number of blocks */
+  int64_t node_level;    /* [S] */
+  int64_t node_moff;     /* [S] offset into members */
+  int64_t node_mcnt;     /* [S] number of members */
+  int64_t node_ord;      /* [S] partial ordinal of the node's first chunk */
+  int64_t members;       /* [S * (FCA_MAX_LEVELS + 1)] sequence ids; leaves last */
+  int64_t items;         /* [max_items * 8] */
+  int64_t max_items;
+  int64_t max_partials;  /* partial slots reserved per sequence */
+  int64_t total_int32;
+} fca_meta_layout;
+
+int fca_version(void);
+const char* fca_last_error(void);
+
+/* Workspace sizes for a plan: metadata (int32 arrays) and the two partial buffers
+ * (fp32 [S * max_partials, Hq, D] and fp32 [S * max_partials, Hq]). */
+int fca_workspace_bytes(const fca_plan* plan, size_t* meta_bytes, size_t* partial_out_bytes, size_t* partial_lse_bytes);
+int fca_meta_describe(const fca_plan* plan, fca_meta_layout* layout);
+
+/* Forest metadata builder: block tables + lengths -> flat node / member / work-item arrays.
+ * Analog of the host-side prompt-group discovery of the trainer
+ * (arctic_platform/rl/zorro_train/zorro_train.py:242-285, seqlen_balancing.py:437-486). */
+int fca_build_metadata(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,
+                       const int32_t* seq_lens_dev, void* meta_dev, void* stream);
+
+/* Shared-prefix pass: work items of shared nodes only.  Writes normalised fp32 partial
+ * outputs and natural-log LSEs into the slots the metadata assigns. */
+int fca_prefix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev,
+                    float* partial_out_dev, float* partial_lse_dev, void* stream);
+/* Per-sequence suffix pass: work items of private leaves only (with max_levels = 0 this
+ * is the non-cascade paged decode kernel). */
+int fca_suffix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev,
+                    float* partial_out_dev, float* partial_lse_dev, void* stream);
+/* Log-sum-exp merge of each sequence's partials (online max / rescaled sum as in
+ * arctic_platform/model/implementations/qwen35/models/layers/lm_head.py:190-202).
+ * out: [S, Hq, D] bf16 or f32; lse: fp32 [S, Hq], natural log, may be NULL. */
+int fca_merge(const fca_plan* plan, const void* meta_dev, const float* partial_out_dev,
+              const float* partial_lse_dev, void* out_dev, int64_t out_seq_stride, int64_t out_head_stride,
+              int32_t out_dtype, float* lse_dev, void* stream);
+/* One layer's decode attention: prefix and suffix items in one launch, then the merge. */
+int fca_decode_step(const fca_plan* plan, const fca_tensors* t, void* meta_dev,
+                    float* partial_out_dev, float* partial_lse_dev, void* out_dev, int64_t out_seq_stride,
+                    int64_t out_head_stride, int32_t out_dtype, float* lse_dev, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ZORRO_FCA_H */

@@ -1,0 +1,89 @@
+"""Shared-prefix discovery over block tables, by brute force with Python containers.
+
+Grouping semantics follow the reference's prompt-group discovery: rows are compared with
+the first member of each existing group, groups appear in first-seen order and members in
+ascending row order (``ZoRRoTrain.find_prompt_groups``,
+arctic_platform/rl/zorro_train/zorro_train.py:242-285; the hash-map variant
+``create_prompt_groups``, arctic_platform/rl/zorro_train/seqlen_balancing.py:437-486).
+Here the compared rows are leading runs of physical block ids instead of prompt tokens,
+and the comparison is applied recursively, which turns the flat groups into a forest.
+
+A node is a maximal run of leading block-table positions whose physical ids are identical
+for a fixed set of two or more sequences.  Only full blocks can be shared.  What is left
+of a sequence below its deepest shared node is its private leaf.
+"""
+
+from __future__ import annotations
+
+from collections import OrderedDict
+
+BLOCK = 16
+
+
+def discover_forest(block_table, seq_lens, block_size=BLOCK, max_levels=8):
+    """Returns (nodes, leaves).
+
+    nodes: list of dict(members, blk_start, num_blocks, level, parent) for shared runs.
+    leaves: per sequence dict(blk_start, tokens, parent): the private remainder.
+    """
+    bt = [list(map(int, row)) for row in block_table]
+    lens = [int(n) for n in seq_lens]
+    nfull = [n // block_size for n in lens]
+    nodes = []
+    leaf_start = [0] * len(lens)
+    leaf_parent = [-1] * len(lens)
+
+    def descend(members, pos, level, parent):
+        if level >= max_levels:
+            return
+        groups = OrderedDict()
+        for s in members:
+            if pos < nfull[s]:
+                groups.setdefault(bt[s][pos], []).append(s)
+        for group in groups.values():
+            if len(group) < 2:
+                continue
+            limit = min(nfull[s] for s in group) - pos
+            first = group[0]
+            run = 0
+            while run < limit and all(bt[s][pos + run] == bt[first][pos + run] for s in group):
+                run += 1
+            node_id = len(nodes)
+            nodes.append(dict(members=list(group), blk_start=pos, num_blocks=run, level=level, parent=parent))
+            for s in group:
+                leaf_start[s] = pos + run
+                leaf_parent[s] = node_id
+            descend(group, pos + run, level + 1, node_id)
+
+    descend(list(range(len(lens))), 0, 0, -1)
+    leaves = [
+        dict(blk_start=leaf_start[s], tokens=lens[s] - leaf_start[s] * block_size, parent=leaf_parent[s])
+        for s in range(len(lens))
+    ]
+    return nodes, leaves
+
+
+def prompt_groups(block_table, seq_lens, block_size=BLOCK):
+    """Top-level groups only, in first-seen order with ascending members: the shape of
+    the reference's ``prompt_groups`` result (zorro_train.py:262-283)."""
+    nodes, _ = discover_forest(block_table, seq_lens, block_size, max_levels=1)
+    group_of = {}
+    for node in nodes:
+        for s in node["members"]:
+            group_of[s] = node["members"]
+    out, seen = [], set()
+    for s in range(len(seq_lens)):
+        g = group_of.get(s, [s])
+        if id(g) not in seen and g[0] == s:
+            out.append(list(g))
+            seen.add(id(g))
+    return out
+
+
+def canonical_nodes(nodes):
+    """Order-free form of a node list for comparisons."""
+    return sorted((tuple(sorted(n["members"])), n["blk_start"], n["num_blocks"]) for n in nodes)
+
+
+def unique_tokens(nodes, leaves, block_size=BLOCK):
+    return sum(n["num_blocks"] * block_size for n in nodes) + sum(l["tokens"] for l in leaves)
