@@ -25,7 +25,7 @@ def __getattr__(name):
         from . import forest
 
         return getattr(forest, name)
-    if name in ("forest_cascade_decode", "prefix_pass", "suffix_pass", "merge_partials"):
+    if name in ("forest_cascade_decode", "prefix_pass", "suffix_pass", "forest_pass", "merge_partials"):
         from . import ops
 
         return getattr(ops, name)

@@ -25,6 +25,7 @@ EXPORTS = (
     "fca_build_metadata",
     "fca_prefix_pass",
     "fca_suffix_pass",
+    "fca_forest_pass",
     "fca_merge",
     "fca_decode_step",
 )
@@ -128,6 +129,7 @@ def load_library() -> ctypes.CDLL:
     attend = [P(FcaPlan), P(FcaTensors), VP, VP, VP, VP]
     lib.fca_prefix_pass.argtypes = attend
     lib.fca_suffix_pass.argtypes = attend
+    lib.fca_forest_pass.argtypes = attend
     lib.fca_merge.argtypes = [P(FcaPlan), VP, VP, VP, VP, I64, I64, I32, VP, VP]
     lib.fca_decode_step.argtypes = [P(FcaPlan), P(FcaTensors), VP, VP, VP, VP, I64, I64, I32, VP, VP]
     for name in EXPORTS:

@@ -203,6 +203,11 @@ int fca_suffix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev, 
   return run_attend(plan, t, meta_dev, partial_out_dev, partial_lse_dev, 2, stream);
 }
 
+int fca_forest_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev, float* partial_out_dev,
+                    float* partial_lse_dev, void* stream) {
+  return run_attend(plan, t, meta_dev, partial_out_dev, partial_lse_dev, 0, stream);
+}
+
 int fca_merge(const fca_plan* plan, const void* meta_dev, const float* partial_out_dev, const float* partial_lse_dev,
               void* out_dev, int64_t out_seq_stride, int64_t out_head_stride, int32_t out_dtype, float* lse_dev,
               void* stream) {

@@ -132,6 +132,18 @@ def suffix_pass(q, kv_cache, meta: ForestMetadata, scale, k_scale=None, v_scale=
     )
 
 
+def forest_pass(q, kv_cache, meta: ForestMetadata, scale, k_scale=None, v_scale=None):
+    """Shared and private work items in one launch; fills every live partial slot."""
+    lib = _lib.load_library()
+    t = _tensors(q, kv_cache, meta, scale, k_scale, v_scale)
+    _lib.check(
+        lib.fca_forest_pass(
+            ctypes.byref(meta.plan), ctypes.byref(t), meta.meta.data_ptr(), meta.partial_out.data_ptr(),
+            meta.partial_lse.data_ptr(), _stream_ptr(q.device),
+        )
+    )
+
+
 def merge_partials(meta: ForestMetadata, q_like, out=None, return_lse=True, out_dtype=None):
     """Log-sum-exp merge of the partial buffers into ``out`` (and ``lse``)."""
     lib = _lib.load_library()

@@ -1,0 +1,256 @@
+"""Decode-attention benchmark of the forest cascade path on one MI355X.
+
+A step is one attention layer's decode call (shared-prefix items and per-sequence suffix
+items in one launch, then the log-sum-exp merge) over the whole batch.  The forest
+metadata is rebuilt once every ``--layers`` steps, the way a model forward shares one
+build across its attention layers (Qwen3-4B: 36), and each layer reads its own KV cache
+copy so no step finds its KV in a cache left by the previous one.
+
+Prints one JSON line: step latency in microseconds, the share of the 8 TB/s HBM peak that
+the unique KV bytes per step amount to, a roofline object for the attention kernel
+(timed with events on the launch stream inside the timed region), the same shape through
+the non-cascade kernel, and a CPU baseline (the oracle's flat attention on a sample).
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+METRIC = "cascade decode-attn µs/step & % of HBM peak, Qwen3-4B shape 512 seqs"
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=720)
+    ap.add_argument("--warmup", type=int, default=72)
+    ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1-5 (default: the Qwen3-4B decode step)")
+    ap.add_argument("--layers", type=int, default=36, help="attention layers sharing one metadata build")
+    ap.add_argument("--kv-copies", type=int, default=4, help="distinct KV caches cycled over the layers")
+    ap.add_argument("--chunk", type=int, default=0, help="split-K chunk in tokens (0 = default of the configuration)")
+    ap.add_argument("--rows", type=int, default=0, help="query rows per work item, 32 or 64 (0 = default)")
+    ap.add_argument("--cpu-seqs", type=int, default=512, help="sequences in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--skip-noncascade", action="store_true")
+    return ap.parse_args()
+
+
+def median(xs):
+    xs = sorted(xs)
+    return xs[len(xs) // 2]
+
+
+def run_steps(torch, ops, build, w, caches, md, out, lse, steps, layers, timed_events=None):
+    """``steps`` layer calls; metadata rebuilt at every ``layers``-th one.  When
+    ``timed_events`` is a list, the attention launch of each rebuilt step is bracketed by
+    events on the launch stream."""
+    for i in range(steps):
+        cache = caches[i % len(caches)]
+        if i % layers == 0:
+            build()
+            if timed_events is not None:
+                a = torch.cuda.Event(enable_timing=True)
+                b = torch.cuda.Event(enable_timing=True)
+                a.record()
+                ops.forest_pass(w.q, cache, md, w.scale, w.k_scale, w.v_scale)
+                b.record()
+                ops.merge_partials(md, w.q, out=out, return_lse=False)
+                timed_events.append((a, b))
+                continue
+        ops.forest_cascade_decode(w.q, cache, md, w.scale, w.k_scale, w.v_scale, out=out, return_lse=False)
+
+
+def time_steps(torch, ops, build, w, caches, md, out, lse, steps, warmup, layers):
+    run_steps(torch, ops, build, w, caches, md, out, lse, warmup, layers)
+    torch.cuda.synchronize()
+    events = []
+    t0 = time.perf_counter()
+    run_steps(torch, ops, build, w, caches, md, out, lse, steps, layers, events)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kernel_us = [a.elapsed_time(b) * 1e3 for a, b in events]
+    return wall, kernel_us
+
+
+def cpu_baseline(torch, w, nseq):
+    """The oracle's flat attention (fp32, every sequence gathers its own pages, no
+    sharing exploited) on the first ``nseq`` sequences, scaled to the whole batch."""
+    from oracle.attention import flat_decode_attention
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    nseq = min(nseq, w.num_seqs)
+    seqs = list(range(nseq))
+    need = sorted({int(b) for s in seqs for b in w.block_table[s, : (int(w.seq_lens[s]) + 15) // 16].tolist()})
+    remap = torch.zeros(w.kv_cache.shape[1], dtype=torch.long)
+    remap[need] = torch.arange(len(need))
+    cache = w.kv_cache[:, torch.as_tensor(need, device=w.kv_cache.device)].cpu()
+    table = remap[w.block_table[:nseq].cpu().long()].to(torch.int32)
+    q, lens = w.q[:nseq].cpu(), w.seq_lens[:nseq].cpu()
+    ks = None if w.k_scale is None else w.k_scale.cpu()
+    vs = None if w.v_scale is None else w.v_scale.cpu()
+    times = []
+    for it in range(3):
+        t0 = time.perf_counter()
+        flat_decode_attention(q, cache, table, lens, w.scale, ks, vs, dtype=torch.float32)
+        times.append(time.perf_counter() - t0)
+    sample_s = median(times[1:]) if len(times) > 1 else times[0]
+    scale_up = float(w.seq_lens.sum()) / float(lens.sum())
+    return {
+        "value": sample_s * scale_up * 1e6,
+        "unit": "us/step",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"first {nseq} of {w.num_seqs} sequences ({int(lens.sum())} of {int(w.seq_lens.sum())} gathered tokens), "
+        f"flat fp32 attention on torch-CPU, {sample_s:.2f} s measured, scaled by tokens x{scale_up:.2f}",
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path uses no collectives and the boxes have one GPU; run with --gpus 1")
+    import torch
+
+    from arctic_platform_amd import ops
+    from arctic_platform_amd.forest import build_forest_metadata
+    from arctic_platform_amd.workloads import make_config
+
+    dev = torch.device("cuda:0")
+    w = make_config(args.config, device=dev)
+    # distinct copies at distinct addresses: same values, so every copy gives the same result
+    caches = [w.kv_cache] + [w.kv_cache.clone() for _ in range(max(1, args.kv_copies) - 1)]
+    chunk = args.chunk or 1024
+    rows = args.rows or (64 if args.config == 3 else 32)
+    kw = dict(num_q_heads=w.num_q_heads, num_kv_heads=w.num_kv_heads, head_dim=w.head_dim, chunk_tokens=chunk, rows_per_item=rows)
+    out = torch.empty_like(w.q)
+
+    md = build_forest_metadata(w.block_table, w.seq_lens, **kw)
+    torch.cuda.synchronize()
+    md.check()
+    hdr = md.header()
+    unique_bytes = hdr["unique_tokens"] * w.kv_bytes_per_token
+    assert unique_bytes == w.unique_kv_bytes, "builder and generator disagree on unique KV tokens"
+
+    def build():
+        build_forest_metadata(w.block_table, w.seq_lens, out=md, **kw)
+
+    wall, kern_us = time_steps(torch, ops, build, w, caches, md, out, None, args.steps, args.warmup, args.layers)
+    step_us = wall / args.steps * 1e6
+    kern = sum(kern_us) / len(kern_us)
+
+    # builder and merge on their own, for the breakdown
+    def ev_time(fn, n=20):
+        fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(n):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            torch.cuda.synchronize()
+            ts.append(a.elapsed_time(b) * 1e3)
+        return median(ts)
+
+    build_us = ev_time(build)
+    merge_us = ev_time(lambda: ops.merge_partials(md, w.q, out=out, return_lse=False))
+
+    result = {
+        "metric": METRIC,
+        "value": round(step_us, 2),
+        "unit": "us/step",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_us / 1e3, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8 KV / bf16 MFMA / f32 accumulate" if args.config == 5 else "bf16 MFMA / f32 accumulate",
+        "data": "synthetic",
+        "config": {
+            "workload": w.name,
+            "seed": 1000 + args.config,
+            "num_seqs": w.num_seqs,
+            "unique_kv_bytes": unique_bytes,
+            "flat_kv_bytes": w.flat_kv_bytes,
+            "layers_per_metadata_build": args.layers,
+            "kv_cache_copies": len(caches),
+            "chunk_tokens": chunk,
+            "rows_per_item": rows,
+            "work_items": hdr["items"],
+            "shared_nodes": hdr["shared_nodes"],
+        },
+        "pct_hbm_peak_unique_bytes": round(unique_bytes / (step_us * 1e-6) / 1e9 / HBM_PEAK_GBS * 100, 2),
+        "breakdown_us": {
+            "attention_kernel": round(kern, 2),
+            "merge_kernel": round(merge_us, 2),
+            "metadata_builder": round(build_us, 2),
+            "builder_per_step": round(build_us / args.layers, 2),
+        },
+        "roofline": {
+            "kernel": "fca_attend_kernel",
+            "bound": "hbm",
+            "achieved": round(unique_bytes / (kern * 1e-6) / 1e9, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(unique_bytes / (kern * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "launches_timed": len(kern_us),
+        },
+    }
+
+    if not args.skip_noncascade:
+        nc = build_forest_metadata(w.block_table, w.seq_lens, cascade=False, **kw)
+        torch.cuda.synchronize()
+
+        def nc_build():
+            build_forest_metadata(w.block_table, w.seq_lens, cascade=False, out=nc, **kw)
+
+        nsteps = max(args.layers, args.steps // 4)
+        nwall, _ = time_steps(torch, ops, nc_build, w, caches, nc, out, None, nsteps, args.layers, args.layers)
+        nc_us = nwall / nsteps * 1e6
+        result["noncascade"] = {
+            "us_per_step": round(nc_us, 2),
+            "speedup_of_cascade": round(nc_us / step_us, 3),
+            "order": "natural (the samples of a group are adjacent rows)",
+            "gbs_on_flat_bytes": round(w.flat_kv_bytes / (nc_us * 1e-6) / 1e9, 1),
+        }
+        # same batch with the rows of each group spread across the batch
+        perm = torch.arange(w.num_seqs, device=dev).view(-1, 8).t().reshape(-1) if w.num_seqs % 8 == 0 else None
+        if perm is not None:
+            bt2, sl2 = w.block_table[perm].contiguous(), w.seq_lens[perm].contiguous()
+            nc2 = build_forest_metadata(bt2, sl2, cascade=False, **kw)
+
+            def nc2_build():
+                build_forest_metadata(bt2, sl2, cascade=False, out=nc2, **kw)
+
+            import dataclasses
+
+            w2 = dataclasses.replace(w, q=w.q[perm].contiguous(), block_table=bt2, seq_lens=sl2)
+            nwall2, _ = time_steps(torch, ops, nc2_build, w2, caches, nc2, out, None, nsteps, args.layers, args.layers)
+            nc2_us = nwall2 / nsteps * 1e6
+            result["noncascade_interleaved"] = {
+                "us_per_step": round(nc2_us, 2),
+                "speedup_of_cascade": round(nc2_us / step_us, 3),
+                "order": "group-interleaved (row i of every group, then row i+1, ...)",
+            }
+        del nc
+
+    if args.cpu_seqs > 0:
+        result["cpu_baseline"] = cpu_baseline(torch, w, args.cpu_seqs)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -125,6 +125,9 @@ int fca_prefix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev,
  * is the non-cascade paged decode kernel). */
 int fca_suffix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev,
                     float* partial_out_dev, float* partial_lse_dev, void* stream);
+/* Both classes of work items in one launch (what fca_decode_step runs before its merge). */
+int fca_forest_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev,
+                    float* partial_out_dev, float* partial_lse_dev, void* stream);
 /* Log-sum-exp merge of each sequence's partials (online max / rescaled sum as in
  * arctic_platform/model/implementations/qwen35/models/layers/lm_head.py:190-202).
  * out: [S, Hq, D] bf16 or f32; lse: fp32 [S, Hq], natural log, may be NULL. */
