@@ -71,12 +71,11 @@ def prompt_groups(block_table, seq_lens, block_size=BLOCK):
     for node in nodes:
         for s in node["members"]:
             group_of[s] = node["members"]
-    out, seen = [], set()
+    out = []
     for s in range(len(seq_lens)):
         g = group_of.get(s, [s])
-        if id(g) not in seen and g[0] == s:
+        if g[0] == s:  # a group is emitted when its first member comes up
             out.append(list(g))
-            seen.add(id(g))
     return out
 
 

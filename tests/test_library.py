@@ -1,0 +1,91 @@
+"""The C-ABI library without a GPU: it loads, exports what include/zorro_fca.h declares,
+sizes workspaces and rejects bad arguments before any launch."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from arctic_platform_amd import _lib
+from arctic_platform_amd.forest import make_plan
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(_lib.LIB_PATH):
+        _lib.build_library()
+    return _lib.load_library()
+
+
+def test_exports_every_declared_symbol(lib):
+    header = open(os.path.join(ROOT, "include", "zorro_fca.h")).read()
+    declared = set(re.findall(r"^(?:int|const char\*)\s+(fca_\w+)\s*\(", header, flags=re.M))
+    assert declared == set(_lib.EXPORTS)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.fca_version() == 100
+
+
+def test_struct_sizes_match_header():
+    assert ctypes.sizeof(_lib.FcaPlan) == 9 * 4
+    assert ctypes.sizeof(_lib.FcaMetaLayout) == 15 * 8
+    assert ctypes.sizeof(_lib.FcaTensors) == 104
+
+
+def test_workspace_sizes(lib):
+    plan = make_plan(512, 320, 32, 8, 128, chunk_tokens=512, max_levels=4)
+    layout = _lib.FcaMetaLayout()
+    assert lib.fca_meta_describe(ctypes.byref(plan), ctypes.byref(layout)) == 0
+    assert layout.max_partials == 320 * 16 // 512 + 4 + 1
+    assert layout.max_items == 512 * layout.max_partials
+    nm, no, nl = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    assert lib.fca_workspace_bytes(ctypes.byref(plan), ctypes.byref(nm), ctypes.byref(no), ctypes.byref(nl)) == 0
+    assert nm.value == layout.total_int32 * 4
+    assert no.value == 512 * layout.max_partials * 32 * 128 * 4
+    assert nl.value == 512 * layout.max_partials * 32 * 4
+
+
+@pytest.mark.parametrize(
+    "kw,fragment",
+    [
+        (dict(chunk_tokens=100), "chunk_tokens"),
+        (dict(chunk_tokens=2048), "chunk_tokens"),
+        (dict(rows_per_item=48), "rows_per_item"),
+        (dict(max_levels=9), "max_levels"),
+        (dict(head_dim=96), "head_dim"),
+        (dict(num_q_heads=30), "num_q_heads"),
+    ],
+)
+def test_bad_plans_are_rejected(lib, kw, fragment):
+    base = dict(num_seqs=4, max_blocks=8, num_q_heads=32, num_kv_heads=8, head_dim=128)
+    tiling = dict(chunk_tokens=512, rows_per_item=32, max_levels=4)
+    for k, v in kw.items():
+        (base if k in base else tiling)[k] = v
+    plan = make_plan(**base, **tiling)
+    rc = lib.fca_meta_describe(ctypes.byref(plan), ctypes.byref(_lib.FcaMetaLayout()))
+    assert rc < 0 and fragment in lib.fca_last_error().decode()
+
+
+def test_block_size_and_null_pointers(lib):
+    plan = make_plan(4, 8, 32, 8, 128)
+    plan.block_size = 32
+    assert lib.fca_meta_describe(ctypes.byref(plan), ctypes.byref(_lib.FcaMetaLayout())) == -2
+    plan.block_size = 16
+    assert lib.fca_build_metadata(ctypes.byref(plan), None, 8, None, None, None) == -1
+    assert "non-NULL" in lib.fca_last_error().decode()
+    t = _lib.FcaTensors()
+    assert lib.fca_decode_step(ctypes.byref(plan), ctypes.byref(t), None, None, None, None, 0, 0, 0, None, None) == -1
+
+
+def test_operators_refuse_cpu_tensors():
+    import torch
+
+    from arctic_platform_amd.forest import build_forest_metadata
+
+    with pytest.raises(RuntimeError, match="GPU"):
+        build_forest_metadata(
+            torch.zeros(2, 4, dtype=torch.int32), torch.ones(2, dtype=torch.int32), num_q_heads=8, num_kv_heads=2, head_dim=64
+        )
