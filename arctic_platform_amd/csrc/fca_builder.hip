@@ -236,7 +236,8 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   __syncthreads();
 
   // Work list: one item per (node chunk, tile of members), shared items first, each
-  // class in descending size order so the dynamic queue ends on the small ones.
+  // class in descending size order: the attention kernel deals the list to its waves in
+  // alternating directions, which balances a descending list well.
   const int total_nodes = node_base + S;
   auto node_fields = [&](int n, int& rep, int& blk, int& tokens, int& moff, int& mcnt, int& o) {
     if (n < node_base) {

@@ -44,8 +44,6 @@ class ForestMetadata:
             items=h[0],
             shared_items=h[1],
             shared_nodes=h[2],
-            ticket=h[3],
-            done=h[4],
             error=h[5],
             unique_tokens=(h[6] & 0xFFFFFFFF) | (h[7] << 32),
             levels=h[8],

@@ -89,7 +89,7 @@ def three_level_forest(gen, system_len, segments, samples, segment_range, suffix
     return seg_len, paths
 
 
-def page_forest(seg_len, paths, gen, spare_blocks=0.125):
+def page_forest(seg_len, paths, gen, spare_blocks=0.125, shuffle_blocks=True):
     """Assign physical blocks.  Returns (block_table, seq_lens, slot_src, num_blocks).
 
     ``slot_src[b * 16 + t]`` is the index of the logical token (position in the
@@ -121,7 +121,9 @@ def page_forest(seg_len, paths, gen, spare_blocks=0.125):
         lens.append(n)
     used = len(key_to_block)
     num_blocks = used + max(1, int(used * spare_blocks))
-    perm = torch.randperm(num_blocks, generator=gen).numpy()
+    perm = torch.randperm(num_blocks, generator=gen).numpy()  # drawn even if unused: keeps later draws in place
+    if not shuffle_blocks:
+        perm = np.arange(num_blocks)
     slot_src = np.full(num_blocks * BLOCK_SIZE, -1, dtype=np.int64)
     for blk, src in fills:
         base = int(perm[blk]) * BLOCK_SIZE
@@ -146,10 +148,11 @@ def make_forest_workload(
     kv_dtype=None,
     device="cpu",
     poison_unused=False,
+    shuffle_blocks=True,
 ):
     """Build q, the paged cache and the block table for a forest of segments."""
     kv_dtype = kv_dtype or dtype
-    table, lens, slot_src, num_blocks = page_forest(seg_len, paths, gen)
+    table, lens, slot_src, num_blocks = page_forest(seg_len, paths, gen, shuffle_blocks=shuffle_blocks)
     total = int(sum(seg_len))
     dev_gen = gen
     if torch.device(device).type != "cpu":
@@ -216,7 +219,7 @@ CONFIG_NAMES = {
 }
 
 
-def make_config(index: int, device="cpu", *, shrink: int = 1, dtype=None, poison_unused=False, seed=None):
+def make_config(index: int, device="cpu", *, shrink: int = 1, dtype=None, poison_unused=False, seed=None, shuffle_blocks=True):
     """The five benchmark configurations.  ``shrink`` divides group counts and lengths
     (for CPU-sized variants of the same shape); ``dtype`` overrides the q/KV element type
     of configuration 1 (fp32 by definition) so the bf16 kernels can run it.
@@ -241,4 +244,6 @@ def make_config(index: int, device="cpu", *, shrink: int = 1, dtype=None, poison
     else:
         raise ValueError(f"unknown configuration {index}")
     name = CONFIG_NAMES[index] + (f" (lengths and groups / {shrink})" if shrink > 1 else "")
-    return make_forest_workload(name, seg_len, paths, gen, device=device, poison_unused=poison_unused, **kw)
+    return make_forest_workload(
+        name, seg_len, paths, gen, device=device, poison_unused=poison_unused, shuffle_blocks=shuffle_blocks, **kw
+    )

@@ -20,8 +20,9 @@
  *     performs no host<->device synchronisation and allocates nothing;
  *   - the caller owns every buffer, including the metadata and partial workspaces whose
  *     sizes fca_workspace_bytes() reports;
- *   - one metadata workspace must not be used by two streams at the same time (it holds
- *     the work-queue ticket of the attention kernel).
+ *   - the attention and merge calls only read the metadata workspace; the partial
+ *     workspaces are written by the attention call and read by the merge, so two layers
+ *     running concurrently on different streams need separate partial workspaces.
  */
 #ifndef ZORRO_FCA_H
 #define ZORRO_FCA_H
@@ -85,7 +86,7 @@ typedef struct fca_tensors {
  * inspection and tests.  Item records are 8 x int32:
  * {rep_seq, blk_start, tok_len, member_off, member_cnt, ord, node, 0}. */
 typedef struct fca_meta_layout {
-  int64_t header;        /* [16]: 0 items, 1 shared items, 2 nodes (shared), 3 ticket, 4 done,
+  int64_t header;        /* [16]: 0 items, 1 shared items, 2 nodes (shared), 3-4 reserved,
                             5 error flag, 6/7 unique tokens lo/hi, 8 levels found */
   int64_t seq_npart;     /* [S] partial slots used per sequence */
   int64_t seq_leaf_blk;  /* [S] first block position of the private leaf */

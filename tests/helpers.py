@@ -38,3 +38,25 @@ def assert_matches_oracle(out, lse, ref_out, ref_lse, seqs=None, what=""):
     lerr = (lse - ref_lse).abs().max()
     assert lerr <= LSE_ATOL, f"{what}: lse max abs err {lerr:.4g}"
     return float(err.max()), float(lerr)
+
+
+def oracle_for_sample(w, seqs):
+    """Oracle on a few rows of a large workload: only the blocks those rows use are
+    brought to the CPU (block ids are renumbered; values are untouched)."""
+    seqs = list(seqs)
+    lens = w.seq_lens.cpu()
+    table = w.block_table.cpu()
+    need = sorted({int(b) for s in seqs for b in table[s, : (int(lens[s]) + 15) // 16].tolist()})
+    remap = torch.zeros(w.kv_cache.shape[1], dtype=torch.long)
+    remap[need] = torch.arange(len(need))
+    cache = w.kv_cache[:, torch.as_tensor(need, device=w.kv_cache.device)].cpu()
+    sub_table = remap[table[seqs].long()].to(torch.int32)
+    return flat_decode_attention(
+        w.q[seqs].cpu(),
+        cache,
+        sub_table,
+        lens[seqs],
+        w.scale,
+        None if w.k_scale is None else w.k_scale.cpu(),
+        None if w.v_scale is None else w.v_scale.cpu(),
+    )
