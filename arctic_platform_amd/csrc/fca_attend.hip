@@ -180,7 +180,7 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
       }
     }
   };
-  auto load_tile = [&](KT& kt, VT& vt, int my_blk, int nblk, int kvh, int ti) {
+  auto load_k = [&](KT& kt, int my_blk, int nblk, int kvh, int ti) {
     const int p0 = 2 * ti, p1 = min(2 * ti + 1, nblk - 1);
     const int b0 = __builtin_amdgcn_readlane(my_blk, p0);
     const int b1 = __builtin_amdgcn_readlane(my_blk, p1);
@@ -188,6 +188,11 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
     const char* kp = p.k_cache + (int64_t)kvh * p.kv_head_bytes + (int64_t)kb * p.kv_block_bytes + k_lane_off;
 #pragma unroll
     for (int i = 0; i < KT::NK; ++i) kt.k[i] = *reinterpret_cast<const i32x4*>(kp + i * 512);
+  };
+  auto load_v = [&](VT& vt, int my_blk, int nblk, int kvh, int ti) {
+    const int p0 = 2 * ti, p1 = min(2 * ti + 1, nblk - 1);
+    const int b0 = __builtin_amdgcn_readlane(my_blk, p0);
+    const int b1 = __builtin_amdgcn_readlane(my_blk, p1);
     const char* vbase = p.v_cache + (int64_t)kvh * p.kv_head_bytes + v_lane_off;
     const char* vp0 = vbase + (int64_t)b0 * p.kv_block_bytes;
     const char* vp1 = vbase + (int64_t)b1 * p.kv_block_bytes;
@@ -196,6 +201,10 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
       vt.v[0][db] = *reinterpret_cast<const typename RawV<FP8>::type*>(vp0 + db * V_DB_STEP);
       vt.v[1][db] = *reinterpret_cast<const typename RawV<FP8>::type*>(vp1 + db * V_DB_STEP);
     }
+  };
+  auto load_tile = [&](KT& kt, VT& vt, int my_blk, int nblk, int kvh, int ti) {
+    load_k(kt, my_blk, nblk, kvh, ti);
+    load_v(vt, my_blk, nblk, kvh, ti);
   };
 
   // ---- first item of this wave: fetched with the waits exposed
@@ -255,41 +264,37 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
 
       // One 32-token tile.  RAGGED is the variant for the single tile that may run past the
       // end of the chunk: it masks scores and zeroes V there; full tiles carry no mask code.
-      auto compute_tile = [&](const KT& kt, const VT& vt, int ti, auto ragged) {
+      bf16x8 pb[NRT][2];  // probabilities of the current tile as B operands
+      auto scores_softmax = [&](const KT& kt, int ti, auto ragged) {
         constexpr bool RAGGED = decltype(ragged)::value;
         const int tok0 = ti * kTile;
-        f32x16 s[NRT];
-#pragma unroll
-        for (int rt = 0; rt < NRT; ++rt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) s[rt][r] = 0.f;
-#pragma unroll
-        for (int i = 0; i < KS; ++i) {
-          bf16x8 a;
-          if constexpr (FP8) {
-            const i32x4 w = kt.k[i >> 1];
-            a = (i & 1) ? fp8x8_to_bf16(w[2], w[3]) : fp8x8_to_bf16(w[0], w[1]);
-          } else {
-            a = __builtin_bit_cast(bf16x8, kt.k[i]);
-          }
-          s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[0][i], s[0], 0, 0, 0);
-          if constexpr (NRT > 1) {
-            if (two_tiles) s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[1][i], s[1], 0, 0, 0);
-          }
-        }
-        bf16x8 pb[NRT][2];
 #pragma unroll
         for (int rt = 0; rt < NRT; ++rt) {
           if (rt > 0 && !two_tiles) continue;
+          // scores of one row tile at a time: the second tile reuses the score registers
+          f32x16 sr;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sr[r] = 0.f;
+#pragma unroll
+          for (int i = 0; i < KS; ++i) {
+            bf16x8 a;
+            if constexpr (FP8) {
+              const i32x4 w = kt.k[i >> 1];
+              a = (i & 1) ? fp8x8_to_bf16(w[2], w[3]) : fp8x8_to_bf16(w[0], w[1]);
+            } else {
+              a = __builtin_bit_cast(bf16x8, kt.k[i]);
+            }
+            sr = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[rt][i], sr, 0, 0, 0);
+          }
           // register r holds token 16 * (r / 8) + 8 * h + r % 8 of the tile
           if constexpr (RAGGED) {
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-              if (tok0 + 16 * (r >> 3) + 8 * h + (r & 7) >= tok_len) s[rt][r] = -INFINITY;
+              if (tok0 + 16 * (r >> 3) + 8 * h + (r & 7) >= tok_len) sr[r] = -INFINITY;
           }
-          float mx = s[rt][0];
+          float mx = sr[0];
 #pragma unroll
-          for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[rt][r]);
+          for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sr[r]);
           mx = fmaxf(mx, __shfl_xor(mx, 32));
           // sc > 0, so the maximum of the scaled scores is the scaled maximum.  mrow is the
           // reference the exponentials are taken against, not the exact running maximum: it
@@ -312,12 +317,16 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
           float sum = 0.f;
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const float e = fast_exp2(__builtin_fmaf(s[rt][r], sc, -mref));
+            const float e = fast_exp2(__builtin_fmaf(sr[r], sc, -mref));
             sum += e;
             pb[rt][r >> 3][r & 7] = (__bf16)e;
           }
           lrow[rt] += sum;
         }
+      };
+      auto weighted_values = [&](const VT& vt, int ti, auto ragged) {
+        constexpr bool RAGGED = decltype(ragged)::value;
+        const int tok0 = ti * kTile;
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
           // tokens this lane feeds for this block: 8h .. 8h+7; on the ragged tile zero the
@@ -359,28 +368,49 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
         }
       };
 
-      // Tile pipeline with two register buffers; k0/v0 already hold (or await) tile 0.  The
-      // prefetch past the end is clamped to the last tile instead of skipped, so the
-      // outstanding-load count is the same on every path and every wait covers exactly the
-      // tile about to be used.  Each trip also advances the next item's chain by one hop:
-      // the per-lane data is (re)read from the record fetched one trip earlier, then the
-      // record is (re)read from the ticket; both are idempotent, so no branch is needed.
+      auto compute_tile = [&](const KT& kt, const VT& vt, int ti, auto ragged) {
+        scores_softmax(kt, ti, ragged);
+        weighted_values(vt, ti, ragged);
+      };
+
+      // Tile pipeline; k0/v0 already hold (or await) tile 0.  Prefetches past the end are
+      // clamped to the last tile instead of skipped, so the outstanding-load count is the
+      // same on every path and every wait covers exactly the tile about to be used.  Each
+      // trip also advances the next item's chain by one hop: the per-lane data is (re)read
+      // from the record fetched one trip earlier, then the record is (re)read from the
+      // ticket; both are idempotent, so no branch is needed.
       int ti = 0, trips = 0;
-      for (; ti + 1 < nfull; ti += 2, ++trips) {
-        load_tile(k1, v1, my_blk, nblk, kvh, ti + 1);
-        compute_tile(k0, v0, ti, std::false_type{});
-        load_tile(k0, v0, my_blk, nblk, kvh, min(ti + 2, last));
-        compute_tile(k1, v1, ti + 1, std::false_type{});
-        load_lane_meta(n0, n1, nmy_blk, nseq);
-        load_record(t_next, n0, n1, nkvh);
-      }
-      // k0/v0 hold tile ti if ti < ntiles; zero, one or two tiles remain
-      if (ti < nfull) {
-        load_tile(k1, v1, my_blk, nblk, kvh, min(ti + 1, last));
-        compute_tile(k0, v0, ti, std::false_type{});
-        if (ti + 1 < ntiles) compute_tile(k1, v1, ti + 1, std::true_type{});
-      } else if (ti < ntiles) {
-        compute_tile(k0, v0, ti, std::true_type{});
+      if constexpr (NRT == 1) {
+        // two register buffers: the whole next tile is in flight while this one is consumed
+        for (; ti + 1 < nfull; ti += 2, ++trips) {
+          load_tile(k1, v1, my_blk, nblk, kvh, ti + 1);
+          compute_tile(k0, v0, ti, std::false_type{});
+          load_tile(k0, v0, my_blk, nblk, kvh, min(ti + 2, last));
+          compute_tile(k1, v1, ti + 1, std::false_type{});
+          load_lane_meta(n0, n1, nmy_blk, nseq);
+          load_record(t_next, n0, n1, nkvh);
+        }
+        // k0/v0 hold tile ti if ti < ntiles; zero, one or two tiles remain
+        if (ti < nfull) {
+          load_tile(k1, v1, my_blk, nblk, kvh, min(ti + 1, last));
+          compute_tile(k0, v0, ti, std::false_type{});
+          if (ti + 1 < ntiles) compute_tile(k1, v1, ti + 1, std::true_type{});
+        } else if (ti < ntiles) {
+          compute_tile(k0, v0, ti, std::true_type{});
+        }
+      } else {
+        // 64 query rows leave no room for a second tile buffer: one buffer, refilled in
+        // halves -- the next K as soon as the scores have issued, the next V as soon as the
+        // value product has
+        for (; ti < nfull; ++ti, ++trips) {
+          scores_softmax(k0, ti, std::false_type{});
+          load_k(k0, my_blk, nblk, kvh, min(ti + 1, last));
+          weighted_values(v0, ti, std::false_type{});
+          load_v(v0, my_blk, nblk, kvh, min(ti + 1, last));
+          load_lane_meta(n0, n1, nmy_blk, nseq);
+          load_record(t_next, n0, n1, nkvh);
+        }
+        if (ti < ntiles) compute_tile(k0, v0, ti, std::true_type{});
       }
 
       // finish the chain for items too short to have done it on the way
