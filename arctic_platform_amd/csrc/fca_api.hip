@@ -223,4 +223,12 @@ int fca_decode_step(const fca_plan* plan, const fca_tensors* t, void* meta_dev, 
                    lse_dev, stream);
 }
 
+int fca_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void* stream) {
+  if (!src_dev || !dst_dev || (bytes & 15) || (reinterpret_cast<uintptr_t>(src_dev) & 15) ||
+      (reinterpret_cast<uintptr_t>(dst_dev) & 15))
+    return fail(FCA_ERR_INVALID_ARG, "calibration copy needs 16-byte aligned pointers and a multiple of 16 bytes");
+  hipError_t e = fca::launch_copy(src_dev, dst_dev, bytes, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? FCA_OK : hip_fail(e, "calibration copy launch");
+}
+
 }  // extern "C"

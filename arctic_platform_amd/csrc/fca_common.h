@@ -148,5 +148,6 @@ struct MergeParams {
 hipError_t launch_build(const BuildParams& p, hipStream_t stream);
 hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, hipStream_t stream);
 hipError_t launch_merge(const MergeParams& p, hipStream_t stream);
+hipError_t launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
 
 }  // namespace fca

@@ -53,6 +53,18 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
   if (p.lse && sub == 0) p.lse[row] = wsum > 0.f ? m + __logf(wsum) : -INFINITY;
 }
 
+// Plain 16-bytes-per-lane copy, the yardstick the hardware traffic counters are scaled by.
+__global__ __launch_bounds__(256) void fca_copy_kernel(const int4* __restrict__ src, int4* __restrict__ dst, size_t n) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+}
+
+hipError_t launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream) {
+  hipLaunchKernelGGL(fca_copy_kernel, dim3(2048), dim3(256), 0, stream, static_cast<const int4*>(src),
+                     static_cast<int4*>(dst), bytes / 16);
+  return hipGetLastError();
+}
+
 hipError_t launch_merge(const MergeParams& p, hipStream_t stream) {
   const int rows = p.num_seqs * p.num_q_heads;
   const int per_block = kMergeThreads / kLanesPerRow;

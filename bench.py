@@ -23,6 +23,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the attention kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE
+# passes summarised in profiles/, keyed by (configuration, chunk_tokens, rows_per_item).
+# Counters cannot be read from inside this process; other shapes report null.
+MEASURED_TRAFFIC_BYTES = {(2, 1024, 32): 1_857_900_000}
 METRIC = "cascade decode-attn µs/step & % of HBM peak, Qwen3-4B shape 512 seqs"
 
 
@@ -38,6 +42,7 @@ def parse_args():
     ap.add_argument("--rows", type=int, default=0, help="query rows per work item, 32 or 64 (0 = default)")
     ap.add_argument("--cpu-seqs", type=int, default=512, help="sequences in the CPU baseline sample (0 = skip)")
     ap.add_argument("--skip-noncascade", action="store_true")
+    ap.add_argument("--calibrate", action="store_true", help="also run the library's plain copy kernel over 1 GiB (counter yardstick)")
     return ap.parse_args()
 
 
@@ -203,10 +208,22 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(unique_bytes / (kern * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, chunk, rows)),
             "launches_timed": len(kern_us),
         },
     }
+
+    if args.calibrate:
+        from arctic_platform_amd import _lib
+        from arctic_platform_amd.forest import _stream_ptr
+
+        src = torch.ones(1 << 28, dtype=torch.int32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            _lib.check(_lib.load_library().fca_calibration_copy(src.data_ptr(), dst.data_ptr(), src.numel() * 4, _stream_ptr(dev)))
+        torch.cuda.synchronize()
+        result["calibration_copy_bytes"] = src.numel() * 4
+        del src, dst
 
     if not args.skip_noncascade:
         nc = build_forest_metadata(w.block_table, w.seq_lens, cascade=False, **kw)

@@ -140,6 +140,11 @@ int fca_decode_step(const fca_plan* plan, const fca_tensors* t, void* meta_dev,
                     float* partial_out_dev, float* partial_lse_dev, void* out_dev, int64_t out_seq_stride,
                     int64_t out_head_stride, int32_t out_dtype, float* lse_dev, void* stream);
 
+/* Plain device-to-device copy with 16-byte loads and stores.  No counterpart in the
+ * reference: it is the known-size yardstick for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE
+ * readings of the kernels above. */
+int fca_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
