@@ -45,7 +45,6 @@ constexpr int kWaves = 4;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 constexpr float kRescaleSlack = 8.f;  // log2 units: rescale when a row maximum rises by more than 2^8
-constexpr int kOutStride = 32 + 4;   // floats per row of the per-wave LDS transpose buffer (padded)
 
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ inline float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
@@ -93,18 +92,25 @@ __device__ inline bf16x8 fp8x8_to_bf16(int lo, int hi) {
 __device__ long long* g_prof = nullptr;  // [waves][8] wall-clock ticks (100 MHz), debug builds only
 #endif
 
-// One persistent loop per wave that keeps loads in flight across work items.  Tickets are dealt statically, back and forth over
-// the size-ordered list: in round r wave w of W takes ticket r * W + w (r even) or
-// r * W + W - 1 - w (r odd), which evens out the descending sizes between waves.  The
-// kernel touches no shared counter and leaves the metadata read-only: device-wide atomics
-// on one address serialise at roughly 20 ns each across the eight L2s, so a ticket
-// counter costs tens of microseconds whenever the waves ask at about the same time.  While the tiles of the current item stream, the wave fetches
+// One persistent loop per wave that keeps loads in flight across work items.
+//
+// Dealing the work.  Most tickets are dealt statically, back and forth over the
+// size-ordered list: in round r wave w of W takes ticket r * W + w (r even) or
+// r * W + W - 1 - w (r odd), which evens out the descending sizes between waves at no
+// cost.  A shared counter for everything would be expensive: device-wide atomics on one
+// address serialise at roughly 20 ns each across the eight L2s, so 1024 waves asking at
+// once wait tens of microseconds.  But waves do not run at the same speed (odd XCDs
+// stream several percent slower than even ones on identical work), so the last full
+// round and the remainder, the smallest items, come from a counter: each wave draws one
+// item ahead, which hides the atomic's latency, and draws until the list is empty.  The
+// draw that returns the last possible value re-arms the counter for the next launch.
+//
+// Hiding item boundaries.  While the tiles of the current item stream, the wave fetches
 // the next item's record, block ids and member sequences; the next item's query rows and
 // first tile are requested before the current item's partial is written out, so the
 // memory pipe does not drain at item boundaries.
 template <int D, int NRT, bool FP8>
 __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendParams p) {
-  __shared__ __attribute__((aligned(16))) float lds_all[kWaves][32 * kOutStride];
   constexpr int KS = D / 16;   // MFMA steps of the score product
   constexpr int NDB = D / 32;  // 32-channel blocks of the output
   using KT = KTile<D, FP8>;
@@ -119,7 +125,6 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
   const int lane = threadIdx.x & 63;
   const int m = lane & 31, h = lane >> 5;
   const int G = p.group, Hkv = p.num_kv_heads;
-  float* lds_out = lds_all[wave];
   const int32_t* meta = p.meta;
 
   // row n = rt * 32 + m of the stacked query tile is (member n / G, head n % G)
@@ -137,6 +142,9 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
   constexpr int V_DB_STEP = FP8 ? 512 : 1024;
 
   const int nwaves = (int)gridDim.x * kWaves;
+  const int static_tickets = min(ntickets, max(1, ntickets / nwaves - 1) * nwaves);
+  // every wave that has work draws until it fails once
+  const int dynamic_draws = ntickets - static_tickets + min(nwaves, ntickets);
   const int my_wave = (int)blockIdx.x * kWaves + wave;
   // A zero the compiler cannot see through.  Added to the record address it makes the
   // record look lane-dependent, which keeps the compiler from moving its fields into
@@ -221,7 +229,12 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
     load_q(seq, r1.x, kvh);
     KT k0, k1;
     VT v0, v1;
-    load_tile(k0, v0, my_blk, (__builtin_amdgcn_readfirstlane(r0.z) + kBlock - 1) / kBlock, kvh, 0);
+    {
+      const int first_len = __builtin_amdgcn_readfirstlane(r0.z);
+      const int first_nblk = (first_len + kBlock - 1) / kBlock;
+      load_tile(k0, v0, my_blk, first_nblk, kvh, 0);
+      if constexpr (NRT == 1) load_tile(k1, v1, my_blk, first_nblk, kvh, first_len > kTile ? 1 : 0);
+    }
 
     for (;;) {
       const int tok_len = __builtin_amdgcn_readfirstlane(r0.z);
@@ -242,7 +255,17 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
 
       // next item: chase its record and per-lane data during the tile loop
       ++round;
-      const int t_next = round * nwaves + ((round & 1) ? nwaves - 1 - my_wave : my_wave);
+      int t_next_v;  // meaningful in lane 0
+      if (round * nwaves < static_tickets) {
+        t_next_v = round * nwaves + ((round & 1) ? nwaves - 1 - my_wave : my_wave);
+      } else {
+        t_next_v = 0;
+        if (lane == 0) {
+          const int drawn = atomicAdd(&hdr[H_TICKET], 1);
+          if (drawn == dynamic_draws - 1) hdr[H_TICKET] = 0;  // nobody draws after this one
+          t_next_v = static_tickets + drawn;
+        }
+      }
       int4 n0 = r0, n1 = r1;  // harmless defaults for the first refresh below
       int nkvh = kvh, nmy_blk = my_blk, nseq[NRT];
 #pragma unroll
@@ -381,18 +404,20 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
       // ticket; both are idempotent, so no branch is needed.
       int ti = 0, trips = 0;
       if constexpr (NRT == 1) {
-        // two register buffers: the whole next tile is in flight while this one is consumed
+        // two register buffers, both already requested: k0/v0 = tile 0, k1/v1 = tile 1; a
+        // buffer is refilled two tiles ahead as soon as it has been consumed
         for (; ti + 1 < nfull; ti += 2, ++trips) {
-          load_tile(k1, v1, my_blk, nblk, kvh, ti + 1);
           compute_tile(k0, v0, ti, std::false_type{});
           load_tile(k0, v0, my_blk, nblk, kvh, min(ti + 2, last));
           compute_tile(k1, v1, ti + 1, std::false_type{});
-          load_lane_meta(n0, n1, nmy_blk, nseq);
-          load_record(t_next, n0, n1, nkvh);
+          load_tile(k1, v1, my_blk, nblk, kvh, min(ti + 3, last));
+          if (trips >= 1) {  // the first trip leaves a drawn ticket time to arrive
+            load_lane_meta(n0, n1, nmy_blk, nseq);
+            load_record(__builtin_amdgcn_readfirstlane(t_next_v), n0, n1, nkvh);
+          }
         }
-        // k0/v0 hold tile ti if ti < ntiles; zero, one or two tiles remain
+        // k0/v0 hold tile ti and k1/v1 tile ti + 1 (clamped); zero, one or two tiles remain
         if (ti < nfull) {
-          load_tile(k1, v1, my_blk, nblk, kvh, min(ti + 1, last));
           compute_tile(k0, v0, ti, std::false_type{});
           if (ti + 1 < ntiles) compute_tile(k1, v1, ti + 1, std::true_type{});
         } else if (ti < ntiles) {
@@ -407,27 +432,35 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
           load_k(k0, my_blk, nblk, kvh, min(ti + 1, last));
           weighted_values(v0, ti, std::false_type{});
           load_v(v0, my_blk, nblk, kvh, min(ti + 1, last));
-          load_lane_meta(n0, n1, nmy_blk, nseq);
-          load_record(t_next, n0, n1, nkvh);
+          if (trips >= 1) {
+            load_lane_meta(n0, n1, nmy_blk, nseq);
+            load_record(__builtin_amdgcn_readfirstlane(t_next_v), n0, n1, nkvh);
+          }
         }
         if (ti < ntiles) compute_tile(k0, v0, ti, std::true_type{});
       }
 
       // finish the chain for items too short to have done it on the way
-      if (trips < 1) load_record(t_next, n0, n1, nkvh);
-      if (trips < 2) load_lane_meta(n0, n1, nmy_blk, nseq);
+      const int t_next = __builtin_amdgcn_readfirstlane(t_next_v);
+      if (trips < 2) load_record(t_next, n0, n1, nkvh);
+      if (trips < 3) load_lane_meta(n0, n1, nmy_blk, nseq);
       const bool more = t_next < ntickets;
       if (more) {
         // q registers and both tile buffers are dead now: request the next item's query
         // rows and first tile before writing this item's partial
         load_q(nseq, n1.x, nkvh);
-        load_tile(k0, v0, nmy_blk, (__builtin_amdgcn_readfirstlane(n0.z) + kBlock - 1) / kBlock, nkvh, 0);
+        const int next_len = __builtin_amdgcn_readfirstlane(n0.z);
+        const int next_nblk = (next_len + kBlock - 1) / kBlock;
+        load_tile(k0, v0, nmy_blk, next_nblk, nkvh, 0);
+        if constexpr (NRT == 1) load_tile(k1, v1, nmy_blk, next_nblk, nkvh, next_len > kTile ? 1 : 0);
       }
 
-      // Normalise in registers (every accumulator register of a lane belongs to its own
-      // query row), then transpose 32 channels at a time through this wave's LDS slab so
-      // each partial row leaves as 128 contiguous bytes.  LDS operations of one wave execute
-      // in issue order; the fences only keep the compiler from reordering them.
+      // Write the partial.  Every accumulator register of a lane belongs to the lane's own
+      // query row, so normalisation is per lane; a lane stores its 4-channel groups straight
+      // from the accumulator layout (two lanes cover 32 adjacent bytes, the 16 stores of a
+      // row tile cover whole rows).  L2 is write-back, so the pieces of a line written within
+      // a microsecond by one wave leave for HBM as full lines; a transpose through LDS was
+      // measured and only added latency.
 #ifdef FCA_PROFILE
       const long long t_e0 = wall_clock64();
       n_items += 1;
@@ -440,29 +473,19 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
         if (rt > 0 && !two_tiles) continue;
         const float l = lrow[rt] + __shfl_xor(lrow[rt], 32);
         const float inv = vs / l;
-        if (h == 0 && prow[rt] >= 0) p.partial_lse[prow[rt]] = (mrow[rt] + fast_log2(l)) * kLn2;
-        const int orow = lane >> 3, opart = lane & 7;  // 8 rows per pass, 8 lanes x 16 bytes per row
+        if (prow[rt] >= 0) {
+          if (h == 0) p.partial_lse[prow[rt]] = (mrow[rt] + fast_log2(l)) * kLn2;
+          float* dst = p.partial_out + prow[rt] * D + h * 4;
 #pragma unroll
-        for (int db = 0; db < NDB; ++db) {
+          for (int db = 0; db < NDB; ++db)
 #pragma unroll
-          for (int q4 = 0; q4 < 4; ++q4) {
-            f32x4 v;
+            for (int q4 = 0; q4 < 4; ++q4) {
+              f32x4 v;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = acc[rt][db][q4 * 4 + e] * inv;
-            // accumulator register 4 * q4 + e holds channel 32 * db + 8 * q4 + 4 * h + e
-            *reinterpret_cast<f32x4*>(&lds_out[m * kOutStride + q4 * 8 + h * 4]) = v;
-          }
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          __builtin_amdgcn_wave_barrier();
-#pragma unroll
-          for (int pass = 0; pass < 4; ++pass) {
-            const int r = pass * 8 + orow;
-            const f32x4 v = *reinterpret_cast<const f32x4*>(&lds_out[r * kOutStride + opart * 4]);
-            const int64_t dst_row = __shfl(prow[rt], r);  // lanes 0..31 hold rows 0..31
-            if (dst_row >= 0) *reinterpret_cast<f32x4*>(p.partial_out + dst_row * D + db * 32 + opart * 4) = v;
-          }
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-          __builtin_amdgcn_wave_barrier();
+              for (int e = 0; e < 4; ++e) v[e] = acc[rt][db][q4 * 4 + e] * inv;
+              // accumulator register 4 * q4 + e holds channel 32 * db + 8 * q4 + 4 * h + e
+              *reinterpret_cast<f32x4*>(dst + db * 32 + q4 * 8) = v;
+            }
         }
       }
 #ifdef FCA_PROFILE

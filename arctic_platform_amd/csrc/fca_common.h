@@ -20,7 +20,7 @@ enum HeaderSlot {
   H_ITEMS = 0,
   H_SHARED_ITEMS = 1,
   H_NODES = 2,
-  H_RESERVED0 = 3,
+  H_TICKET = 3,
   H_RESERVED1 = 4,
   H_ERROR = 5,
   H_TOKENS_LO = 6,
