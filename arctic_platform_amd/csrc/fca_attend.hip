@@ -49,16 +49,10 @@ constexpr float kRescaleSlack = 8.f;  // log2 units: rescale when a row maximum 
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ inline float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
-template <bool FP8>
-struct RawV {
-  using type = i32x4;
-};
-template <>
-struct RawV<true> {
-  using type = i32x2;
-};
-
-// Raw operand registers of one 32-token tile.
+// Raw operand registers of one 32-token tile.  bf16 V: one 16-byte load per 32-channel
+// block and token block.  fp8 V: a lane fetches the whole 16-token row (16 bytes) of one
+// channel, lane half h taking the channel blocks of parity h; the halves are exchanged
+// with the lane 32 away just before use, so there is one load per pair of channel blocks.
 template <int D, bool FP8>
 struct KTile {
   static constexpr int NK = FP8 ? D / 32 : D / 16;  // 16-byte K loads per lane
@@ -66,26 +60,19 @@ struct KTile {
 };
 template <int D, bool FP8>
 struct VTile {
-  static constexpr int NDB = D / 32;  // 32-channel blocks of V per token block
-  typename RawV<FP8>::type v[2][NDB];
+  static constexpr int NV = FP8 ? D / 64 : D / 32;  // 16-byte V loads per lane and token block
+  i32x4 v[2][NV];
 };
 
-// 8 fp8 e4m3 values (two dwords) -> 8 bf16.  Exact: every e4m3 value is a bf16 value.
+// 8 fp8 e4m3 values (two dwords) -> 8 bf16 with the packed converter of gfx950 (scale 1:
+// every e4m3 value is a bf16 value, so the conversion is exact).
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 __device__ inline bf16x8 fp8x8_to_bf16(int lo, int hi) {
-  f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false);
-  f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8(lo, true);
-  f32x2 c = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false);
-  f32x2 d = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
-  bf16x8 r;
-  r[0] = (__bf16)a[0];
-  r[1] = (__bf16)a[1];
-  r[2] = (__bf16)b[0];
-  r[3] = (__bf16)b[1];
-  r[4] = (__bf16)c[0];
-  r[5] = (__bf16)c[1];
-  r[6] = (__bf16)d[0];
-  r[7] = (__bf16)d[1];
-  return r;
+  const bf16x2 a = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false);
+  const bf16x2 b = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true);
+  const bf16x2 c = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false);
+  const bf16x2 d = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true);
+  return bf16x8{a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
 }
 
 #ifdef FCA_PROFILE
@@ -138,8 +125,9 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
   // accumulator then holds, per lane half, tokens 8h..8h+7 of each block in register order.
   const int tok_of_m = (m & 3) | ((m & 4) << 1) | ((m & 8) >> 1);
   const int k_lane_off = h * 256 + tok_of_m * 16;
-  const int v_lane_off = FP8 ? m * 16 + h * 8 : m * 32 + h * 16;
-  constexpr int V_DB_STEP = FP8 ? 512 : 1024;
+  // bf16: channel 32 * db + m, tokens 8h..8h+7; fp8: channel 32 * (2 * pair + h) + m, all 16 tokens
+  const int v_lane_off = FP8 ? (h * 32 + m) * 16 : m * 32 + h * 16;
+  constexpr int V_STEP = 1024;
 
   const int nwaves = (int)gridDim.x * kWaves;
   const int static_tickets = min(ntickets, max(1, ntickets / nwaves - 1) * nwaves);
@@ -205,9 +193,9 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
     const char* vp0 = vbase + (int64_t)b0 * p.kv_block_bytes;
     const char* vp1 = vbase + (int64_t)b1 * p.kv_block_bytes;
 #pragma unroll
-    for (int db = 0; db < NDB; ++db) {
-      vt.v[0][db] = *reinterpret_cast<const typename RawV<FP8>::type*>(vp0 + db * V_DB_STEP);
-      vt.v[1][db] = *reinterpret_cast<const typename RawV<FP8>::type*>(vp1 + db * V_DB_STEP);
+    for (int i = 0; i < VT::NV; ++i) {
+      vt.v[0][i] = *reinterpret_cast<const i32x4*>(vp0 + i * V_STEP);
+      vt.v[1][i] = *reinterpret_cast<const i32x4*>(vp1 + i * V_STEP);
     }
   };
   auto load_tile = [&](KT& kt, VT& vt, int my_blk, int nblk, int kvh, int ti) {
@@ -227,14 +215,19 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
     load_record(my_wave, r0, r1, kvh);
     load_lane_meta(r0, r1, my_blk, seq);
     load_q(seq, r1.x, kvh);
-    KT k0, k1;
-    VT v0, v1;
-    {
-      const int first_len = __builtin_amdgcn_readfirstlane(r0.z);
-      const int first_nblk = (first_len + kBlock - 1) / kBlock;
-      load_tile(k0, v0, my_blk, first_nblk, kvh, 0);
-      if constexpr (NRT == 1) load_tile(k1, v1, my_blk, first_nblk, kvh, first_len > kTile ? 1 : 0);
-    }
+    // Tile buffers of the rotation.  All indices into kb/vb are compile-time constants
+    // after unrolling, so the buffers live in registers.  32-row tiles: two buffers;
+    // 64-row tiles: one buffer refilled in halves.
+    constexpr int NBUF = NRT > 1 ? 1 : 2;
+    KT kb[NBUF];
+    VT vb[NBUF];
+    auto request_first_tiles = [&](int blk_ids, int len, int head) {
+      const int nb = (len + kBlock - 1) / kBlock;
+      const int lt = (len + kTile - 1) / kTile - 1;
+#pragma unroll
+      for (int j = 0; j < NBUF; ++j) load_tile(kb[j], vb[j], blk_ids, nb, head, min(j, lt));
+    };
+    request_first_tiles(my_blk, __builtin_amdgcn_readfirstlane(r0.z), kvh);
 
     for (;;) {
       const int tok_len = __builtin_amdgcn_readfirstlane(r0.z);
@@ -359,7 +352,13 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
           for (int db = 0; db < NDB; ++db) {
             bf16x8 a;
             if constexpr (FP8) {
-              i32x2 w = vt.v[blk][db];
+              // rows of channel blocks 2 * pair and 2 * pair + 1 sit in the lower and upper
+              // lane halves; the swap hands every lane its tokens 8h..8h+7 of both blocks:
+              // dwords 0,1 become the operand of block 2 * pair, dwords 2,3 of 2 * pair + 1
+              const i32x4 raw = vt.v[blk][db >> 1];
+              const auto s0 = __builtin_amdgcn_permlane32_swap((unsigned)raw[0], (unsigned)raw[2], false, false);
+              const auto s1 = __builtin_amdgcn_permlane32_swap((unsigned)raw[1], (unsigned)raw[3], false, false);
+              i32x2 w = {(int)s0[db & 1], (int)s1[db & 1]};
               if constexpr (RAGGED) {
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
@@ -396,7 +395,7 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
         weighted_values(vt, ti, ragged);
       };
 
-      // Tile pipeline; k0/v0 already hold (or await) tile 0.  Prefetches past the end are
+      // Tile pipeline; the first tiles are already requested.  Prefetches past the end are
       // clamped to the last tile instead of skipped, so the outstanding-load count is the
       // same on every path and every wait covers exactly the tile about to be used.  Each
       // trip also advances the next item's chain by one hop: the per-lane data is (re)read
@@ -404,40 +403,43 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
       // ticket; both are idempotent, so no branch is needed.
       int ti = 0, trips = 0;
       if constexpr (NRT == 1) {
-        // two register buffers, both already requested: k0/v0 = tile 0, k1/v1 = tile 1; a
-        // buffer is refilled two tiles ahead as soon as it has been consumed
-        for (; ti + 1 < nfull; ti += 2, ++trips) {
-          compute_tile(k0, v0, ti, std::false_type{});
-          load_tile(k0, v0, my_blk, nblk, kvh, min(ti + 2, last));
-          compute_tile(k1, v1, ti + 1, std::false_type{});
-          load_tile(k1, v1, my_blk, nblk, kvh, min(ti + 3, last));
+        // all NBUF buffers are already requested (tiles 0 .. NBUF-1, clamped); a buffer is
+        // refilled NBUF tiles ahead as soon as it has been consumed
+        for (; ti + NBUF - 1 < nfull; ti += NBUF, ++trips) {
+#pragma unroll
+          for (int j = 0; j < NBUF; ++j) {
+            compute_tile(kb[j], vb[j], ti + j, std::false_type{});
+            load_tile(kb[j], vb[j], my_blk, nblk, kvh, min(ti + NBUF + j, last));
+          }
           if (trips >= 1) {  // the first trip leaves a drawn ticket time to arrive
             load_lane_meta(n0, n1, nmy_blk, nseq);
             load_record(__builtin_amdgcn_readfirstlane(t_next_v), n0, n1, nkvh);
           }
         }
-        // k0/v0 hold tile ti and k1/v1 tile ti + 1 (clamped); zero, one or two tiles remain
-        if (ti < nfull) {
-          compute_tile(k0, v0, ti, std::false_type{});
-          if (ti + 1 < ntiles) compute_tile(k1, v1, ti + 1, std::true_type{});
-        } else if (ti < ntiles) {
-          compute_tile(k0, v0, ti, std::true_type{});
+        // buffer j holds tile ti + j (clamped); fewer than NBUF full tiles remain, and
+        // possibly the ragged one
+#pragma unroll
+        for (int j = 0; j < NBUF; ++j) {
+          if (ti + j < nfull)
+            compute_tile(kb[j], vb[j], ti + j, std::false_type{});
+          else if (ti + j < ntiles)
+            compute_tile(kb[j], vb[j], ti + j, std::true_type{});
         }
       } else {
         // 64 query rows leave no room for a second tile buffer: one buffer, refilled in
         // halves -- the next K as soon as the scores have issued, the next V as soon as the
         // value product has
         for (; ti < nfull; ++ti, ++trips) {
-          scores_softmax(k0, ti, std::false_type{});
-          load_k(k0, my_blk, nblk, kvh, min(ti + 1, last));
-          weighted_values(v0, ti, std::false_type{});
-          load_v(v0, my_blk, nblk, kvh, min(ti + 1, last));
+          scores_softmax(kb[0], ti, std::false_type{});
+          load_k(kb[0], my_blk, nblk, kvh, min(ti + 1, last));
+          weighted_values(vb[0], ti, std::false_type{});
+          load_v(vb[0], my_blk, nblk, kvh, min(ti + 1, last));
           if (trips >= 1) {
             load_lane_meta(n0, n1, nmy_blk, nseq);
             load_record(__builtin_amdgcn_readfirstlane(t_next_v), n0, n1, nkvh);
           }
         }
-        if (ti < ntiles) compute_tile(k0, v0, ti, std::true_type{});
+        if (ti < ntiles) compute_tile(kb[0], vb[0], ti, std::true_type{});
       }
 
       // finish the chain for items too short to have done it on the way
@@ -449,10 +451,7 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
         // q registers and both tile buffers are dead now: request the next item's query
         // rows and first tile before writing this item's partial
         load_q(nseq, n1.x, nkvh);
-        const int next_len = __builtin_amdgcn_readfirstlane(n0.z);
-        const int next_nblk = (next_len + kBlock - 1) / kBlock;
-        load_tile(k0, v0, nmy_blk, next_nblk, nkvh, 0);
-        if constexpr (NRT == 1) load_tile(k1, v1, nmy_blk, next_nblk, nkvh, next_len > kTile ? 1 : 0);
+        request_first_tiles(nmy_blk, __builtin_amdgcn_readfirstlane(n0.z), nkvh);
       }
 
       // Write the partial.  Every accumulator register of a lane belongs to the lane's own
@@ -536,7 +535,8 @@ static int env_int(const char* name, int fallback) {
 hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, hipStream_t stream) {
   const bool fp8 = kv_dtype == FCA_FP8_E4M3;
   const int nrt = plan.rows_per_item / 32;
-  // one workgroup of four independent waves per CU (the kernel needs the whole register file)
+  // one workgroup of four independent waves per CU (the kernel uses the whole register
+  // file; two waves per SIMD were measured for the fp8 kernel, which would fit, and lost)
   static const int wgs_per_cu = env_int("FCA_WGS_PER_CU", 1);
   const int64_t max_tickets = (int64_t)plan.num_seqs *
                               ((int64_t)plan.max_blocks * kBlock / plan.chunk_tokens + plan.max_levels + 1) *
