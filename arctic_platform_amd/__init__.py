@@ -15,6 +15,7 @@ __all__ = [
     "convert_cache",
     "build_forest_metadata",
     "forest_cascade_decode",
+    "append_kv",
 ]
 
 
@@ -29,4 +30,8 @@ def __getattr__(name):
         from . import ops
 
         return getattr(ops, name)
+    if name == "append_kv":
+        from . import cache
+
+        return cache.append_kv
     raise AttributeError(name)

@@ -28,6 +28,7 @@ EXPORTS = (
     "fca_forest_pass",
     "fca_merge",
     "fca_decode_step",
+    "fca_append_kv",
     "fca_calibration_copy",
 )
 
@@ -133,6 +134,7 @@ def load_library() -> ctypes.CDLL:
     lib.fca_forest_pass.argtypes = attend
     lib.fca_merge.argtypes = [P(FcaPlan), VP, VP, VP, VP, I64, I64, I32, VP, VP]
     lib.fca_decode_step.argtypes = [P(FcaPlan), P(FcaTensors), VP, VP, VP, VP, I64, I64, I32, VP, VP]
+    lib.fca_append_kv.argtypes = [VP, VP, I64, I64, I32, I32, I32, VP, VP, VP, I64, I64, I32, VP, VP, VP]
     lib.fca_calibration_copy.argtypes = [VP, VP, ctypes.c_size_t, VP]
     for name in EXPORTS:
         if name not in ("fca_version", "fca_last_error"):

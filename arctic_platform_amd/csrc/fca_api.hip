@@ -223,6 +223,43 @@ int fca_decode_step(const fca_plan* plan, const fca_tensors* t, void* meta_dev, 
                    lse_dev, stream);
 }
 
+int fca_append_kv(const void* key_dev, const void* value_dev, int64_t token_stride, int64_t head_stride,
+                  int32_t num_tokens, int32_t num_kv_heads, int32_t head_dim, const int64_t* slot_mapping_dev,
+                  void* k_cache_dev, void* v_cache_dev, int64_t kv_block_stride, int64_t kv_head_stride, int32_t kv_dtype,
+                  const float* k_scale_dev, const float* v_scale_dev, void* stream) {
+  if (num_tokens < 0 || num_kv_heads < 1) return fail(FCA_ERR_INVALID_ARG, "num_tokens must be >= 0 and num_kv_heads >= 1");
+  if (head_dim != 64 && head_dim != 128) return fail(FCA_ERR_UNSUPPORTED, "head_dim %d is not supported (64 or 128)", head_dim);
+  if (kv_dtype != FCA_BF16 && kv_dtype != FCA_FP8_E4M3)
+    return fail(FCA_ERR_UNSUPPORTED, "kv_dtype %d is not supported (bf16 or fp8 e4m3)", kv_dtype);
+  if (num_tokens == 0) return FCA_OK;
+  if (!key_dev || !value_dev || !slot_mapping_dev || !k_cache_dev || !v_cache_dev)
+    return fail(FCA_ERR_INVALID_ARG, "key, value, slot_mapping and the cache planes must be non-NULL");
+  const int esz = kv_dtype == FCA_FP8_E4M3 ? 1 : 2;
+  if ((reinterpret_cast<uintptr_t>(key_dev) & 15) || (reinterpret_cast<uintptr_t>(value_dev) & 15) || token_stride % 8 ||
+      head_stride % 8)
+    return fail(FCA_ERR_INVALID_ARG, "key and value must be 16-byte aligned with strides that are multiples of 8 elements");
+  if ((reinterpret_cast<uintptr_t>(k_cache_dev) & 15) || (reinterpret_cast<uintptr_t>(v_cache_dev) & 15) ||
+      (kv_block_stride * esz) % 16 || (kv_head_stride * esz) % 16 || kv_head_stride < (int64_t)FCA_BLOCK_SIZE * head_dim)
+    return fail(FCA_ERR_INVALID_ARG, "KV cache planes must be 16-byte aligned with 16-byte-multiple strides of at least one tile");
+  fca::AppendParams a{};
+  a.key = key_dev;
+  a.value = value_dev;
+  a.token_stride = token_stride;
+  a.head_stride = head_stride;
+  a.slot_mapping = slot_mapping_dev;
+  a.k_cache = k_cache_dev;
+  a.v_cache = v_cache_dev;
+  a.cache_block_stride = kv_block_stride;
+  a.cache_head_stride = kv_head_stride;
+  a.k_scale = k_scale_dev;
+  a.v_scale = v_scale_dev;
+  a.num_tokens = num_tokens;
+  a.num_kv_heads = num_kv_heads;
+  a.head_dim = head_dim;
+  hipError_t e = fca::launch_append(a, kv_dtype, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? FCA_OK : hip_fail(e, "cache append launch");
+}
+
 int fca_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void* stream) {
   if (!src_dev || !dst_dev || (bytes & 15) || (reinterpret_cast<uintptr_t>(src_dev) & 15) ||
       (reinterpret_cast<uintptr_t>(dst_dev) & 15))

@@ -56,8 +56,7 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   __shared__ int lds_cursor[2 * kSizeBuckets];
   __shared__ unsigned long long lds_tokens;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int nwaves = kBuildThreads / 64;
+  const int tid = threadIdx.x;
   const int S = p.plan.num_seqs;
   const int chunk = p.plan.chunk_tokens;
   const int group = p.plan.num_q_heads / p.plan.num_kv_heads;
@@ -134,25 +133,31 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       }
     }
     __syncthreads();
-    // Common run with the leader: one wave per sequence, 256 positions per round.
-    for (int s = wave; s < S; s += nwaves) {
-      const int t = leader[s];
-      if (t < 0 || t == s) continue;
-      const int lim = min(nfull[s], nfull[t]) - pos[s];
-      const int32_t* row_s = p.block_table + s * p.bt_stride + pos[s];
-      const int32_t* row_t = p.block_table + t * p.bt_stride + pos[s];
-      int first = lim;
-      for (int j0 = 0; j0 < lim && first == lim; j0 += 256) {
-        int mine = lim;
+    // Common run with the leader = first position where the two rows differ.  Every group
+    // of 16 lanes takes its own sequence (64 sequences in flight per pass) and scans 256
+    // positions per round, 16 independent loads per lane and row.
+    {
+      const int gid = tid >> 4, glane = tid & 15;
+      constexpr int kGroups = kBuildThreads / 16, kPerLane = 16;
+      for (int s = gid; s < S; s += kGroups) {
+        const int t = leader[s];
+        if (t < 0 || t == s) continue;
+        const int lim = min(nfull[s], nfull[t]) - pos[s];
+        const int32_t* row_s = p.block_table + s * p.bt_stride + pos[s];
+        const int32_t* row_t = p.block_table + t * p.bt_stride + pos[s];
+        int first = lim;
+        for (int j0 = 0; j0 < lim && first == lim; j0 += 16 * kPerLane) {
+          int mine = lim;
 #pragma unroll
-        for (int u = 3; u >= 0; --u) {
-          int j = j0 + u * 64 + lane;
-          if (j < lim && row_s[j] != row_t[j]) mine = j;
+          for (int u = kPerLane - 1; u >= 0; --u) {
+            const int j = j0 + u * 16 + glane;
+            if (j < lim && row_s[j] != row_t[j]) mine = j;
+          }
+          for (int off = 8; off; off >>= 1) mine = min(mine, __shfl_xor(mine, off, 16));
+          first = mine;
         }
-        for (int off = 32; off; off >>= 1) mine = min(mine, __shfl_xor(mine, off));
-        first = mine;
+        if (glane == 0) lcp[s] = min(lcp[s], first);
       }
-      if (lane == 0) lcp[s] = min(lcp[s], first);
     }
     __syncthreads();
     for (int s = tid; s < S; s += kBuildThreads) {
@@ -188,15 +193,14 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
     }
     __syncthreads();
     // Member lists in ascending sequence order: rank = members of the same leader below s.
-    for (int s = wave; s < S; s += nwaves) {
+    // One thread per sequence scans [leader, s); the members of a group are usually
+    // adjacent rows, so the scan is a handful of steps.
+    for (int s = tid; s < S; s += kBuildThreads) {
       const int t = leader[s];
       if (t < 0 || cnt[t] < 2) continue;
       int below = 0;
-      for (int j0 = t; j0 < s; j0 += 64) {
-        int j = j0 + lane;
-        below += __popcll(__ballot(j < s && leader[j] == t));
-      }
-      if (lane == 0) members[meta[L.node_moff + tmp0[t]] + below] = s;
+      for (int j = t; j < s; ++j) below += leader[j] == t ? 1 : 0;
+      members[meta[L.node_moff + tmp0[t]] + below] = s;
     }
     __syncthreads();
     for (int s = tid; s < S; s += kBuildThreads) {

@@ -145,7 +145,21 @@ struct MergeParams {
   int32_t num_seqs, num_q_heads, head_dim, max_partials, out_dtype;
 };
 
+struct AppendParams {
+  const void* key;    // bf16 [T, Hkv, D]
+  const void* value;
+  int64_t token_stride, head_stride;  // elements
+  const int64_t* slot_mapping;        // [T]
+  void* k_cache;
+  void* v_cache;
+  int64_t cache_block_stride, cache_head_stride;  // elements
+  const float* k_scale;
+  const float* v_scale;
+  int32_t num_tokens, num_kv_heads, head_dim;
+};
+
 hipError_t launch_build(const BuildParams& p, hipStream_t stream);
+hipError_t launch_append(const AppendParams& p, int kv_dtype, hipStream_t stream);
 hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, hipStream_t stream);
 hipError_t launch_merge(const MergeParams& p, hipStream_t stream);
 hipError_t launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);

@@ -140,6 +140,17 @@ int fca_decode_step(const fca_plan* plan, const fca_tensors* t, void* meta_dev,
                     float* partial_out_dev, float* partial_lse_dev, void* out_dev, int64_t out_seq_stride,
                     int64_t out_head_stride, int32_t out_dtype, float* lse_dev, void* stream);
 
+/* KV-cache append, the step before decode attention in every layer: scatter the new
+ * tokens' K and V (bf16 [T, Hkv, D]) into the cache tiles at slot = block * 16 + offset
+ * (negative slot = padding, skipped), quantising to fp8 e4m3 with per-KV-head scales
+ * (stored = clamp(x / scale, +-448) rounded to nearest even) when kv_dtype says so.
+ * Replaces the external engine's cache-write op on this layout; in-tree the reference only
+ * names the cache dtype it forwards to that engine (vllm_config, server_models.py:143-165). */
+int fca_append_kv(const void* key_dev, const void* value_dev, int64_t token_stride, int64_t head_stride,
+                  int32_t num_tokens, int32_t num_kv_heads, int32_t head_dim, const int64_t* slot_mapping_dev,
+                  void* k_cache_dev, void* v_cache_dev, int64_t kv_block_stride, int64_t kv_head_stride, int32_t kv_dtype,
+                  const float* k_scale_dev, const float* v_scale_dev, void* stream);
+
 /* Plain device-to-device copy with 16-byte loads and stores.  No counterpart in the
  * reference: it is the known-size yardstick for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE
  * readings of the kernels above. */
