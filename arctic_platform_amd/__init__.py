@@ -30,6 +30,10 @@ def __getattr__(name):
         from . import ops
 
         return getattr(ops, name)
+    if name in ("ForestCascadeAttentionBackend", "ForestCascadeMetadataBuilder", "ForestCascadeAttentionImpl"):
+        from . import backend
+
+        return getattr(backend, name)
     if name == "append_kv":
         from . import cache
 

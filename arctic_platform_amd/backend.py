@@ -1,0 +1,190 @@
+"""Attention-backend surface of forest cascade attention.
+
+The platform's sampling job hands attention to its engine's backend plug-in: the engine
+asks the backend for the KV-cache shape, calls a metadata builder once per scheduler
+step and the implementation's ``forward`` once per attention layer
+(engine start-up: arctic_platform/common/ray_server.py:395-404; the feature switch that
+selects this backend: arctic_platform/common/utils/server_models.py:123-140 and the raw
+engine kwarg ``forest_cascade_attn_configs`` used by
+recipes/rl/skyrl/txt2sql/run_qwen3_8b_bird_grpo_arl.sh:98-111).  The engine itself is
+not part of the reference tree, so the class and argument names below follow the engine's
+public plug-in convention from its documentation, not from code in the reference.
+
+Decode batches only (one query token per sequence).  Prefill and mixed batches belong to
+a stock backend on the same cache; they are rejected here with a clear error when the
+metadata is built, never in the middle of a layer.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+import json
+
+import torch
+
+from .cache import append_kv
+from .config import ModelConfig, validate_fca_support
+from .forest import ForestMetadata, build_forest_metadata
+from .kv_layout import BLOCK_SIZE, kv_cache_shape
+from .ops import forest_cascade_decode
+
+
+@dataclasses.dataclass
+class CommonAttentionMetadata:
+    """The per-step fields of the engine's common metadata that this backend reads."""
+
+    query_start_loc: torch.Tensor  # [num_reqs + 1] int32, cumulative query tokens
+    seq_lens: torch.Tensor  # [num_reqs] int32, tokens in the cache incl. the new one
+    block_table_tensor: torch.Tensor  # [num_reqs, max_blocks] int32
+    slot_mapping: torch.Tensor  # [num_tokens] int64
+    num_reqs: int
+    max_query_len: int
+    num_actual_tokens: int | None = None
+
+
+@dataclasses.dataclass
+class ForestCascadeMetadata:
+    forest: ForestMetadata
+    slot_mapping: torch.Tensor
+    num_decode_tokens: int
+
+
+def parse_forest_cascade_configs(value) -> dict:
+    """``forest_cascade_attn_configs`` arrives as a JSON string (``"{}"`` in the recipes)
+    or a dict.  Known keys: chunk_tokens, rows_per_item, max_levels, enable."""
+    if value is None or value == "":
+        return {}
+    cfg = json.loads(value) if isinstance(value, str) else dict(value)
+    unknown = set(cfg) - {"chunk_tokens", "rows_per_item", "max_levels", "enable"}
+    if unknown:
+        raise ValueError(f"unknown forest_cascade_attn_configs keys: {sorted(unknown)}")
+    return cfg
+
+
+class ForestCascadeAttentionBackend:
+    accept_output_buffer = True
+
+    @staticmethod
+    def get_name() -> str:
+        return "FOREST_CASCADE_ATTN"
+
+    @staticmethod
+    def get_impl_cls():
+        return ForestCascadeAttentionImpl
+
+    @staticmethod
+    def get_metadata_cls():
+        return ForestCascadeMetadata
+
+    @staticmethod
+    def get_builder_cls():
+        return ForestCascadeMetadataBuilder
+
+    @staticmethod
+    def get_supported_head_sizes():
+        return [64, 128]
+
+    @staticmethod
+    def get_kv_cache_shape(num_blocks: int, block_size: int, num_kv_heads: int, head_size: int):
+        return kv_cache_shape(num_blocks, block_size, num_kv_heads, head_size)
+
+
+class ForestCascadeMetadataBuilder:
+    """Builds the forest once per scheduler step.  Workspaces are kept per batch shape
+    (num_reqs, max_blocks), so a steady decode loop allocates nothing."""
+
+    def __init__(self, num_q_heads, num_kv_heads, head_dim, device="cuda", forest_cascade_attn_configs=None):
+        cfg = parse_forest_cascade_configs(forest_cascade_attn_configs)
+        validate_fca_support(
+            ModelConfig(use_fca=True), head_dim=head_dim, num_q_heads=num_q_heads, num_kv_heads=num_kv_heads
+        )
+        self.num_q_heads, self.num_kv_heads, self.head_dim = num_q_heads, num_kv_heads, head_dim
+        self.device = torch.device(device)
+        self.enabled = bool(cfg.get("enable", True))
+        self.chunk_tokens = int(cfg.get("chunk_tokens", 1024))
+        self.max_levels = int(cfg.get("max_levels", 4))
+        group = num_q_heads // num_kv_heads
+        self.rows_per_item = int(cfg.get("rows_per_item", 64 if group > 32 else 32))
+        if group > self.rows_per_item:
+            raise ValueError(f"{group} query heads per KV head do not fit rows_per_item={self.rows_per_item}")
+        self._workspaces: dict = {}
+
+    def build(self, common_prefix_len: int, common_attn_metadata: CommonAttentionMetadata) -> ForestCascadeMetadata:
+        m = common_attn_metadata
+        if m.max_query_len != 1:
+            raise NotImplementedError(
+                "forest cascade attention handles decode batches (one query token per sequence); "
+                f"got max_query_len={m.max_query_len}: route prefill and mixed batches to a stock backend"
+            )
+        bt, sl = m.block_table_tensor[: m.num_reqs], m.seq_lens[: m.num_reqs]
+        key = (m.num_reqs, bt.shape[1])
+        forest = build_forest_metadata(
+            bt,
+            sl,
+            num_q_heads=self.num_q_heads,
+            num_kv_heads=self.num_kv_heads,
+            head_dim=self.head_dim,
+            block_size=BLOCK_SIZE,
+            chunk_tokens=self.chunk_tokens,
+            rows_per_item=self.rows_per_item,
+            cascade=self.enabled,
+            max_levels=self.max_levels,
+            out=self._workspaces.get(key),
+        )
+        self._workspaces[key] = forest
+        return ForestCascadeMetadata(forest=forest, slot_mapping=m.slot_mapping[: m.num_reqs], num_decode_tokens=m.num_reqs)
+
+
+class ForestCascadeAttentionImpl:
+    def __init__(
+        self,
+        num_heads: int,
+        head_size: int,
+        scale: float,
+        num_kv_heads: int | None = None,
+        alibi_slopes=None,
+        sliding_window=None,
+        kv_cache_dtype: str = "auto",
+        logits_soft_cap=None,
+        attn_type: str = "decoder",
+    ):
+        if alibi_slopes is not None or sliding_window is not None or logits_soft_cap is not None:
+            raise NotImplementedError("forest cascade attention supports plain softmax attention only (no ALiBi, sliding window or soft cap)")
+        if attn_type != "decoder":
+            raise NotImplementedError(f"attention type {attn_type!r} is not supported")
+        self.num_heads = num_heads
+        self.num_kv_heads = num_kv_heads or num_heads
+        self.head_size = head_size
+        self.scale = float(scale)
+        self.kv_cache_dtype = kv_cache_dtype
+        validate_fca_support(
+            ModelConfig(use_fca=True, kv_cache_dtype=kv_cache_dtype),
+            head_dim=head_size,
+            num_q_heads=num_heads,
+            num_kv_heads=self.num_kv_heads,
+        )
+
+    def forward(self, layer, query, key, value, kv_cache, attn_metadata: ForestCascadeMetadata, output=None):
+        """query ``[T, Hq*D]`` or ``[T, Hq, D]``; key/value ``[T, Hkv*D]`` / ``[T, Hkv, D]`` or
+        None when the cache already holds the step's tokens; returns ``output`` shaped like
+        ``query``.  Per-KV-head fp8 scales are read from ``layer.k_scale`` / ``layer.v_scale``."""
+        t = attn_metadata.num_decode_tokens
+        q = query[:t].view(t, self.num_heads, self.head_size)
+        k_scale = getattr(layer, "k_scale", None)
+        v_scale = getattr(layer, "v_scale", None)
+        if key is not None:
+            append_kv(
+                key[:t].view(t, self.num_kv_heads, self.head_size),
+                value[:t].view(t, self.num_kv_heads, self.head_size),
+                kv_cache,
+                attn_metadata.slot_mapping,
+                k_scale,
+                v_scale,
+            )
+        if output is None:
+            output = torch.empty_like(query)
+        forest_cascade_decode(
+            q, kv_cache, attn_metadata.forest, self.scale, k_scale, v_scale,
+            out=output[:t].view(t, self.num_heads, self.head_size), return_lse=False,
+        )
+        return output
