@@ -21,23 +21,28 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
   const int np = p.seq_npart[s];
   const int64_t base = (int64_t)s * p.max_partials;
 
-  float m = -INFINITY;
-  for (int i = 0; i < np; ++i) m = fmaxf(m, p.partial_lse[(base + i) * p.num_q_heads + hq]);
+  // One online pass (running maximum, rescaled sum): the loads of successive partials do
+  // not depend on each other, so unrolling keeps several of them in flight.
+  float m = -INFINITY, wsum = 0.f;
   float acc[V];
 #pragma unroll
   for (int e = 0; e < V; ++e) acc[e] = 0.f;
-  float wsum = 0.f;
-  if (m > -INFINITY) {
-    for (int i = 0; i < np; ++i) {
-      const int64_t pr = (base + i) * p.num_q_heads + hq;
-      const float l = p.partial_lse[pr];
-      if (!(l > -INFINITY)) continue;  // empty partial: weight 0, its output is not read
-      const float w = __expf(l - m);
-      wsum += w;
-      const float* src = p.partial_out + pr * D + sub * V;
+#pragma unroll 4
+  for (int i = 0; i < np; ++i) {
+    const int64_t pr = (base + i) * p.num_q_heads + hq;
+    const float l = p.partial_lse[pr];
+    float o[V];
+    const float* src = p.partial_out + pr * D + sub * V;
 #pragma unroll
-      for (int e = 0; e < V; ++e) acc[e] += w * src[e];
-    }
+    for (int e = 0; e < V; ++e) o[e] = src[e];
+    if (!(l > -INFINITY)) continue;  // empty partial: weight 0, whatever its output holds
+    const float m_new = fmaxf(m, l);
+    const float keep = __expf(m - m_new);  // exp(-inf) = 0 on the first live partial
+    const float w = __expf(l - m_new);
+    wsum = wsum * keep + w;
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = acc[e] * keep + w * o[e];
+    m = m_new;
   }
   const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
   const int64_t o = (int64_t)s * p.out_seq_stride + (int64_t)hq * p.out_head_stride + sub * V;
