@@ -202,7 +202,7 @@ def main():
             "builder_per_step": round(build_us / args.layers, 2),
         },
         "roofline": {
-            "kernel": "fca_attend_kernel",
+            "kernel": "fca_attend_stream_kernel",
             "bound": "hbm",
             "achieved": round(unique_bytes / (kern * 1e-6) / 1e9, 1),
             "peak": HBM_PEAK_GBS,

@@ -86,7 +86,8 @@ typedef struct fca_tensors {
  * inspection and tests.  Item records are 8 x int32:
  * {rep_seq, blk_start, tok_len, member_off, member_cnt, ord, node, 0}. */
 typedef struct fca_meta_layout {
-  int64_t header;        /* [16]: 0 items, 1 shared items, 2 nodes (shared), 3-4 reserved,
+  int64_t header;        /* [16]: 0 items, 1 shared items, 2 nodes (shared), 3 work ticket
+                            (self-resetting, owned by the attention kernel), 4 reserved,
                             5 error flag, 6/7 unique tokens lo/hi, 8 levels found */
   int64_t seq_npart;     /* [S] partial slots used per sequence */
   int64_t seq_leaf_blk;  /* [S] first block position of the private leaf */
