@@ -29,51 +29,9 @@
 #include <cstring>
 #include <type_traits>
 
-#include "fca_common.h"
+#include "fca_attend_common.h"
 
 namespace fca {
-
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef int i32x4 __attribute__((ext_vector_type(4)));
-typedef int i32x2 __attribute__((ext_vector_type(2)));
-
-constexpr int kThreads = 256;
-constexpr int kWaves = 4;
-constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kLn2 = 0.6931471805599453f;
-constexpr float kRescaleSlack = 8.f;  // log2 units: rescale when a row maximum rises by more than 2^8
-
-__device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-__device__ inline float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
-
-// Raw operand registers of one 32-token tile.  bf16 V: one 16-byte load per 32-channel
-// block and token block.  fp8 V: a lane fetches the whole 16-token row (16 bytes) of one
-// channel, lane half h taking the channel blocks of parity h; the halves are exchanged
-// with the lane 32 away just before use, so there is one load per pair of channel blocks.
-template <int D, bool FP8>
-struct KTile {
-  static constexpr int NK = FP8 ? D / 32 : D / 16;  // 16-byte K loads per lane
-  i32x4 k[NK];
-};
-template <int D, bool FP8>
-struct VTile {
-  static constexpr int NV = FP8 ? D / 64 : D / 32;  // 16-byte V loads per lane and token block
-  i32x4 v[2][NV];
-};
-
-// 8 fp8 e4m3 values (two dwords) -> 8 bf16 with the packed converter of gfx950 (scale 1:
-// every e4m3 value is a bf16 value, so the conversion is exact).
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-__device__ inline bf16x8 fp8x8_to_bf16(int lo, int hi) {
-  const bf16x2 a = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false);
-  const bf16x2 b = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true);
-  const bf16x2 c = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false);
-  const bf16x2 d = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true);
-  return bf16x8{a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
-}
 
 #ifdef FCA_PROFILE
 __device__ long long* g_prof = nullptr;  // [waves][8] wall-clock ticks (100 MHz), debug builds only
@@ -544,6 +502,8 @@ hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dty
   int grid = cached_cu_count() * wgs_per_cu;
   if ((int64_t)grid * kWaves > max_tickets) grid = (int)((max_tickets + kWaves - 1) / kWaves);
   if (grid < 1) grid = 1;
+  static const int use32 = env_int("FCA_ATTEND32", 1);
+  if (nrt == 1 && use32) return launch_attend32(p, plan, kv_dtype, grid, stream);
 #define FCA_LAUNCH(D_, N_, F_) \
   hipLaunchKernelGGL((fca_attend_stream_kernel<D_, N_, F_>), dim3(grid), dim3(kThreads), 0, stream, p)
   if (plan.head_dim == 128) {

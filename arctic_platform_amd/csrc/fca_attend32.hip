@@ -1,0 +1,452 @@
+// Forest cascade attention pass for query tiles of up to 32 rows: the tile stream of a
+// wave never drains at an item boundary.
+//
+// Same work items, arithmetic and register-staged tiles as the kernel in fca_attend.hip;
+// what differs is the schedule around the boundaries between items.  A wave looks four
+// items ahead: at one fixed point of every item it takes one step for each of the
+// following items -- query rows of item k+1, block ids and member sequences of item k+2,
+// record of item k+3, ticket of item k+4 -- so every step reads what the step before it
+// fetched one whole item earlier, and nothing is ever waited for at the place it was
+// requested.  With the next item's block ids at hand, the two tile buffers are refilled
+// with the next item's first tiles as soon as the current item's last tiles have been
+// consumed, exactly as they are refilled inside an item.
+//
+// All loads sit at fixed places of the instruction stream (none inside a data-dependent
+// branch): the hardware counts outstanding vector memory operations in order and the
+// compiler picks each wait's count for the shortest path, so a load issued on only some
+// paths would turn the waits behind it into full drains of the tile stream.
+#include <type_traits>
+
+#include "fca_attend_common.h"
+
+namespace fca {
+
+#ifdef FCA_PROFILE
+__device__ long long* g_prof32 = nullptr;
+#define STAMP(i) { const long long t_ = wall_clock64(); prof[i] += t_ - t_prev; t_prev = t_; }
+#else
+#define STAMP(i)
+#endif
+
+template <int D, bool FP8, bool STREAM>
+__global__ __launch_bounds__(kThreads, 1) void fca_attend32_kernel(AttendParams p) {
+  constexpr int KS = D / 16;   // MFMA steps of the score product
+  constexpr int NDB = D / 32;  // 32-channel blocks of the output
+  using KT = KTile<D, FP8>;
+  using VT = VTile<D, FP8>;
+
+  int32_t* hdr = p.meta + p.off_header;
+  const int total = hdr[H_ITEMS], shared = hdr[H_SHARED_ITEMS];
+  const int first = p.select == 2 ? shared : 0;
+  const int last_item = p.select == 1 ? shared : total;
+  const int ntickets = (last_item - first) * p.num_kv_heads;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int m = lane & 31, h = lane >> 5;
+  const int G = p.group, Hkv = p.num_kv_heads;
+  const int32_t* meta = p.meta;
+  const int nwaves = (int)gridDim.x * kWaves;
+  const int my_wave = (int)blockIdx.x * kWaves + wave;
+  if (my_wave >= ntickets) return;
+
+  // row m of the stacked query tile is (member m / G, head m % G)
+  const int row_member = m / G;
+  const int row_head = m - row_member * G;
+  // MFMA row m carries the token whose index has bits 2 and 3 of m swapped: the score
+  // accumulator then holds, per lane half, tokens 8h..8h+7 of each block in register order.
+  const int tok_of_m = (m & 3) | ((m & 4) << 1) | ((m & 8) >> 1);
+  const int k_lane_off = h * 256 + tok_of_m * 16;
+  // bf16: channel 32 * db + m, tokens 8h..8h+7; fp8: channel 32 * (2 * pair + h) + m, all 16 tokens
+  const int v_lane_off = FP8 ? (h * 32 + m) * 16 : m * 32 + h * 16;
+  constexpr int V_STEP = 1024;
+  // wave-private strip of LDS for the output rows: D values + the partial row index
+  constexpr int kStripStride = D + 4;  // floats; keeps rows 16-byte aligned
+  __shared__ float strips[kWaves][32 * kStripStride];
+  float* strip = strips[wave];
+
+  // Dealing the work.  Round r gives wave w of W ticket r * W + w (r even) or
+  // r * W + W - 1 - w (r odd) over the size-ordered list, for all rounds but the last full
+  // one and the remainder: those come from a counter in the metadata header, drawn four
+  // items ahead of use, so a wave that streams faster takes more of the small items.  A
+  // list shorter than five rounds is dealt statically as a whole.  Every wave draws until
+  // its first failing draw; the draw that returns the last possible value resets the
+  // counter for the next launch.
+  const int static_tickets = ntickets < 5 * nwaves ? ntickets : (ntickets / nwaves - 1) * nwaves;
+  const int dynamic_draws = ntickets - static_tickets + nwaves;
+  bool drawing = static_tickets < ntickets;
+  // A zero the compiler cannot see through; it makes an address look lane-dependent.
+  int opaque_zero;
+  asm volatile("v_mov_b32 %0, 0" : "=v"(opaque_zero));
+  // Tickets of static rounds are computed when they are resolved.  A drawn ticket lives
+  // in lane 0 of tv_drawn from the draw to its resolution one item later; the static
+  // rounds never touch that register, so they never wait for it.
+  int tv_drawn = 0;
+  auto issue_ticket = [&](int r) {
+    // (behind a uniform address the compiler would read the result back on the spot to share
+    // it between lanes, and wait for every load in flight)
+    if (r * nwaves >= static_tickets && drawing && lane == 0)
+      tv_drawn = atomicAdd(&hdr[H_TICKET + opaque_zero], 1);
+  };
+  // ticket of round r; ntickets or more = none
+  auto resolve_ticket = [&](int r) -> int {
+    if (r * nwaves < static_tickets) return r * nwaves + ((r & 1) ? nwaves - 1 - my_wave : my_wave);
+    if (!drawing) return ntickets;
+    const int drawn = __builtin_amdgcn_readfirstlane(tv_drawn);
+    if (drawn == dynamic_draws - 1 && lane == 0) hdr[H_TICKET] = 0;  // nobody draws after this one
+    const int t = static_tickets + drawn;
+    if (t >= ntickets) drawing = false;
+    return t;
+  };
+
+  // The opaque zero in the record address keeps the compiler from moving the record's
+  // fields into scalar registers right behind the load: that move would wait for every
+  // load in flight.
+  // Item record of a ticket (clamped, so a ticket past the end reads a valid record).
+  auto load_record = [&](int t, int4& r0, int4& r1, int& kvh) {
+    const int tc = min(t, ntickets - 1);
+    const int it = tc / Hkv;
+    kvh = tc - it * Hkv;
+    const int4* rec =
+        reinterpret_cast<const int4*>(meta + p.off_items + (int64_t)(first + it) * kItemInts + opaque_zero);
+    r0 = rec[0];  // rep, blk_start, tok_len, member_off
+    r1 = rec[1];  // member_cnt, ord, node, -
+  };
+  // Per-lane data that hangs off a record: one block id of the chunk per lane (a chunk has
+  // at most 64 blocks) and the member sequence of this lane's query row.
+  auto load_lane_meta = [&](const int4& r0, const int4& r1, int& my_blk, int& seq) {
+    const int nblk = (r0.z + kBlock - 1) / kBlock;
+    my_blk = p.block_table[(int64_t)r0.x * p.bt_stride + r0.y + min(lane, nblk - 1)];
+    seq = meta[p.off_members + r0.w + (row_member < r1.x ? row_member : 0)];
+  };
+  auto load_q = [&](bf16x8 (&q)[KS], int seq, int mcnt, int kvh) {
+    const bool live = row_member < mcnt;
+    const __bf16* qp = reinterpret_cast<const __bf16*>(p.q) + (int64_t)seq * p.q_seq_stride +
+                       (int64_t)(kvh * G + row_head) * p.q_head_stride;
+#pragma unroll
+    for (int i = 0; i < KS; ++i) {
+      // channel offset of MFMA step i for this lane half: the K tile hands a lane 16 bytes
+      // of one token, i.e. 8 channels (bf16) or 16 channels = two steps (fp8)
+      const int dq = FP8 ? 32 * (i >> 1) + 16 * h + 8 * (i & 1) : 16 * i + 8 * h;
+      bf16x8 v = *reinterpret_cast<const bf16x8*>(qp + dq);
+      if (!live) v = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      q[i] = v;
+    }
+  };
+  // The fences keep the compiler from sinking the loads below the first instructions of
+  // the next tile's arithmetic, which start with a wait for that tile: a refill must be on
+  // its way before the wave blocks.
+  auto load_tile = [&](KT& kt, VT& vt, int my_blk, int nblk, int kvh, int ti) {
+    __builtin_amdgcn_sched_barrier(0);
+    const int p0 = 2 * ti, p1 = min(2 * ti + 1, nblk - 1);
+    const int b0 = __builtin_amdgcn_readlane(my_blk, p0);
+    const int b1 = __builtin_amdgcn_readlane(my_blk, p1);
+    const int kb = (m & 16) ? b1 : b0;
+    const char* kp = p.k_cache + (int64_t)kvh * p.kv_head_bytes + (int64_t)kb * p.kv_block_bytes + k_lane_off;
+#pragma unroll
+    for (int i = 0; i < KT::NK; ++i) kt.k[i] = load16<STREAM>(kp + i * 512);
+    const char* vbase = p.v_cache + (int64_t)kvh * p.kv_head_bytes + v_lane_off;
+    const char* vp0 = vbase + (int64_t)b0 * p.kv_block_bytes;
+    const char* vp1 = vbase + (int64_t)b1 * p.kv_block_bytes;
+#pragma unroll
+    for (int i = 0; i < VT::NV; ++i) {
+      vt.v[0][i] = load16<STREAM>(vp0 + i * V_STEP);
+      vt.v[1][i] = load16<STREAM>(vp1 + i * V_STEP);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // ---- set-up: the first three items of this wave; their tickets are static
+  int4 r0, r1, a0, a1, b0, b1;  // records of the current item and the two after it
+  int kvh, akvh, bkvh;
+  int my_blk, seq, a_blk, a_seq;  // per-lane data of the current and the next item
+  int ta = resolve_ticket(1);  // rounds 0 to 3 are static, or the whole list is
+  int tb = resolve_ticket(2);
+  load_record(my_wave, r0, r1, kvh);
+  load_record(ta, a0, a1, akvh);
+  load_record(tb, b0, b1, bkvh);
+  load_lane_meta(r0, r1, my_blk, seq);
+  load_lane_meta(a0, a1, a_blk, a_seq);
+  bf16x8 qreg[KS], nq[KS];
+  load_q(qreg, seq, r1.x, kvh);
+  KT kb0, kb1;
+  VT vb0, vb1;
+  {
+    const int len = __builtin_amdgcn_readfirstlane(r0.z);
+    const int nb = (len + kBlock - 1) / kBlock;
+    const int lt = (len + kTile - 1) / kTile - 1;
+    load_tile(kb0, vb0, my_blk, nb, kvh, 0);
+    load_tile(kb1, vb1, my_blk, nb, kvh, min(1, lt));
+  }
+
+#ifdef FCA_PROFILE
+  long long prof[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  long long t_prev = wall_clock64();
+  const long long t_begin = t_prev;
+#endif
+  for (int round = 0;; ++round) {
+    const int tok_len = __builtin_amdgcn_readfirstlane(r0.z);
+    const int mcnt = __builtin_amdgcn_readfirstlane(r1.x);
+    const int ord = __builtin_amdgcn_readfirstlane(r1.y);
+    const int nblk = (tok_len + kBlock - 1) / kBlock;
+    const int ntiles = (tok_len + kTile - 1) / kTile;
+    const int nfull = tok_len / kTile;  // tiles with all 32 tokens live; at most one ragged tile follows
+    const int last = ntiles - 1;
+    const int npairs = (ntiles + 1) >> 1;
+    // partial row this lane's query row is written to, -1 for a dead row
+    const int64_t prow = row_member < mcnt
+                             ? ((int64_t)seq * p.max_partials + ord) * p.num_q_heads + kvh * G + row_head
+                             : -1;
+    const int a_len = __builtin_amdgcn_readfirstlane(a0.z);
+    const int a_nblk = (a_len + kBlock - 1) / kBlock;
+    const int a_last = (a_len + kTile - 1) / kTile - 1;
+
+    f32x16 acc[NDB];
+    float mrow = -INFINITY, lrow = 0.f;  // reference maximum (scaled, log2 domain) and running sum
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
+    float sc = p.scale * kLog2e;
+    if (FP8 && p.k_scale) sc *= p.k_scale[kvh];
+
+    // One 32-token tile.  RAGGED is the variant for the single tile that may run past the
+    // end of the chunk: it masks scores and zeroes V there; full tiles carry no mask code.
+    auto compute_tile = [&](const KT& kt, const VT& vt, int ti, auto ragged) {
+      constexpr bool RAGGED = decltype(ragged)::value;
+      const int tok0 = ti * kTile;
+      f32x16 sr;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sr[r] = 0.f;
+#pragma unroll
+      for (int i = 0; i < KS; ++i) {
+        bf16x8 a;
+        if constexpr (FP8) {
+          const i32x4 w = kt.k[i >> 1];
+          a = (i & 1) ? fp8x8_to_bf16(w[2], w[3]) : fp8x8_to_bf16(w[0], w[1]);
+        } else {
+          a = __builtin_bit_cast(bf16x8, kt.k[i]);
+        }
+        sr = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[i], sr, 0, 0, 0);
+      }
+      // register r holds token 16 * (r / 8) + 8 * h + r % 8 of the tile
+      if constexpr (RAGGED) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (tok0 + 16 * (r >> 3) + 8 * h + (r & 7) >= tok_len) sr[r] = -INFINITY;
+      }
+      float mx = sr[0];
+#pragma unroll
+      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sr[r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      // sc > 0, so the maximum of the scaled scores is the scaled maximum.  mrow is the
+      // reference the exponentials are taken against, not the exact running maximum: it
+      // moves (and the accumulators are rescaled) only when a row's maximum rises more than
+      // kRescaleSlack above it, so probabilities stay below 2^kRescaleSlack and the rescale,
+      // which touches every accumulator register, is rare.  The log-sum-exp m + log2(l)
+      // does not depend on the reference.
+      // The first tile sets the reference without a rescale (the accumulators are zero).
+      const float mtile = mx * sc;
+      if (ti == 0) mrow = mtile;
+      if (__builtin_amdgcn_readfirstlane(__any(mtile > mrow + kRescaleSlack))) {
+        const float mnew = fmaxf(mrow, mtile);
+        const float alpha = fast_exp2(mrow - mnew);
+        lrow *= alpha;
+        mrow = mnew;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[db][r] *= alpha;
+      }
+      const float mref = mrow;
+      float sum = 0.f;
+      bf16x8 pb[2];  // probabilities of the tile as B operands
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float e = fast_exp2(__builtin_fmaf(sr[r], sc, -mref));
+        sum += e;
+        pb[r >> 3][r & 7] = (__bf16)e;
+      }
+      lrow += sum;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) {
+        // tokens this lane feeds for this block: 8h .. 8h+7; on the ragged tile zero the
+        // ones past the end so stale cache contents (possibly NaN) cannot leak through 0 * x
+        const int nv = tok_len - (tok0 + 16 * blk + 8 * h);
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+          bf16x8 a;
+          if constexpr (FP8) {
+            // rows of channel blocks 2 * pair and 2 * pair + 1 sit in the lower and upper
+            // lane halves; the swap hands every lane its tokens 8h..8h+7 of both blocks:
+            // dwords 0,1 become the operand of block 2 * pair, dwords 2,3 of 2 * pair + 1
+            const i32x4 raw = vt.v[blk][db >> 1];
+            const auto s0 = __builtin_amdgcn_permlane32_swap((unsigned)raw[0], (unsigned)raw[2], false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap((unsigned)raw[1], (unsigned)raw[3], false, false);
+            i32x2 w = {(int)s0[db & 1], (int)s1[db & 1]};
+            if constexpr (RAGGED) {
+#pragma unroll
+              for (int j = 0; j < 2; ++j) {
+                unsigned keep = 0;
+#pragma unroll
+                for (int b = 0; b < 4; ++b)
+                  if (4 * j + b < nv) keep |= 0xffu << (8 * b);
+                w[j] &= keep;
+              }
+            }
+            a = fp8x8_to_bf16(w[0], w[1]);
+          } else {
+            i32x4 w = vt.v[blk][db];
+            if constexpr (RAGGED) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                unsigned keep = (2 * j < nv ? 0xffffu : 0u) | (2 * j + 1 < nv ? 0xffff0000u : 0u);
+                w[j] &= keep;
+              }
+            }
+            a = __builtin_bit_cast(bf16x8, w);
+          }
+          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[blk], acc[db], 0, 0, 0);
+        }
+      }
+    };
+
+    // ---- all pairs of tiles but the last: both tiles full, refills from this item.
+    // Buffer 0 holds tile ti, buffer 1 tile ti + 1; a refill past the end (odd tile count)
+    // repeats the last tile so that the number of loads in flight never varies.
+    for (int pr = 0; pr < npairs - 1; ++pr) {
+      const int ti = 2 * pr;
+      compute_tile(kb0, vb0, ti, std::false_type{});
+      load_tile(kb0, vb0, my_blk, nblk, kvh, ti + 2);
+      compute_tile(kb1, vb1, ti + 1, std::false_type{});
+      load_tile(kb1, vb1, my_blk, nblk, kvh, min(ti + 3, last));
+    }
+
+    STAMP(0)
+    // ---- one step for each of the items ahead
+    int b_blk, b_seq;
+    load_lane_meta(b0, b1, b_blk, b_seq);
+    const int tc = resolve_ticket(round + 3);
+    int4 c0, c1;
+    int ckvh;
+    load_record(tc, c0, c1, ckvh);
+    issue_ticket(round + 4);
+    load_q(nq, a_seq, a1.x, akvh);
+
+    STAMP(1)
+    // ---- the last pair: refills come from the next item (of a ticket past the end: from
+    // the last record of the list, loads nobody uses)
+    const int ti = 2 * (npairs - 1);
+    if (ti < nfull)
+      compute_tile(kb0, vb0, ti, std::false_type{});
+    else
+      compute_tile(kb0, vb0, ti, std::true_type{});
+    STAMP(2)
+    load_tile(kb0, vb0, a_blk, a_nblk, akvh, 0);
+    if (ti + 1 < nfull)
+      compute_tile(kb1, vb1, ti + 1, std::false_type{});
+    else if (ti + 1 <= last)
+      compute_tile(kb1, vb1, ti + 1, std::true_type{});
+
+    STAMP(3)
+    // Write the partial (before the second refill: stores count as outstanding memory
+    // operations too, and behind the refill they would be waited for together with it).
+    // Every accumulator register of a lane belongs to the lane's own query row, so
+    // normalisation is per lane.  The rows then pass through a wave-private strip of LDS
+    // so that they leave as whole rows, two per store instruction: stored straight from
+    // the accumulator layout a row goes out in sixteen 32-byte pieces, and back-to-back
+    // partial writes to one cache line cost a wave several microseconds per item.
+    {
+      float vs = 1.f;
+      if (FP8 && p.v_scale) vs = p.v_scale[kvh];
+      const float l = lrow + __shfl_xor(lrow, 32);
+      const float inv = vs / l;
+      if (prow >= 0) {
+        if (h == 0) {
+          p.partial_lse[prow] = (mrow + fast_log2(l)) * kLn2;
+          *reinterpret_cast<int64_t*>(strip + m * kStripStride + D) = prow;
+        }
+        float* dst = strip + m * kStripStride + h * 4;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            f32x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = acc[db][q4 * 4 + e] * inv;
+            // accumulator register 4 * q4 + e holds channel 32 * db + 8 * q4 + 4 * h + e
+            *reinterpret_cast<f32x4*>(dst + db * 32 + q4 * 8) = v;
+          }
+      }
+      __builtin_amdgcn_wave_barrier();
+      // D = 128: lane (m, h) of store s carries channels 4m .. 4m+3 of row 2s + h
+      constexpr int LPR = D / 4;        // lanes per row
+      constexpr int RPS = 64 / LPR;     // rows per store
+      const int sub = lane / LPR, c = (lane % LPR) * 4;
+      const int rows = mcnt * G;
+      for (int r0s = 0; r0s < rows; r0s += RPS) {
+        const int r = r0s + sub;
+        if (r < rows) {
+          const float* src = strip + r * kStripStride;
+          const int64_t pr = *reinterpret_cast<const int64_t*>(src + D);
+          store16<STREAM>(p.partial_out + pr * D + c, *reinterpret_cast<const f32x4*>(src + c));
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+    STAMP(4)
+    load_tile(kb1, vb1, a_blk, a_nblk, akvh, min(1, a_last));
+
+    // ---- move on
+#ifdef FCA_PROFILE
+    prof[7] += 1;
+#endif
+    if (ta >= ntickets) break;
+#pragma unroll
+    for (int i = 0; i < KS; ++i) qreg[i] = nq[i];
+    r0 = a0, r1 = a1, kvh = akvh, my_blk = a_blk, seq = a_seq;
+    a0 = b0, a1 = b1, akvh = bkvh, a_blk = b_blk, a_seq = b_seq;
+    b0 = c0, b1 = c1, bkvh = ckvh;
+    ta = tb;
+    tb = tc;
+    STAMP(5)
+  }
+#ifdef FCA_PROFILE
+  if (lane == 0 && g_prof32) {
+    long long* dst = g_prof32 + (long long)my_wave * 10;
+    for (int i = 0; i < 8; ++i) dst[i] = prof[i];
+    dst[8] = t_begin;
+    dst[9] = wall_clock64();
+  }
+#endif
+  // loads nobody uses are still in flight: let them land before the wave ends
+  __builtin_amdgcn_s_waitcnt(0);
+}
+
+hipError_t launch_attend32(const AttendParams& p, const fca_plan& plan, int kv_dtype, int grid, hipStream_t stream) {
+  const bool fp8 = kv_dtype == FCA_FP8_E4M3;
+  // With sharing on, a launch reads every KV block once: stream it past the caches.  With
+  // sharing off, sequences of a group read the same blocks again and again and the
+  // memory-side cache serves the repeats, so the loads stay ordinary.
+  const bool stream_kv = plan.max_levels > 0;
+#define FCA_LAUNCH(D_, F_, S_) \
+  hipLaunchKernelGGL((fca_attend32_kernel<D_, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, p)
+#define FCA_PICK(D_, F_) \
+  if (stream_kv) FCA_LAUNCH(D_, F_, true); else FCA_LAUNCH(D_, F_, false)
+  if (plan.head_dim == 128) {
+    if (fp8) { FCA_PICK(128, true); } else { FCA_PICK(128, false); }
+  } else {
+    if (fp8) { FCA_PICK(64, true); } else { FCA_PICK(64, false); }
+  }
+#undef FCA_PICK
+#undef FCA_LAUNCH
+  return hipGetLastError();
+}
+
+}  // namespace fca
+
+#ifdef FCA_PROFILE
+extern "C" int fca_debug_set_profile_buffer32(void* dev_ptr) {
+  long long* v = static_cast<long long*>(dev_ptr);
+  return (int)hipMemcpyToSymbol(HIP_SYMBOL(fca::g_prof32), &v, sizeof(v));
+}
+#endif

@@ -161,6 +161,7 @@ struct AppendParams {
 hipError_t launch_build(const BuildParams& p, hipStream_t stream);
 hipError_t launch_append(const AppendParams& p, int kv_dtype, hipStream_t stream);
 hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, hipStream_t stream);
+hipError_t launch_attend32(const AttendParams& p, const fca_plan& plan, int kv_dtype, int grid, hipStream_t stream);
 hipError_t launch_merge(const MergeParams& p, hipStream_t stream);
 hipError_t launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
 
