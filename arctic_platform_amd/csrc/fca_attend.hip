@@ -1,16 +1,16 @@
-// Forest cascade attention pass for gfx950: one persistent kernel serves both the
-// shared-prefix pass (query rows of every member sequence x the GQA heads of one KV head
-// stacked into a 32- or 64-row tile) and the per-sequence suffix pass (the same tile with
-// only Hq/Hkv live rows).
+// Forest cascade attention pass for gfx950: one persistent kernel per query-tile height
+// serves both the shared-prefix pass (query rows of every member sequence x the GQA heads
+// of one KV head stacked into a 32- or 64-row tile) and the per-sequence suffix pass (the
+// same tile with only Hq/Hkv live rows).  This file holds the 64-row kernel and the launch
+// dispatch; the 32-row kernel is in fca_attend32.hip.
 //
 // Work item = (node chunk, tile of members) x KV head.  Every wavefront is its own worker:
 // it walks its share of the size-ordered work list, streams each chunk's 32-token tiles
 // with private online-softmax state and writes one normalised partial per item.  There is
-// no workgroup barrier and no shared counter anywhere.  The kernel runs one wave per SIMD
-// with the whole 512-entry register file: registers, not LDS, are the staging buffer,
-// because the cache already stores tiles in MFMA operand order and a tile in flight needs
-// a place to land either way.  LDS only transposes the output tile so partial rows leave
-// as whole 128-byte lines.
+// no workgroup barrier.  The kernel runs one wave per SIMD with the whole 512-entry
+// register file: registers, not LDS, are the staging buffer for K and V, because the cache
+// already stores tiles in MFMA operand order and a tile in flight needs a place to land
+// either way.
 //
 // Per tile and wave, with tokens on the MFMA M dimension (the transposed product):
 //   St[32 tok x 32 rows] = K[32 x D] . Qt[D x 32]       D/16 x mfma_f32_32x32x16_bf16
@@ -18,10 +18,9 @@
 //   exchange with the lane 32 away (both hold the same query row)
 //   Ot[D x 32 rows]     += Vt[D x 32 tok] . Pt[32 x 32]  D/32 x 2 mfma
 // The cache stores K as [D/x][16 tok][x] and V as [D][16 tok], which are the A-operand
-// orders of these two products: every operand is one contiguous 16-byte (8-byte for fp8 V)
-// global load per lane.  The K rows are fed in the token order that makes the softmax
-// output registers line up with the B operand of the second product, so P never leaves
-// registers.
+// orders of these two products: every operand is one contiguous 16-byte global load per
+// lane.  The K rows are fed in the token order that makes the softmax output registers
+// line up with the B operand of the second product, so P never leaves registers.
 //
 // Semantics (softmax scale, GQA head mapping h -> h / (Hq/Hkv), no mask for the decode
 // token) follow arctic_platform/model/implementations/qwen35/models/qwen3_5_moe/
@@ -33,9 +32,6 @@
 
 namespace fca {
 
-#ifdef FCA_PROFILE
-__device__ long long* g_prof = nullptr;  // [waves][8] wall-clock ticks (100 MHz), debug builds only
-#endif
 
 // One persistent loop per wave that keeps loads in flight across work items.
 //
@@ -54,8 +50,8 @@ __device__ long long* g_prof = nullptr;  // [waves][8] wall-clock ticks (100 MHz
 // the next item's record, block ids and member sequences; the next item's query rows and
 // first tile are requested before the current item's partial is written out, so the
 // memory pipe does not drain at item boundaries.
-template <int D, int NRT, bool FP8>
-__global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendParams p) {
+template <int D, int NRT, bool FP8, bool STREAM>
+__global__ __launch_bounds__(kThreads, 1) void fca_attend64_kernel(AttendParams p) {
   constexpr int KS = D / 16;   // MFMA steps of the score product
   constexpr int NDB = D / 32;  // 32-channel blocks of the output
   using KT = KTile<D, FP8>;
@@ -86,6 +82,10 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
   // bf16: channel 32 * db + m, tokens 8h..8h+7; fp8: channel 32 * (2 * pair + h) + m, all 16 tokens
   const int v_lane_off = FP8 ? (h * 32 + m) * 16 : m * 32 + h * 16;
   constexpr int V_STEP = 1024;
+  // wave-private strip of LDS for the output rows: D values + the partial row index
+  constexpr int kStripStride = D + 4;  // floats; keeps rows 16-byte aligned
+  __shared__ float strips[kWaves][NRT * 32 * kStripStride];
+  float* strip = strips[wave];
 
   const int nwaves = (int)gridDim.x * kWaves;
   const int static_tickets = min(ntickets, max(1, ntickets / nwaves - 1) * nwaves);
@@ -134,16 +134,21 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
       }
     }
   };
+  // The fences keep the compiler from sinking the loads below the arithmetic that follows,
+  // which starts with a wait: a refill must be on its way before the wave blocks.
   auto load_k = [&](KT& kt, int my_blk, int nblk, int kvh, int ti) {
+    __builtin_amdgcn_sched_barrier(0);
     const int p0 = 2 * ti, p1 = min(2 * ti + 1, nblk - 1);
     const int b0 = __builtin_amdgcn_readlane(my_blk, p0);
     const int b1 = __builtin_amdgcn_readlane(my_blk, p1);
     const int kb = (m & 16) ? b1 : b0;
     const char* kp = p.k_cache + (int64_t)kvh * p.kv_head_bytes + (int64_t)kb * p.kv_block_bytes + k_lane_off;
 #pragma unroll
-    for (int i = 0; i < KT::NK; ++i) kt.k[i] = *reinterpret_cast<const i32x4*>(kp + i * 512);
+    for (int i = 0; i < KT::NK; ++i) kt.k[i] = load16<STREAM>(kp + i * 512);
+    __builtin_amdgcn_sched_barrier(0);
   };
   auto load_v = [&](VT& vt, int my_blk, int nblk, int kvh, int ti) {
+    __builtin_amdgcn_sched_barrier(0);
     const int p0 = 2 * ti, p1 = min(2 * ti + 1, nblk - 1);
     const int b0 = __builtin_amdgcn_readlane(my_blk, p0);
     const int b1 = __builtin_amdgcn_readlane(my_blk, p1);
@@ -152,9 +157,10 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
     const char* vp1 = vbase + (int64_t)b1 * p.kv_block_bytes;
 #pragma unroll
     for (int i = 0; i < VT::NV; ++i) {
-      vt.v[0][i] = *reinterpret_cast<const i32x4*>(vp0 + i * V_STEP);
-      vt.v[1][i] = *reinterpret_cast<const i32x4*>(vp1 + i * V_STEP);
+      vt.v[0][i] = load16<STREAM>(vp0 + i * V_STEP);
+      vt.v[1][i] = load16<STREAM>(vp1 + i * V_STEP);
     }
+    __builtin_amdgcn_sched_barrier(0);
   };
   auto load_tile = [&](KT& kt, VT& vt, int my_blk, int nblk, int kvh, int ti) {
     load_k(kt, my_blk, nblk, kvh, ti);
@@ -162,10 +168,6 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
   };
 
   // ---- first item of this wave: fetched with the waits exposed
-#ifdef FCA_PROFILE
-  const long long t_start = wall_clock64();
-  long long n_items = 0, n_tiles = 0, t_epi = 0;
-#endif
   int round = 0;
   if (my_wave < ntickets) {
     int4 r0, r1;
@@ -276,7 +278,9 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
           // than kRescaleSlack above it, so probabilities stay below 2^kRescaleSlack and the
           // rescale, which touches every accumulator register, is rare.  The log-sum-exp
           // m + log2(l) does not depend on the reference.
+          // The first tile sets the reference without a rescale (the accumulators are zero).
           const float mtile = mx * sc;
+          if (ti == 0) mrow[rt] = mtile;
           if (__builtin_amdgcn_readfirstlane(__any(mtile > mrow[rt] + kRescaleSlack))) {
             const float mnew = fmaxf(mrow[rt], mtile);
             const float alpha = fast_exp2(mrow[rt] - mnew);
@@ -413,16 +417,10 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
       }
 
       // Write the partial.  Every accumulator register of a lane belongs to the lane's own
-      // query row, so normalisation is per lane; a lane stores its 4-channel groups straight
-      // from the accumulator layout (two lanes cover 32 adjacent bytes, the 16 stores of a
-      // row tile cover whole rows).  L2 is write-back, so the pieces of a line written within
-      // a microsecond by one wave leave for HBM as full lines; a transpose through LDS was
-      // measured and only added latency.
-#ifdef FCA_PROFILE
-      const long long t_e0 = wall_clock64();
-      n_items += 1;
-      n_tiles += ntiles;
-#endif
+      // query row, so normalisation is per lane.  The rows then pass through a wave-private
+      // strip of LDS so that they leave as whole rows: stored straight from the accumulator
+      // layout a row goes out in sixteen 32-byte pieces, and partial writes of a cache line
+      // are slow.
       float vs = 1.f;
       if (FP8 && p.v_scale) vs = p.v_scale[kvh];
 #pragma unroll
@@ -431,8 +429,12 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
         const float l = lrow[rt] + __shfl_xor(lrow[rt], 32);
         const float inv = vs / l;
         if (prow[rt] >= 0) {
-          if (h == 0) p.partial_lse[prow[rt]] = (mrow[rt] + fast_log2(l)) * kLn2;
-          float* dst = p.partial_out + prow[rt] * D + h * 4;
+          const int row = rt * 32 + m;
+          if (h == 0) {
+            p.partial_lse[prow[rt]] = (mrow[rt] + fast_log2(l)) * kLn2;
+            *reinterpret_cast<int64_t*>(strip + row * kStripStride + D) = prow[rt];
+          }
+          float* dst = strip + row * kStripStride + h * 4;
 #pragma unroll
           for (int db = 0; db < NDB; ++db)
 #pragma unroll
@@ -445,9 +447,21 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
             }
         }
       }
-#ifdef FCA_PROFILE
-      t_epi += wall_clock64() - t_e0;
-#endif
+      __builtin_amdgcn_wave_barrier();
+      {
+        constexpr int LPR = D / 4;     // lanes per row
+        constexpr int RPS = 64 / LPR;  // rows per store
+        const int sub = lane / LPR, c = (lane % LPR) * 4;
+        for (int r0s = 0; r0s < rows; r0s += RPS) {
+          const int r = r0s + sub;
+          if (r < rows) {
+            const float* src = strip + r * kStripStride;
+            const int64_t pr = *reinterpret_cast<const int64_t*>(src + D);
+            store16<STREAM>(p.partial_out + pr * D + c, *reinterpret_cast<const f32x4*>(src + c));
+          }
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
       if (!more) break;
       r0 = n0;
       r1 = n1;
@@ -457,19 +471,6 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_stream_kernel(AttendPa
       for (int rt = 0; rt < NRT; ++rt) seq[rt] = nseq[rt];
     }
   }
-#ifdef FCA_PROFILE
-  if (lane == 0 && g_prof) {
-    long long* dst = g_prof + (long long)my_wave * 8;
-    dst[0] = 0;
-    dst[1] = 0;
-    dst[2] = t_epi;
-    dst[3] = 0;
-    dst[4] = n_items;
-    dst[5] = n_tiles;
-    dst[6] = wall_clock64() - t_start;
-    dst[7] = t_start;
-  }
-#endif
 }
 
 static int cached_cu_count() {
@@ -502,32 +503,24 @@ hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dty
   int grid = cached_cu_count() * wgs_per_cu;
   if ((int64_t)grid * kWaves > max_tickets) grid = (int)((max_tickets + kWaves - 1) / kWaves);
   if (grid < 1) grid = 1;
-  static const int use32 = env_int("FCA_ATTEND32", 1);
-  if (nrt == 1 && use32) return launch_attend32(p, plan, kv_dtype, grid, stream);
-#define FCA_LAUNCH(D_, N_, F_) \
-  hipLaunchKernelGGL((fca_attend_stream_kernel<D_, N_, F_>), dim3(grid), dim3(kThreads), 0, stream, p)
+  if (nrt == 1) return launch_attend32(p, plan, kv_dtype, grid, stream);
+  // With sharing on, a launch reads every KV block once: stream it past the caches.  With
+  // sharing off, sequences of a group read the same blocks again and again and the
+  // memory-side cache serves the repeats, so the loads stay ordinary.
+  const bool stream_kv = plan.max_levels > 0;
+#define FCA_LAUNCH(D_, F_, S_) \
+  hipLaunchKernelGGL((fca_attend64_kernel<D_, 2, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, p)
+#define FCA_PICK(D_, F_) \
+  if (stream_kv) FCA_LAUNCH(D_, F_, true); else FCA_LAUNCH(D_, F_, false)
   if (plan.head_dim == 128) {
-    if (nrt == 1) {
-      if (fp8) FCA_LAUNCH(128, 1, true); else FCA_LAUNCH(128, 1, false);
-    } else {
-      if (fp8) FCA_LAUNCH(128, 2, true); else FCA_LAUNCH(128, 2, false);
-    }
+    if (fp8) { FCA_PICK(128, true); } else { FCA_PICK(128, false); }
   } else {
-    if (nrt == 1) {
-      if (fp8) FCA_LAUNCH(64, 1, true); else FCA_LAUNCH(64, 1, false);
-    } else {
-      if (fp8) FCA_LAUNCH(64, 2, true); else FCA_LAUNCH(64, 2, false);
-    }
+    if (fp8) { FCA_PICK(64, true); } else { FCA_PICK(64, false); }
   }
+#undef FCA_PICK
 #undef FCA_LAUNCH
   return hipGetLastError();
 }
 
 }  // namespace fca
 
-#ifdef FCA_PROFILE
-extern "C" int fca_debug_set_profile_buffer(void* dev_ptr) {
-  long long* v = static_cast<long long*>(dev_ptr);
-  return (int)hipMemcpyToSymbol(HIP_SYMBOL(fca::g_prof), &v, sizeof(v));
-}
-#endif

@@ -21,12 +21,6 @@
 
 namespace fca {
 
-#ifdef FCA_PROFILE
-__device__ long long* g_prof32 = nullptr;
-#define STAMP(i) { const long long t_ = wall_clock64(); prof[i] += t_ - t_prev; t_prev = t_; }
-#else
-#define STAMP(i)
-#endif
 
 template <int D, bool FP8, bool STREAM>
 __global__ __launch_bounds__(kThreads, 1) void fca_attend32_kernel(AttendParams p) {
@@ -178,11 +172,6 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend32_kernel(AttendParams 
     load_tile(kb1, vb1, my_blk, nb, kvh, min(1, lt));
   }
 
-#ifdef FCA_PROFILE
-  long long prof[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  long long t_prev = wall_clock64();
-  const long long t_begin = t_prev;
-#endif
   for (int round = 0;; ++round) {
     const int tok_len = __builtin_amdgcn_readfirstlane(r0.z);
     const int mcnt = __builtin_amdgcn_readfirstlane(r1.x);
@@ -321,7 +310,6 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend32_kernel(AttendParams 
       load_tile(kb1, vb1, my_blk, nblk, kvh, min(ti + 3, last));
     }
 
-    STAMP(0)
     // ---- one step for each of the items ahead
     int b_blk, b_seq;
     load_lane_meta(b0, b1, b_blk, b_seq);
@@ -332,7 +320,6 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend32_kernel(AttendParams 
     issue_ticket(round + 4);
     load_q(nq, a_seq, a1.x, akvh);
 
-    STAMP(1)
     // ---- the last pair: refills come from the next item (of a ticket past the end: from
     // the last record of the list, loads nobody uses)
     const int ti = 2 * (npairs - 1);
@@ -340,14 +327,12 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend32_kernel(AttendParams 
       compute_tile(kb0, vb0, ti, std::false_type{});
     else
       compute_tile(kb0, vb0, ti, std::true_type{});
-    STAMP(2)
     load_tile(kb0, vb0, a_blk, a_nblk, akvh, 0);
     if (ti + 1 < nfull)
       compute_tile(kb1, vb1, ti + 1, std::false_type{});
     else if (ti + 1 <= last)
       compute_tile(kb1, vb1, ti + 1, std::true_type{});
 
-    STAMP(3)
     // Write the partial (before the second refill: stores count as outstanding memory
     // operations too, and behind the refill they would be waited for together with it).
     // Every accumulator register of a lane belongs to the lane's own query row, so
@@ -393,13 +378,9 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend32_kernel(AttendParams 
       }
       __builtin_amdgcn_wave_barrier();
     }
-    STAMP(4)
     load_tile(kb1, vb1, a_blk, a_nblk, akvh, min(1, a_last));
 
     // ---- move on
-#ifdef FCA_PROFILE
-    prof[7] += 1;
-#endif
     if (ta >= ntickets) break;
 #pragma unroll
     for (int i = 0; i < KS; ++i) qreg[i] = nq[i];
@@ -408,16 +389,7 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend32_kernel(AttendParams 
     b0 = c0, b1 = c1, bkvh = ckvh;
     ta = tb;
     tb = tc;
-    STAMP(5)
   }
-#ifdef FCA_PROFILE
-  if (lane == 0 && g_prof32) {
-    long long* dst = g_prof32 + (long long)my_wave * 10;
-    for (int i = 0; i < 8; ++i) dst[i] = prof[i];
-    dst[8] = t_begin;
-    dst[9] = wall_clock64();
-  }
-#endif
   // loads nobody uses are still in flight: let them land before the wave ends
   __builtin_amdgcn_s_waitcnt(0);
 }
@@ -444,9 +416,3 @@ hipError_t launch_attend32(const AttendParams& p, const fca_plan& plan, int kv_d
 
 }  // namespace fca
 
-#ifdef FCA_PROFILE
-extern "C" int fca_debug_set_profile_buffer32(void* dev_ptr) {
-  long long* v = static_cast<long long*>(dev_ptr);
-  return (int)hipMemcpyToSymbol(HIP_SYMBOL(fca::g_prof32), &v, sizeof(v));
-}
-#endif
