@@ -153,3 +153,37 @@ def test_empty_sequence_in_batch(gpu):
     assert (out[1] == 0).all() and torch.isinf(lse[1]).all() and (lse[1] < 0).all()
     ref_out, ref_lse = oracle_for(w)
     assert_matches_oracle(out, lse, ref_out, ref_lse, seqs=[0, 2], what="batch with an empty row")
+
+
+@pytest.mark.parametrize("rows,dtype", [(32, torch.bfloat16), (64, torch.bfloat16), (32, torch.float8_e4m3fn)])
+def test_many_small_items_drawn_from_the_counter(gpu, rows, dtype):
+    """More work items than five per wavefront of the device, all tiny: the tail of the work
+    list is then drawn from the counter in the metadata header, one- and two-tile items
+    follow each other without a gap, and the counter must be back at zero after every
+    launch so that the same metadata serves the next one."""
+    from arctic_platform_amd.forest import build_forest_metadata
+    from arctic_platform_amd.ops import forest_cascade_decode
+    from arctic_platform_amd.workloads import three_level_forest
+
+    gen = torch.Generator().manual_seed(21)
+    # 840 sequences in 168 small groups under one root: ~1000 items x 8 KV heads
+    seg_len, paths = three_level_forest(gen, 20, 168, 5, (1, 70), (1, 45))
+    w = make_forest_workload("small-items", seg_len, paths, gen, num_q_heads=32, num_kv_heads=8, head_dim=128,
+                             kv_dtype=dtype, device=gpu)
+    kw = dict(num_q_heads=32, num_kv_heads=8, head_dim=128, chunk_tokens=32, rows_per_item=rows)
+    md = build_forest_metadata(w.block_table, w.seq_lens, **kw)
+    torch.cuda.synchronize()
+    tickets = md.header()["items"] * 8
+    waves = 4 * torch.cuda.get_device_properties(gpu).multi_processor_count
+    assert tickets > 5 * waves, f"the case is meant to exceed five items per wave ({tickets} tickets, {waves} waves)"
+    ref_out, ref_lse = oracle_for(w)
+    first = None
+    for launch in range(3):
+        out, lse = forest_cascade_decode(w.q, w.kv_cache, md, w.scale, w.k_scale, w.v_scale)
+        torch.cuda.synchronize()
+        assert int(md.meta[md.layout.header + 3]) == 0, f"ticket counter not back at zero after launch {launch}"
+        assert_matches_oracle(out, lse, ref_out, ref_lse, what=f"small items, launch {launch}")
+        if first is None:
+            first = (out.clone(), lse.clone())
+        else:
+            assert torch.equal(out, first[0]) and torch.equal(lse, first[1]), "launches on one metadata differ"
