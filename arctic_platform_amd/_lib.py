@@ -23,6 +23,7 @@ EXPORTS = (
     "fca_workspace_bytes",
     "fca_meta_describe",
     "fca_build_metadata",
+    "fca_update_metadata",
     "fca_prefix_pass",
     "fca_suffix_pass",
     "fca_forest_pass",
@@ -128,6 +129,7 @@ def load_library() -> ctypes.CDLL:
     lib.fca_workspace_bytes.argtypes = [P(FcaPlan), SZ, SZ, SZ]
     lib.fca_meta_describe.argtypes = [P(FcaPlan), P(FcaMetaLayout)]
     lib.fca_build_metadata.argtypes = [P(FcaPlan), VP, I64, VP, VP, VP]
+    lib.fca_update_metadata.argtypes = [P(FcaPlan), VP, I64, VP, VP, VP]
     attend = [P(FcaPlan), P(FcaTensors), VP, VP, VP, VP]
     lib.fca_prefix_pass.argtypes = attend
     lib.fca_suffix_pass.argtypes = attend

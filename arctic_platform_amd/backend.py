@@ -51,11 +51,11 @@ class ForestCascadeMetadata:
 
 def parse_forest_cascade_configs(value) -> dict:
     """``forest_cascade_attn_configs`` arrives as a JSON string (``"{}"`` in the recipes)
-    or a dict.  Known keys: chunk_tokens, rows_per_item, max_levels, enable."""
+    or a dict.  Known keys: chunk_tokens, rows_per_item, max_levels, enable, rebuild_every."""
     if value is None or value == "":
         return {}
     cfg = json.loads(value) if isinstance(value, str) else dict(value)
-    unknown = set(cfg) - {"chunk_tokens", "rows_per_item", "max_levels", "enable"}
+    unknown = set(cfg) - {"chunk_tokens", "rows_per_item", "max_levels", "enable", "rebuild_every"}
     if unknown:
         raise ValueError(f"unknown forest_cascade_attn_configs keys: {sorted(unknown)}")
     return cfg
@@ -90,8 +90,12 @@ class ForestCascadeAttentionBackend:
 
 
 class ForestCascadeMetadataBuilder:
-    """Builds the forest once per scheduler step.  Workspaces are kept per batch shape
-    (num_reqs, max_blocks), so a steady decode loop allocates nothing."""
+    """Makes the forest metadata once per scheduler step.  Workspaces are kept per batch
+    shape (num_reqs, max_blocks), so a steady decode loop allocates nothing.  A step on a
+    shape seen before asks for an update: the device keeps the forest of the last build when
+    the rows still carry it (sequences only grew) and builds anew otherwise.  Every
+    ``rebuild_every``-th step is a full build regardless, so sharing that appeared since
+    (a new request with a cached prompt) is picked up."""
 
     def __init__(self, num_q_heads, num_kv_heads, head_dim, device="cuda", forest_cascade_attn_configs=None):
         cfg = parse_forest_cascade_configs(forest_cascade_attn_configs)
@@ -103,11 +107,13 @@ class ForestCascadeMetadataBuilder:
         self.enabled = bool(cfg.get("enable", True))
         self.chunk_tokens = int(cfg.get("chunk_tokens", 1024))
         self.max_levels = int(cfg.get("max_levels", 4))
+        self.rebuild_every = max(1, int(cfg.get("rebuild_every", 32)))
         group = num_q_heads // num_kv_heads
         self.rows_per_item = int(cfg.get("rows_per_item", 64 if group > 32 else 32))
         if group > self.rows_per_item:
             raise ValueError(f"{group} query heads per KV head do not fit rows_per_item={self.rows_per_item}")
         self._workspaces: dict = {}
+        self._steps_since_build: dict = {}
 
     def build(self, common_prefix_len: int, common_attn_metadata: CommonAttentionMetadata) -> ForestCascadeMetadata:
         m = common_attn_metadata
@@ -118,6 +124,9 @@ class ForestCascadeMetadataBuilder:
             )
         bt, sl = m.block_table_tensor[: m.num_reqs], m.seq_lens[: m.num_reqs]
         key = (m.num_reqs, bt.shape[1])
+        since = self._steps_since_build.get(key, self.rebuild_every)
+        update = key in self._workspaces and since + 1 < self.rebuild_every
+        self._steps_since_build[key] = since + 1 if update else 0
         forest = build_forest_metadata(
             bt,
             sl,
@@ -130,6 +139,7 @@ class ForestCascadeMetadataBuilder:
             cascade=self.enabled,
             max_levels=self.max_levels,
             out=self._workspaces.get(key),
+            update=update,
         )
         self._workspaces[key] = forest
         return ForestCascadeMetadata(forest=forest, slot_mapping=m.slot_mapping[: m.num_reqs], num_decode_tokens=m.num_reqs)

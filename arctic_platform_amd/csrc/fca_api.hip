@@ -172,8 +172,8 @@ int fca_meta_describe(const fca_plan* plan, fca_meta_layout* out) {
   return FCA_OK;
 }
 
-int fca_build_metadata(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,
-                       const int32_t* seq_lens_dev, void* meta_dev, void* stream) {
+static int run_build(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,
+                     const int32_t* seq_lens_dev, void* meta_dev, int try_update, void* stream) {
   if (int rc = check_plan(plan)) return rc;
   if (!block_table_dev || !seq_lens_dev || !meta_dev)
     return fail(FCA_ERR_INVALID_ARG, "block_table, seq_lens and metadata workspace must be non-NULL");
@@ -189,8 +189,19 @@ int fca_build_metadata(const fca_plan* plan, const int32_t* block_table_dev, int
   b.seq_lens = seq_lens_dev;
   b.meta = static_cast<int32_t*>(meta_dev);
   b.L = fca::make_layout(*plan);
+  b.try_update = try_update;
   hipError_t e = fca::launch_build(b, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? FCA_OK : hip_fail(e, "metadata builder launch");
+}
+
+int fca_build_metadata(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,
+                       const int32_t* seq_lens_dev, void* meta_dev, void* stream) {
+  return run_build(plan, block_table_dev, block_table_stride, seq_lens_dev, meta_dev, 0, stream);
+}
+
+int fca_update_metadata(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,
+                        const int32_t* seq_lens_dev, void* meta_dev, void* stream) {
+  return run_build(plan, block_table_dev, block_table_stride, seq_lens_dev, meta_dev, 1, stream);
 }
 
 int fca_prefix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev, float* partial_out_dev,

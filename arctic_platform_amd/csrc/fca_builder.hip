@@ -9,6 +9,14 @@
 // them; sequences left alone become private leaves.  Grouping semantics (compare with
 // the group's first member, members ascending) follow the trainer's host-side discovery,
 // arctic_platform/rl/zorro_train/zorro_train.py:242-285.
+//
+// Between two scheduler steps of a decode loop only the lengths change: every sequence
+// grows by a token and now and then takes a new private block.  The forest is a function
+// of the shared blocks alone, so an update keeps it as long as every row still carries
+// the blocks its shared nodes were built from (a 64-bit fingerprint per row, taken at
+// build time, is compared) and those blocks are still full blocks of the row; only the
+// leaves and the work list are made again.  Any mismatch falls back to the full build in
+// the same launch, so an update is always safe to ask for.
 #include "fca_common.h"
 
 namespace fca {
@@ -50,8 +58,60 @@ __device__ inline unsigned hash_key(unsigned long long k) {
   return (unsigned)k;
 }
 
+__device__ inline unsigned long long mix64(unsigned long long k) {
+  k ^= k >> 33;
+  k *= 0xff51afd7ed558ccdull;
+  k ^= k >> 33;
+  k *= 0xc4ceb9fe1a85ec53ull;
+  k ^= k >> 33;
+  return k;
+}
+
+// Fingerprint of the first n block ids of a row, computed by a group of 16 lanes (every
+// lane returns it): the sum over positions j of (id_j ^ c) * w_j in 64 bits, with an odd
+// 32-bit weight per position.  A change of one id moves the sum by a non-zero multiple of
+// an odd number, an exchange of two ids by a product of two non-zero numbers below 2^32:
+// neither can be zero modulo 2^64.  One multiply-add per element, eight loads in
+// flight per lane.
+__device__ inline unsigned long long row_fingerprint(const int32_t* row, int n, int glane) {
+  unsigned long long acc = 0;
+  constexpr int kUnroll = 8;  // 128 positions per round trip of the group
+  auto term = [](int id, unsigned j) {
+    return (unsigned long long)((unsigned)id ^ 0xa5a5a5a5u) * ((j * 0x9e3779b1u) | 1u);
+  };
+  int j0 = 0;
+  for (; j0 + 16 * kUnroll <= n; j0 += 16 * kUnroll) {
+    int v[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) v[u] = row[j0 + u * 16 + glane];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) acc += term(v[u], (unsigned)(j0 + u * 16 + glane));
+  }
+  if (j0 < n) {  // the rest in one round trip: loads past the end are clamped and not counted
+    int v[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) v[u] = row[min(j0 + u * 16 + glane, n - 1)];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int j = j0 + u * 16 + glane;
+      if (j < n) acc += term(v[u], (unsigned)j);
+    }
+  }
+  for (int off = 8; off; off >>= 1) acc += __shfl_xor(acc, off, 16);
+  return acc;
+}
+
+__device__ inline int plan_fingerprint(const fca_plan& pl) {
+  unsigned long long k = mix64(((unsigned long long)(unsigned)pl.num_seqs << 32) | (unsigned)pl.max_blocks);
+  k = mix64(k ^ (((unsigned long long)(unsigned)pl.num_q_heads << 32) | (unsigned)pl.num_kv_heads));
+  k = mix64(k ^ (((unsigned long long)(unsigned)pl.chunk_tokens << 32) | (unsigned)pl.rows_per_item));
+  k = mix64(k ^ (unsigned)pl.max_levels);
+  return (int)(k & 0x7fffffff);
+}
+
 __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p) {
   __shared__ int lds_scan[kBuildThreads];
+  __shared__ int lds_mismatch;
   __shared__ int lds_hist[2 * kSizeBuckets];
   __shared__ int lds_cursor[2 * kSizeBuckets];
   __shared__ unsigned long long lds_tokens;
@@ -80,148 +140,206 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   int* hmin = meta + L.hash_min;
   const int hsize = (int)L.hash_size;
   int* members = meta + L.members;
+  unsigned long long* sig = reinterpret_cast<unsigned long long*>(meta + L.s_sig);
+  const int plan_sig = plan_fingerprint(p.plan);
 
-  if (tid < kHeaderInts) hdr[tid] = 0;
-  if (tid == 0) lds_tokens = 0;
-  for (int s = tid; s < S; s += kBuildThreads) {
-    int len = p.seq_lens[s];
-    if (len < 0 || len > p.plan.max_blocks * kBlock) {
-      atomicOr(&hdr[H_ERROR], 1);
-      len = max(0, min(len, p.plan.max_blocks * kBlock));
+  // ---- update: is the forest of the last build on this workspace still the forest of
+  // these rows?  (pos = first private block of a row, ord = chunks of its shared nodes:
+  // both are left in the workspace by the build.)
+  bool reuse = false;
+  if (p.try_update) {
+    if (tid == 0) lds_mismatch = (hdr[H_BUILT] != kBuiltMagic || hdr[H_PLAN_SIG] != plan_sig) ? 1 : 0;
+    __syncthreads();
+    if (!lds_mismatch) {
+      const int gid = tid >> 4, glane = tid & 15;
+      for (int s = gid; s < S; s += kBuildThreads / 16) {
+        const int len = p.seq_lens[s];
+        const int shared_blocks = pos[s];
+        bool ok = len >= 0 && len <= p.plan.max_blocks * kBlock && len / kBlock >= shared_blocks;
+        if (ok) ok = row_fingerprint(p.block_table + s * p.bt_stride, shared_blocks, glane) == sig[s];
+        if (!ok && glane == 0) lds_mismatch = 1;
+      }
     }
-    tmp1[s] = len;  // validated length, kept for the leaf pass
-    nfull[s] = p.plan.max_levels > 0 ? len / kBlock : 0;
-    pos[s] = 0;
-    par[s] = -1;
-    ord[s] = 0;
+    __syncthreads();
+    reuse = !lds_mismatch;
   }
-  __syncthreads();
 
   int node_base = 0, member_base = 0, levels = 0;
-  for (int level = 0; level < p.plan.max_levels; ++level) {
-    for (int i = tid; i < hsize; i += kBuildThreads) {
-      hkeys[i] = kEmptyKey;
-      hmin[i] = 0x7fffffff;
-    }
-    for (int s = tid; s < S; s += kBuildThreads) {
-      run[s] = 0x7fffffff;
-      cnt[s] = 0;
-      leader[s] = -1;
-      slot[s] = -1;
-    }
+  if (reuse) {
+    node_base = hdr[H_NODES];
+    member_base = hdr[H_LEAF_MEMBERS];
+    levels = hdr[H_LEVELS];
+    const int updates = hdr[H_UPDATES];
+    const unsigned long long shared_tokens =
+        (unsigned long long)(unsigned)hdr[H_SHARED_TOK_LO] | ((unsigned long long)(unsigned)hdr[H_SHARED_TOK_HI] << 32);
     __syncthreads();
-    // Key every sequence that still has a full block at its position.  A sequence whose
-    // parent is -2 dropped out of sharing at an earlier level.
+    if (tid == 0) {
+      lds_tokens = shared_tokens;
+      hdr[H_ERROR] = 0;
+      hdr[H_TICKET] = 0;
+      hdr[H_UPDATES] = updates + 1;
+    }
+    for (int s = tid; s < S; s += kBuildThreads) tmp1[s] = p.seq_lens[s];
+    __syncthreads();
+  } else {
+    if (tid < kHeaderInts) hdr[tid] = 0;
+    if (tid == 0) lds_tokens = 0;
     for (int s = tid; s < S; s += kBuildThreads) {
-      if (par[s] == -2 || pos[s] >= nfull[s]) continue;
-      unsigned blk = (unsigned)p.block_table[s * p.bt_stride + pos[s]];
-      unsigned long long key = ((unsigned long long)(unsigned)(par[s] + 1) << 32) | blk;
-      int h = hash_key(key) & (hsize - 1);
-      for (int probe = 0; probe < hsize; ++probe) {
-        unsigned long long prev = atomicCAS(&hkeys[h], kEmptyKey, key);
-        if (prev == kEmptyKey || prev == key) break;
-        h = (h + 1) & (hsize - 1);
+      int len = p.seq_lens[s];
+      if (len < 0 || len > p.plan.max_blocks * kBlock) {
+        atomicOr(&hdr[H_ERROR], 1);
+        len = max(0, min(len, p.plan.max_blocks * kBlock));
       }
-      slot[s] = h;
-      atomicMin(&hmin[h], s);
+      tmp1[s] = len;  // validated length, kept for the leaf pass
+      nfull[s] = p.plan.max_levels > 0 ? len / kBlock : 0;
+      pos[s] = 0;
+      par[s] = -1;
+      ord[s] = 0;
     }
     __syncthreads();
-    for (int s = tid; s < S; s += kBuildThreads) {
-      if (slot[s] >= 0) {
-        leader[s] = hmin[slot[s]];
-        lcp[s] = nfull[s] - pos[s];
+
+    for (int level = 0; level < p.plan.max_levels; ++level) {
+      for (int i = tid; i < hsize; i += kBuildThreads) {
+        hkeys[i] = kEmptyKey;
+        hmin[i] = 0x7fffffff;
       }
+      for (int s = tid; s < S; s += kBuildThreads) {
+        run[s] = 0x7fffffff;
+        cnt[s] = 0;
+        leader[s] = -1;
+        slot[s] = -1;
+      }
+      __syncthreads();
+      // Key every sequence that still has a full block at its position.  A sequence whose
+      // parent is -2 dropped out of sharing at an earlier level.
+      for (int s = tid; s < S; s += kBuildThreads) {
+        if (par[s] == -2 || pos[s] >= nfull[s]) continue;
+        unsigned blk = (unsigned)p.block_table[s * p.bt_stride + pos[s]];
+        unsigned long long key = ((unsigned long long)(unsigned)(par[s] + 1) << 32) | blk;
+        int h = hash_key(key) & (hsize - 1);
+        for (int probe = 0; probe < hsize; ++probe) {
+          unsigned long long prev = atomicCAS(&hkeys[h], kEmptyKey, key);
+          if (prev == kEmptyKey || prev == key) break;
+          h = (h + 1) & (hsize - 1);
+        }
+        slot[s] = h;
+        atomicMin(&hmin[h], s);
+      }
+      __syncthreads();
+      for (int s = tid; s < S; s += kBuildThreads) {
+        if (slot[s] >= 0) {
+          leader[s] = hmin[slot[s]];
+          lcp[s] = nfull[s] - pos[s];
+        }
+      }
+      __syncthreads();
+      // Common run with the leader = first position where the two rows differ.  Every group
+      // of 16 lanes takes its own sequence (64 sequences in flight per pass) and scans 256
+      // positions per round, 16 independent loads per lane and row.
+      {
+        const int gid = tid >> 4, glane = tid & 15;
+        constexpr int kGroups = kBuildThreads / 16, kPerLane = 16;
+        for (int s = gid; s < S; s += kGroups) {
+          const int t = leader[s];
+          if (t < 0 || t == s) continue;
+          const int lim = min(nfull[s], nfull[t]) - pos[s];
+          const int32_t* row_s = p.block_table + s * p.bt_stride + pos[s];
+          const int32_t* row_t = p.block_table + t * p.bt_stride + pos[s];
+          int first = lim;
+          for (int j0 = 0; j0 < lim && first == lim; j0 += 16 * kPerLane) {
+            int mine = lim;
+#pragma unroll
+            for (int u = kPerLane - 1; u >= 0; --u) {
+              const int j = j0 + u * 16 + glane;
+              if (j < lim && row_s[j] != row_t[j]) mine = j;
+            }
+            for (int off = 8; off; off >>= 1) mine = min(mine, __shfl_xor(mine, off, 16));
+            first = mine;
+          }
+          if (glane == 0) lcp[s] = min(lcp[s], first);
+        }
+      }
+      __syncthreads();
+      for (int s = tid; s < S; s += kBuildThreads) {
+        if (leader[s] >= 0) {
+          atomicMin(&run[leader[s]], lcp[s]);
+          atomicAdd(&cnt[leader[s]], 1);
+        }
+      }
+      __syncthreads();
+      for (int s = tid; s < S; s += kBuildThreads) {
+        const bool is_node = leader[s] == s && cnt[s] >= 2;
+        tmp0[s] = is_node ? 1 : 0;
+        nodeof[s] = is_node ? cnt[s] : 0;
+      }
+      __syncthreads();
+      const int new_nodes = block_exclusive_scan(tmp0, tmp0, S, lds_scan);
+      if (new_nodes == 0) break;
+      const int new_members = block_exclusive_scan(nodeof, nodeof, S, lds_scan);
+      ++levels;
+      for (int s = tid; s < S; s += kBuildThreads) {
+        if (leader[s] == s && cnt[s] >= 2) {
+          const int id = node_base + tmp0[s];
+          meta[L.node_rep + id] = s;
+          meta[L.node_blk + id] = pos[s];
+          meta[L.node_nblk + id] = run[s];
+          meta[L.node_level + id] = level;
+          meta[L.node_moff + id] = member_base + nodeof[s];
+          meta[L.node_mcnt + id] = cnt[s];
+          meta[L.node_ord + id] = ord[s];
+          tmp0[s] = id;
+          atomicAdd(&lds_tokens, (unsigned long long)run[s] * kBlock);
+        }
+      }
+      __syncthreads();
+      // Member lists in ascending sequence order: rank = members of the same leader below s.
+      // One thread per sequence scans [leader, s); the members of a group are usually
+      // adjacent rows, so the scan is a handful of steps.
+      for (int s = tid; s < S; s += kBuildThreads) {
+        const int t = leader[s];
+        if (t < 0 || cnt[t] < 2) continue;
+        int below = 0;
+        for (int j = t; j < s; ++j) below += leader[j] == t ? 1 : 0;
+        members[meta[L.node_moff + tmp0[t]] + below] = s;
+      }
+      __syncthreads();
+      for (int s = tid; s < S; s += kBuildThreads) {
+        const int t = leader[s];
+        if (t >= 0 && cnt[t] >= 2) {
+          lcp[s] = run[t];  // advance amount, applied after the barrier (pos[t] is read by others)
+          par[s] = tmp0[t];
+        } else {
+          lcp[s] = 0;
+          par[s] = -2;
+        }
+      }
+      __syncthreads();
+      for (int s = tid; s < S; s += kBuildThreads) {
+        pos[s] += lcp[s];
+        ord[s] += num_chunks_for(lcp[s] * kBlock, chunk);
+      }
+      node_base += new_nodes;
+      member_base += new_members;
+      __syncthreads();
     }
-    __syncthreads();
-    // Common run with the leader = first position where the two rows differ.  Every group
-    // of 16 lanes takes its own sequence (64 sequences in flight per pass) and scans 256
-    // positions per round, 16 independent loads per lane and row.
+    // What a later update starts from: fingerprints of the shared part of every row and
+    // the totals of the shared nodes.
     {
       const int gid = tid >> 4, glane = tid & 15;
-      constexpr int kGroups = kBuildThreads / 16, kPerLane = 16;
-      for (int s = gid; s < S; s += kGroups) {
-        const int t = leader[s];
-        if (t < 0 || t == s) continue;
-        const int lim = min(nfull[s], nfull[t]) - pos[s];
-        const int32_t* row_s = p.block_table + s * p.bt_stride + pos[s];
-        const int32_t* row_t = p.block_table + t * p.bt_stride + pos[s];
-        int first = lim;
-        for (int j0 = 0; j0 < lim && first == lim; j0 += 16 * kPerLane) {
-          int mine = lim;
-#pragma unroll
-          for (int u = kPerLane - 1; u >= 0; --u) {
-            const int j = j0 + u * 16 + glane;
-            if (j < lim && row_s[j] != row_t[j]) mine = j;
-          }
-          for (int off = 8; off; off >>= 1) mine = min(mine, __shfl_xor(mine, off, 16));
-          first = mine;
-        }
-        if (glane == 0) lcp[s] = min(lcp[s], first);
+      for (int s = gid; s < S; s += kBuildThreads / 16) {
+        const unsigned long long f = row_fingerprint(p.block_table + s * p.bt_stride, pos[s], glane);
+        if (glane == 0) sig[s] = f;
+      }
+      if (tid == 0) {
+        hdr[H_LEAF_MEMBERS] = member_base;
+        hdr[H_SHARED_TOK_LO] = (int)(lds_tokens & 0xffffffffull);
+        hdr[H_SHARED_TOK_HI] = (int)(lds_tokens >> 32);
+        hdr[H_PLAN_SIG] = plan_sig;
+        hdr[H_BUILT] = kBuiltMagic;
       }
     }
-    __syncthreads();
-    for (int s = tid; s < S; s += kBuildThreads) {
-      if (leader[s] >= 0) {
-        atomicMin(&run[leader[s]], lcp[s]);
-        atomicAdd(&cnt[leader[s]], 1);
-      }
-    }
-    __syncthreads();
-    for (int s = tid; s < S; s += kBuildThreads) {
-      const bool is_node = leader[s] == s && cnt[s] >= 2;
-      tmp0[s] = is_node ? 1 : 0;
-      nodeof[s] = is_node ? cnt[s] : 0;
-    }
-    __syncthreads();
-    const int new_nodes = block_exclusive_scan(tmp0, tmp0, S, lds_scan);
-    if (new_nodes == 0) break;
-    const int new_members = block_exclusive_scan(nodeof, nodeof, S, lds_scan);
-    ++levels;
-    for (int s = tid; s < S; s += kBuildThreads) {
-      if (leader[s] == s && cnt[s] >= 2) {
-        const int id = node_base + tmp0[s];
-        meta[L.node_rep + id] = s;
-        meta[L.node_blk + id] = pos[s];
-        meta[L.node_nblk + id] = run[s];
-        meta[L.node_level + id] = level;
-        meta[L.node_moff + id] = member_base + nodeof[s];
-        meta[L.node_mcnt + id] = cnt[s];
-        meta[L.node_ord + id] = ord[s];
-        tmp0[s] = id;
-        atomicAdd(&lds_tokens, (unsigned long long)run[s] * kBlock);
-      }
-    }
-    __syncthreads();
-    // Member lists in ascending sequence order: rank = members of the same leader below s.
-    // One thread per sequence scans [leader, s); the members of a group are usually
-    // adjacent rows, so the scan is a handful of steps.
-    for (int s = tid; s < S; s += kBuildThreads) {
-      const int t = leader[s];
-      if (t < 0 || cnt[t] < 2) continue;
-      int below = 0;
-      for (int j = t; j < s; ++j) below += leader[j] == t ? 1 : 0;
-      members[meta[L.node_moff + tmp0[t]] + below] = s;
-    }
-    __syncthreads();
-    for (int s = tid; s < S; s += kBuildThreads) {
-      const int t = leader[s];
-      if (t >= 0 && cnt[t] >= 2) {
-        lcp[s] = run[t];  // advance amount, applied after the barrier (pos[t] is read by others)
-        par[s] = tmp0[t];
-      } else {
-        lcp[s] = 0;
-        par[s] = -2;
-      }
-    }
-    __syncthreads();
-    for (int s = tid; s < S; s += kBuildThreads) {
-      pos[s] += lcp[s];
-      ord[s] += num_chunks_for(lcp[s] * kBlock, chunk);
-    }
-    node_base += new_nodes;
-    member_base += new_members;
-    __syncthreads();
-  }
+  }  // full build
+  __syncthreads();
 
   // Private leaves and per-sequence partial counts.  Node index space for the work list:
   // shared nodes [0, node_base), then leaf of sequence s at node_base + s.

@@ -25,8 +25,16 @@ enum HeaderSlot {
   H_ERROR = 5,
   H_TOKENS_LO = 6,
   H_TOKENS_HI = 7,
-  H_LEVELS = 8
+  H_LEVELS = 8,
+  // state a later update of the same workspace starts from
+  H_LEAF_MEMBERS = 10,   // offset of the leaf entries in the member list
+  H_SHARED_TOK_LO = 11,  // KV tokens held by shared nodes
+  H_SHARED_TOK_HI = 12,
+  H_BUILT = 13,          // kBuiltMagic once a build has completed on this workspace
+  H_UPDATES = 14,        // length-only updates since the last full build
+  H_PLAN_SIG = 15        // fingerprint of the plan the workspace was built for
 };
+constexpr int kBuiltMagic = 0x46434131;
 
 // Offsets in int32 units from the start of the metadata workspace.
 struct MetaLayout {
@@ -37,6 +45,7 @@ struct MetaLayout {
   int64_t items;
   // builder scratch
   int64_t s_pos, s_par, s_ord, s_nfull, s_leader, s_lcp, s_run, s_cnt, s_node, s_slot, s_tmp0, s_tmp1, s_nitems;
+  int64_t s_sig;  // 64-bit fingerprint of each row's shared blocks, 2 int32 each
   int64_t hash_keys;  // 64-bit keys, 2 int32 each
   int64_t hash_min;
   int64_t hash_size;  // entries (power of two)
@@ -83,6 +92,7 @@ inline __host__ MetaLayout make_layout(const fca_plan& p) {
   L.s_tmp0 = take(S);
   L.s_tmp1 = take(S);
   L.s_nitems = take(2 * S);
+  L.s_sig = take(2 * S);
   int64_t hs = 64;
   while (hs < 4 * S) hs <<= 1;
   L.hash_size = hs;
@@ -113,6 +123,7 @@ struct BuildParams {
   const int32_t* seq_lens;
   int32_t* meta;
   MetaLayout L;
+  int32_t try_update;  // keep the forest of the last build if the rows still carry it
 };
 
 struct AttendParams {

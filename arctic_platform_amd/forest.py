@@ -47,6 +47,7 @@ class ForestMetadata:
             error=h[5],
             unique_tokens=(h[6] & 0xFFFFFFFF) | (h[7] << 32),
             levels=h[8],
+            updates=h[14],
         )
 
     def check(self) -> None:
@@ -129,12 +130,16 @@ def build_forest_metadata(
     cascade: bool = True,
     max_levels: int = 4,
     out: ForestMetadata | None = None,
+    update: bool = False,
 ) -> ForestMetadata:
     """Discover the shared-prefix forest of a decode batch on the device.
 
     ``cascade=False`` turns sharing off: every sequence becomes one private node over its
     whole block-table row, which makes the same kernels a plain paged decode attention.
     Pass a previous result as ``out`` to rebuild into the same workspaces (no allocation).
+    With ``update=True`` and such an ``out``, the forest found by the last build is kept if
+    the rows still carry it (``fca_update_metadata``: the next step of a decode loop, where
+    sequences only grew); any other change is detected on the device and built anew.
     """
     if block_size != BLOCK_SIZE:
         raise ValueError(f"block_size must be {BLOCK_SIZE}")
@@ -155,7 +160,8 @@ def build_forest_metadata(
         rows_per_item=rows_per_item,
         max_levels=max_levels if cascade else 0,
     )
-    if out is not None and bytes(out.plan) == bytes(plan):
+    same_workspace = out is not None and bytes(out.plan) == bytes(plan)
+    if same_workspace:
         md = dataclasses.replace(out, block_table=block_table, seq_lens=seq_lens)
     else:
         layout = _lib.FcaMetaLayout()
@@ -167,15 +173,16 @@ def build_forest_metadata(
         md = ForestMetadata(
             plan=plan,
             layout=layout,
-            meta=torch.empty(nm.value // 4, dtype=torch.int32, device=dev),
+            meta=torch.zeros(nm.value // 4, dtype=torch.int32, device=dev),
             partial_out=torch.empty(slots, num_q_heads, head_dim, dtype=torch.float32, device=dev),
             partial_lse=torch.empty(slots, num_q_heads, dtype=torch.float32, device=dev),
             block_table=block_table,
             seq_lens=seq_lens,
         )
         assert md.partial_out.numel() * 4 == no.value and md.partial_lse.numel() * 4 == nl.value
+    entry = lib.fca_update_metadata if update and same_workspace else lib.fca_build_metadata
     _lib.check(
-        lib.fca_build_metadata(
+        entry(
             ctypes.byref(md.plan),
             block_table.data_ptr(),
             block_table.stride(0),

@@ -166,6 +166,7 @@ def main():
         return median(ts)
 
     build_us = ev_time(build)
+    update_us = ev_time(lambda: build_forest_metadata(w.block_table, w.seq_lens, out=md, update=True, **kw))
     merge_us = ev_time(lambda: ops.merge_partials(md, w.q, out=out, return_lse=False))
 
     result = {
@@ -200,6 +201,7 @@ def main():
             "merge_kernel": round(merge_us, 2),
             "metadata_builder": round(build_us, 2),
             "builder_per_step": round(build_us / args.layers, 2),
+            "metadata_update": round(update_us, 2),
         },
         "roofline": {
             "kernel": "fca_attend64_kernel" if rows > 32 else "fca_attend32_kernel",

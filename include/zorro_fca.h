@@ -88,7 +88,9 @@ typedef struct fca_tensors {
 typedef struct fca_meta_layout {
   int64_t header;        /* [16]: 0 items, 1 shared items, 2 nodes (shared), 3 work ticket
                             (self-resetting, owned by the attention kernel), 4 reserved,
-                            5 error flag, 6/7 unique tokens lo/hi, 8 levels found */
+                            5 error flag, 6/7 unique tokens lo/hi, 8 levels found,
+                            10-13 and 15 state for fca_update_metadata, 14 updates since the
+                            last full build */
   int64_t seq_npart;     /* [S] partial slots used per sequence */
   int64_t seq_leaf_blk;  /* [S] first block position of the private leaf */
   int64_t node_rep;      /* [S] shared nodes: representative sequence */
@@ -118,6 +120,19 @@ int fca_meta_describe(const fca_plan* plan, fca_meta_layout* layout);
  * (arctic_platform/rl/zorro_train/zorro_train.py:242-285, seqlen_balancing.py:437-486). */
 int fca_build_metadata(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,
                        const int32_t* seq_lens_dev, void* meta_dev, void* stream);
+
+/* The same for the next scheduler step of a running decode loop, into a workspace that a
+ * build (or an earlier update) has filled: sequences have grown and may have taken new
+ * private blocks.  The forest is kept if every row still starts with the blocks its shared
+ * nodes were built from (compared through a per-row fingerprint) and those are still full
+ * blocks of the row; then only the private leaves and the work list are made again, at a
+ * fraction of the cost.  Otherwise, or on a workspace never built or built for another
+ * plan, this is fca_build_metadata.  Either way the result is valid for the given rows; a
+ * kept forest may miss sharing that only a new build would find.  Header slot 14 counts
+ * the updates since the last full build.  This replaces the per-step rebuild of the host-side
+ * group discovery (arctic_platform/rl/zorro_train/zorro_train.py:242-285 runs once per batch). */
+int fca_update_metadata(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,
+                        const int32_t* seq_lens_dev, void* meta_dev, void* stream);
 
 /* Shared-prefix pass: work items of shared nodes only.  Writes normalised fp32 partial
  * outputs and natural-log LSEs into the slots the metadata assigns. */

@@ -93,3 +93,4 @@ def test_decode_loop_through_backend(gpu, index):
         lse = torch.zeros(w.num_seqs, hq, device=gpu)  # forward() returns no lse; compare outputs only
         assert_matches_oracle(out.view(w.num_seqs, hq, d), ref_lse.float(), ref_out, ref_lse, what=f"C{index} step {step}")
         assert meta.forest.header()["shared_nodes"] == 8
+        assert meta.forest.header()["updates"] == step, "steps after the first are length-only updates"
