@@ -33,25 +33,29 @@
 namespace fca {
 
 
-// One persistent loop per wave that keeps loads in flight across work items.
+// The 64-row kernel: one persistent loop per wave that keeps loads in flight across work
+// items.  Two 32-row tiles of accumulators and query registers leave room for one K/V
+// tile buffer, refilled in halves, and for a one-item lookahead (the four-item lookahead
+// of the 32-row kernel spills here).
 //
 // Dealing the work.  Most tickets are dealt statically, back and forth over the
 // size-ordered list: in round r wave w of W takes ticket r * W + w (r even) or
 // r * W + W - 1 - w (r odd), which evens out the descending sizes between waves at no
 // cost.  A shared counter for everything would be expensive: device-wide atomics on one
 // address serialise at roughly 20 ns each across the eight L2s, so 1024 waves asking at
-// once wait tens of microseconds.  But waves do not run at the same speed (odd XCDs
-// stream several percent slower than even ones on identical work), so the last full
-// round and the remainder, the smallest items, come from a counter: each wave draws one
-// item ahead, which hides the atomic's latency, and draws until the list is empty.  The
-// draw that returns the last possible value re-arms the counter for the next launch.
+// once wait tens of microseconds.  But waves do not run at the same speed (XCDs stream
+// several percent apart on identical work), so the last full round and the remainder,
+// the smallest items, come from a counter: each wave draws one item ahead, which hides
+// the atomic's latency, and draws until the list is empty.  The draw that returns the
+// last possible value re-arms the counter for the next launch.
 //
 // Hiding item boundaries.  While the tiles of the current item stream, the wave fetches
 // the next item's record, block ids and member sequences; the next item's query rows and
 // first tile are requested before the current item's partial is written out, so the
 // memory pipe does not drain at item boundaries.
-template <int D, int NRT, bool FP8, bool STREAM>
+template <int D, bool FP8, bool STREAM>
 __global__ __launch_bounds__(kThreads, 1) void fca_attend64_kernel(AttendParams p) {
+  constexpr int NRT = 2;       // row tiles of 32 query rows
   constexpr int KS = D / 16;   // MFMA steps of the score product
   constexpr int NDB = D / 32;  // 32-channel blocks of the output
   using KT = KTile<D, FP8>;
@@ -175,17 +179,11 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend64_kernel(AttendParams 
     load_record(my_wave, r0, r1, kvh);
     load_lane_meta(r0, r1, my_blk, seq);
     load_q(seq, r1.x, kvh);
-    // Tile buffers of the rotation.  All indices into kb/vb are compile-time constants
-    // after unrolling, so the buffers live in registers.  32-row tiles: two buffers;
-    // 64-row tiles: one buffer refilled in halves.
-    constexpr int NBUF = NRT > 1 ? 1 : 2;
-    KT kb[NBUF];
-    VT vb[NBUF];
+    // The tile buffer, refilled in halves.
+    KT kb;
+    VT vb;
     auto request_first_tiles = [&](int blk_ids, int len, int head) {
-      const int nb = (len + kBlock - 1) / kBlock;
-      const int lt = (len + kTile - 1) / kTile - 1;
-#pragma unroll
-      for (int j = 0; j < NBUF; ++j) load_tile(kb[j], vb[j], blk_ids, nb, head, min(j, lt));
+      load_tile(kb, vb, blk_ids, (len + kBlock - 1) / kBlock, head, 0);
     };
     request_first_tiles(my_blk, __builtin_amdgcn_readfirstlane(r0.z), kvh);
 
@@ -194,7 +192,7 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend64_kernel(AttendParams 
       const int mcnt = __builtin_amdgcn_readfirstlane(r1.x);
       const int ord = __builtin_amdgcn_readfirstlane(r1.y);
       const int rows = mcnt * G;
-      const bool two_tiles = NRT > 1 && rows > 32;
+      const bool two_tiles = rows > 32;
       const int nblk = (tok_len + kBlock - 1) / kBlock;
       const int ntiles = (tok_len + kTile - 1) / kTile;
       const int nfull = tok_len / kTile;  // tiles with all 32 tokens live; at most one ragged tile follows
@@ -344,10 +342,7 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend64_kernel(AttendParams 
               a = __builtin_bit_cast(bf16x8, w);
             }
             acc[0][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[0][blk], acc[0][db], 0, 0, 0);
-            if constexpr (NRT > 1) {
-              if (two_tiles)
-                acc[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[1][blk], acc[1][db], 0, 0, 0);
-            }
+            if (two_tiles) acc[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[1][blk], acc[1][db], 0, 0, 0);
           }
         }
       };
@@ -364,45 +359,19 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend64_kernel(AttendParams 
       // from the record fetched one trip earlier, then the record is (re)read from the
       // ticket; both are idempotent, so no branch is needed.
       int ti = 0, trips = 0;
-      if constexpr (NRT == 1) {
-        // all NBUF buffers are already requested (tiles 0 .. NBUF-1, clamped); a buffer is
-        // refilled NBUF tiles ahead as soon as it has been consumed
-        for (; ti + NBUF - 1 < nfull; ti += NBUF, ++trips) {
-#pragma unroll
-          for (int j = 0; j < NBUF; ++j) {
-            compute_tile(kb[j], vb[j], ti + j, std::false_type{});
-            load_tile(kb[j], vb[j], my_blk, nblk, kvh, min(ti + NBUF + j, last));
-          }
-          if (trips >= 1) {  // the first trip leaves a drawn ticket time to arrive
-            load_lane_meta(n0, n1, nmy_blk, nseq);
-            load_record(__builtin_amdgcn_readfirstlane(t_next_v), n0, n1, nkvh);
-          }
+      // the next K as soon as the scores have issued, the next V as soon as the value
+      // product has
+      for (; ti < nfull; ++ti, ++trips) {
+        scores_softmax(kb, ti, std::false_type{});
+        load_k(kb, my_blk, nblk, kvh, min(ti + 1, last));
+        weighted_values(vb, ti, std::false_type{});
+        load_v(vb, my_blk, nblk, kvh, min(ti + 1, last));
+        if (trips >= 1) {  // the first trip leaves a drawn ticket time to arrive
+          load_lane_meta(n0, n1, nmy_blk, nseq);
+          load_record(__builtin_amdgcn_readfirstlane(t_next_v), n0, n1, nkvh);
         }
-        // buffer j holds tile ti + j (clamped); fewer than NBUF full tiles remain, and
-        // possibly the ragged one
-#pragma unroll
-        for (int j = 0; j < NBUF; ++j) {
-          if (ti + j < nfull)
-            compute_tile(kb[j], vb[j], ti + j, std::false_type{});
-          else if (ti + j < ntiles)
-            compute_tile(kb[j], vb[j], ti + j, std::true_type{});
-        }
-      } else {
-        // 64 query rows leave no room for a second tile buffer: one buffer, refilled in
-        // halves -- the next K as soon as the scores have issued, the next V as soon as the
-        // value product has
-        for (; ti < nfull; ++ti, ++trips) {
-          scores_softmax(kb[0], ti, std::false_type{});
-          load_k(kb[0], my_blk, nblk, kvh, min(ti + 1, last));
-          weighted_values(vb[0], ti, std::false_type{});
-          load_v(vb[0], my_blk, nblk, kvh, min(ti + 1, last));
-          if (trips >= 1) {
-            load_lane_meta(n0, n1, nmy_blk, nseq);
-            load_record(__builtin_amdgcn_readfirstlane(t_next_v), n0, n1, nkvh);
-          }
-        }
-        if (ti < ntiles) compute_tile(kb[0], vb[0], ti, std::true_type{});
       }
+      if (ti < ntiles) compute_tile(kb, vb, ti, std::true_type{});
 
       // finish the chain for items too short to have done it on the way
       const int t_next = __builtin_amdgcn_readfirstlane(t_next_v);
@@ -410,8 +379,8 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend64_kernel(AttendParams 
       if (trips < 3) load_lane_meta(n0, n1, nmy_blk, nseq);
       const bool more = t_next < ntickets;
       if (more) {
-        // q registers and both tile buffers are dead now: request the next item's query
-        // rows and first tile before writing this item's partial
+        // q registers and the tile buffer are dead now: request the next item's query rows
+        // and first tile before writing this item's partial
         load_q(nseq, n1.x, nkvh);
         request_first_tiles(nmy_blk, __builtin_amdgcn_readfirstlane(n0.z), nkvh);
       }
@@ -486,21 +455,14 @@ static int cached_cu_count() {
   return cus;
 }
 
-static int env_int(const char* name, int fallback) {
-  const char* v = getenv(name);
-  return v && *v ? atoi(v) : fallback;
-}
-
 hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, hipStream_t stream) {
   const bool fp8 = kv_dtype == FCA_FP8_E4M3;
   const int nrt = plan.rows_per_item / 32;
-  // one workgroup of four independent waves per CU (the kernel uses the whole register
-  // file; two waves per SIMD were measured for the fp8 kernel, which would fit, and lost)
-  static const int wgs_per_cu = env_int("FCA_WGS_PER_CU", 1);
+  // one workgroup of four independent waves per CU: the kernels use the whole register file
   const int64_t max_tickets = (int64_t)plan.num_seqs *
                               ((int64_t)plan.max_blocks * kBlock / plan.chunk_tokens + plan.max_levels + 1) *
                               plan.num_kv_heads;
-  int grid = cached_cu_count() * wgs_per_cu;
+  int grid = cached_cu_count();
   if ((int64_t)grid * kWaves > max_tickets) grid = (int)((max_tickets + kWaves - 1) / kWaves);
   if (grid < 1) grid = 1;
   if (nrt == 1) return launch_attend32(p, plan, kv_dtype, grid, stream);
@@ -509,7 +471,7 @@ hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dty
   // memory-side cache serves the repeats, so the loads stay ordinary.
   const bool stream_kv = plan.max_levels > 0;
 #define FCA_LAUNCH(D_, F_, S_) \
-  hipLaunchKernelGGL((fca_attend64_kernel<D_, 2, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, p)
+  hipLaunchKernelGGL((fca_attend64_kernel<D_, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, p)
 #define FCA_PICK(D_, F_) \
   if (stream_kv) FCA_LAUNCH(D_, F_, true); else FCA_LAUNCH(D_, F_, false)
   if (plan.head_dim == 128) {
