@@ -69,7 +69,7 @@ int check_tensors(const fca_plan* p, const fca_tensors* t) {
   return FCA_OK;
 }
 
-fca::AttendParams attend_params(const fca_plan* p, const fca_tensors* t, void* meta, float* po, float* pl, int select) {
+fca::AttendParams attend_params(const fca_plan* p, const fca_tensors* t, void* meta, void* po, float* pl, int select) {
   const fca::MetaLayout L = fca::make_layout(*p);
   const int esz = t->kv_dtype == FCA_FP8_E4M3 ? 1 : 2;
   fca::AttendParams a{};
@@ -99,7 +99,7 @@ fca::AttendParams attend_params(const fca_plan* p, const fca_tensors* t, void* m
   return a;
 }
 
-int run_attend(const fca_plan* p, const fca_tensors* t, void* meta, float* po, float* pl, int select, void* stream) {
+int run_attend(const fca_plan* p, const fca_tensors* t, void* meta, void* po, float* pl, int select, void* stream) {
   if (int rc = check_plan(p)) return rc;
   if (int rc = check_tensors(p, t)) return rc;
   if (!meta || !po || !pl) return fail(FCA_ERR_INVALID_ARG, "metadata and partial workspaces must be non-NULL");
@@ -108,7 +108,7 @@ int run_attend(const fca_plan* p, const fca_tensors* t, void* meta, float* po, f
   return e == hipSuccess ? FCA_OK : hip_fail(e, "attention pass launch");
 }
 
-int run_merge(const fca_plan* p, const void* meta, const float* po, const float* pl, void* out, int64_t oss, int64_t ohs,
+int run_merge(const fca_plan* p, const void* meta, const void* po, const float* pl, void* out, int64_t oss, int64_t ohs,
               int32_t out_dtype, float* lse, void* stream) {
   if (int rc = check_plan(p)) return rc;
   if (!meta || !po || !pl || !out) return fail(FCA_ERR_INVALID_ARG, "metadata, partials and out must be non-NULL");
@@ -145,8 +145,8 @@ int fca_workspace_bytes(const fca_plan* plan, size_t* meta_bytes, size_t* partia
   const fca::MetaLayout L = fca::make_layout(*plan);
   const size_t slots = (size_t)plan->num_seqs * (size_t)L.max_partials;
   if (meta_bytes) *meta_bytes = (size_t)L.total * sizeof(int32_t);
-  if (partial_out_bytes) *partial_out_bytes = slots * plan->num_q_heads * plan->head_dim * sizeof(float);
-  if (partial_lse_bytes) *partial_lse_bytes = slots * plan->num_q_heads * sizeof(float);
+  if (partial_out_bytes) *partial_out_bytes = slots * plan->num_q_heads * plan->head_dim * 2;  // half
+  if (partial_lse_bytes) *partial_lse_bytes = slots * plan->num_q_heads * 2 * sizeof(float);    // {lse, scale}
   return FCA_OK;
 }
 
@@ -204,29 +204,29 @@ int fca_update_metadata(const fca_plan* plan, const int32_t* block_table_dev, in
   return run_build(plan, block_table_dev, block_table_stride, seq_lens_dev, meta_dev, 1, stream);
 }
 
-int fca_prefix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev, float* partial_out_dev,
+int fca_prefix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev, void* partial_out_dev,
                     float* partial_lse_dev, void* stream) {
   return run_attend(plan, t, meta_dev, partial_out_dev, partial_lse_dev, 1, stream);
 }
 
-int fca_suffix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev, float* partial_out_dev,
+int fca_suffix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev, void* partial_out_dev,
                     float* partial_lse_dev, void* stream) {
   return run_attend(plan, t, meta_dev, partial_out_dev, partial_lse_dev, 2, stream);
 }
 
-int fca_forest_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev, float* partial_out_dev,
+int fca_forest_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev, void* partial_out_dev,
                     float* partial_lse_dev, void* stream) {
   return run_attend(plan, t, meta_dev, partial_out_dev, partial_lse_dev, 0, stream);
 }
 
-int fca_merge(const fca_plan* plan, const void* meta_dev, const float* partial_out_dev, const float* partial_lse_dev,
+int fca_merge(const fca_plan* plan, const void* meta_dev, const void* partial_out_dev, const float* partial_lse_dev,
               void* out_dev, int64_t out_seq_stride, int64_t out_head_stride, int32_t out_dtype, float* lse_dev,
               void* stream) {
   return run_merge(plan, meta_dev, partial_out_dev, partial_lse_dev, out_dev, out_seq_stride, out_head_stride, out_dtype,
                    lse_dev, stream);
 }
 
-int fca_decode_step(const fca_plan* plan, const fca_tensors* t, void* meta_dev, float* partial_out_dev,
+int fca_decode_step(const fca_plan* plan, const fca_tensors* t, void* meta_dev, void* partial_out_dev,
                     float* partial_lse_dev, void* out_dev, int64_t out_seq_stride, int64_t out_head_stride,
                     int32_t out_dtype, float* lse_dev, void* stream) {
   if (int rc = run_attend(plan, t, meta_dev, partial_out_dev, partial_lse_dev, 0, stream)) return rc;

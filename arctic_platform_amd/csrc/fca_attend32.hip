@@ -53,10 +53,9 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend32_kernel(AttendParams 
   // bf16: channel 32 * db + m, tokens 8h..8h+7; fp8: channel 32 * (2 * pair + h) + m, all 16 tokens
   const int v_lane_off = FP8 ? (h * 32 + m) * 16 : m * 32 + h * 16;
   constexpr int V_STEP = 1024;
-  // wave-private strip of LDS for the output rows: D values + the partial row index
-  constexpr int kStripStride = D + 4;  // floats; keeps rows 16-byte aligned
-  __shared__ float strips[kWaves][32 * kStripStride];
-  float* strip = strips[wave];
+  // wave-private strip of LDS for the output rows
+  __shared__ __attribute__((aligned(16))) char strips[kWaves][32 * strip_row_bytes<D>()];
+  char* strip = strips[wave];
 
   // Dealing the work.  Round r gives wave w of W ticket r * W + w (r even) or
   // r * W + W - 1 - w (r odd) over the size-ordered list, for all rounds but the last full
@@ -337,45 +336,16 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend32_kernel(AttendParams 
     // operations too, and behind the refill they would be waited for together with it).
     // Every accumulator register of a lane belongs to the lane's own query row, so
     // normalisation is per lane.  The rows then pass through a wave-private strip of LDS
-    // so that they leave as whole rows, two per store instruction: stored straight from
-    // the accumulator layout a row goes out in sixteen 32-byte pieces, and back-to-back
-    // partial writes to one cache line cost a wave several microseconds per item.
+    // so that they leave as whole rows: stored straight from the accumulator layout a row
+    // goes out in sixteen pieces, and back-to-back partial writes to one cache line cost a
+    // wave several microseconds per item.
     {
       float vs = 1.f;
       if (FP8 && p.v_scale) vs = p.v_scale[kvh];
       const float l = lrow + __shfl_xor(lrow, 32);
-      const float inv = vs / l;
-      if (prow >= 0) {
-        if (h == 0) {
-          p.partial_lse[prow] = (mrow + fast_log2(l)) * kLn2;
-          *reinterpret_cast<int64_t*>(strip + m * kStripStride + D) = prow;
-        }
-        float* dst = strip + m * kStripStride + h * 4;
-#pragma unroll
-        for (int db = 0; db < NDB; ++db)
-#pragma unroll
-          for (int q4 = 0; q4 < 4; ++q4) {
-            f32x4 v;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = acc[db][q4 * 4 + e] * inv;
-            // accumulator register 4 * q4 + e holds channel 32 * db + 8 * q4 + 4 * h + e
-            *reinterpret_cast<f32x4*>(dst + db * 32 + q4 * 8) = v;
-          }
-      }
+      stage_partial_row<D>(strip, m, h, acc, vs / l, prow, (mrow + fast_log2(l)) * kLn2, p.partial_lse);
       __builtin_amdgcn_wave_barrier();
-      // D = 128: lane (m, h) of store s carries channels 4m .. 4m+3 of row 2s + h
-      constexpr int LPR = D / 4;        // lanes per row
-      constexpr int RPS = 64 / LPR;     // rows per store
-      const int sub = lane / LPR, c = (lane % LPR) * 4;
-      const int rows = mcnt * G;
-      for (int r0s = 0; r0s < rows; r0s += RPS) {
-        const int r = r0s + sub;
-        if (r < rows) {
-          const float* src = strip + r * kStripStride;
-          const int64_t pr = *reinterpret_cast<const int64_t*>(src + D);
-          store16<STREAM>(p.partial_out + pr * D + c, *reinterpret_cast<const f32x4*>(src + c));
-        }
-      }
+      store_partial_rows<D, STREAM>(strip, mcnt * G, lane, p.partial_out);
       __builtin_amdgcn_wave_barrier();
     }
     load_tile(kb1, vb1, a_blk, a_nblk, akvh, min(1, a_last));

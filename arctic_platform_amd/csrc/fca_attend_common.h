@@ -47,10 +47,80 @@ __device__ inline i32x4 load16(const char* ptr) {
   return *q;
 }
 template <bool STREAM>
-__device__ inline void store16(float* ptr, f32x4 v) {
-  f32x4* q = reinterpret_cast<f32x4*>(ptr);
+__device__ inline void store16(void* ptr, i32x4 v) {
+  i32x4* q = reinterpret_cast<i32x4*>(ptr);
   if constexpr (STREAM) __builtin_nontemporal_store(v, q);
   else *q = v;
+}
+
+// ---- partial rows ------------------------------------------------------------------
+// A partial output row is kept as D half-precision values times one power-of-two scale
+// per row (the smallest power of two not below the row's largest magnitude), next to its
+// fp32 log-sum-exp: {lse, scale} per row.  Every element keeps 11 significant bits
+// whatever the magnitude of the row, eight times finer than the bf16 rounding of the
+// probabilities inside the value product, at half the bytes of fp32 rows -- and writing
+// the partials costs several times their share of a launch's bytes.
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+
+// Bytes of one row in a wave's LDS strip: D halves + 16 bytes holding the row's index in
+// the partial buffers.
+template <int D>
+constexpr int strip_row_bytes() { return D * 2 + 16; }
+
+// Smallest power of two >= x for a positive, finite, normal x; 1 for anything else.
+__device__ inline float pow2_ceil(float x) {
+  const unsigned b = __float_as_uint(x);
+  const unsigned e = (b + 0x007fffffu) & 0x7f800000u;
+  return (x > 0.f && e != 0u && e != 0x7f800000u) ? __uint_as_float(e) : 1.f;
+}
+
+// Lane (m, h) holds, in acc[db][4 * q4 + e], channel 32 * db + 8 * q4 + 4 * h + e of query
+// row `row` of the tile.  Normalises the row by `inv` (1 / softmax sum, times the V scale
+// of an fp8 cache), stages it in the strip as scaled halves and, from the lanes with
+// h == 0, writes {lse, scale} and leaves the destination row index in the strip.
+template <int D>
+__device__ inline void stage_partial_row(char* strip, int row, int h, const f32x16 (&acc)[D / 32], float inv,
+                                         int64_t prow, float lse, float* partial_lse) {
+  float amax = 0.f;
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) amax = fmaxf(amax, fabsf(acc[db][r]));
+  amax = fmaxf(amax, __shfl_xor(amax, 32)) * fabsf(inv);
+  const float scale = pow2_ceil(amax);
+  const float k = inv / scale;  // exact: the scale is a power of two
+  if (prow < 0) return;
+  char* dst = strip + row * strip_row_bytes<D>();
+  if (h == 0) {
+    *reinterpret_cast<f32x2*>(partial_lse + 2 * prow) = f32x2{lse, scale};
+    *reinterpret_cast<int64_t*>(dst + D * 2) = prow;
+  }
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      f16x4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = (_Float16)(acc[db][q4 * 4 + e] * k);
+      *reinterpret_cast<f16x4*>(dst + (db * 32 + q4 * 8 + h * 4) * 2) = v;
+    }
+}
+
+// The staged rows 0 .. rows-1 leave as whole rows, 16 bytes per lane, 64 * 8 / D rows per
+// store instruction.
+template <int D, bool STREAM>
+__device__ inline void store_partial_rows(const char* strip, int rows, int lane, void* partial_out) {
+  constexpr int LPR = D / 8;     // lanes per row
+  constexpr int RPS = 64 / LPR;  // rows per store
+  const int sub = lane / LPR, c = (lane % LPR) * 8;
+  for (int r0 = 0; r0 < rows; r0 += RPS) {
+    const int r = r0 + sub;
+    if (r < rows) {
+      const char* src = strip + r * strip_row_bytes<D>();
+      const int64_t pr = *reinterpret_cast<const int64_t*>(src + D * 2);
+      store16<STREAM>(static_cast<char*>(partial_out) + (pr * D + c) * 2, *reinterpret_cast<const i32x4*>(src + c * 2));
+    }
+  }
 }
 
 // 8 fp8 e4m3 values (two dwords) -> 8 bf16 with the packed converter of gfx950 (scale 1:

@@ -139,8 +139,8 @@ struct AttendParams {
   float scale;
   int32_t* meta;
   int64_t off_header, off_items, off_members;
-  float* partial_out;
-  float* partial_lse;
+  void* partial_out;   // half [rows, Hq, D], each row times its scale
+  float* partial_lse;  // [rows, Hq, 2]: natural-log lse, scale of the row
   int32_t num_q_heads, num_kv_heads, group;  // group = Hq / Hkv
   int32_t max_partials;
   int32_t select;  // 0 all items, 1 shared only, 2 leaves only
@@ -148,7 +148,7 @@ struct AttendParams {
 
 struct MergeParams {
   const int32_t* seq_npart;
-  const float* partial_out;
+  const void* partial_out;
   const float* partial_lse;
   void* out;
   int64_t out_seq_stride, out_head_stride;

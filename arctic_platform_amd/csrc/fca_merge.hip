@@ -8,18 +8,24 @@
 namespace fca {
 
 constexpr int kMergeThreads = 256;
-constexpr int kLanesPerRow = 32;
 
-// 32 lanes per (sequence, query head) row; each lane owns D / 32 adjacent channels.
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+// D / 8 lanes per (sequence, query head) row; each lane owns 8 adjacent channels (16 bytes
+// of a half-precision partial row).  A partial row is its stored halves times the row's
+// scale; {lse, scale} sit side by side.
 template <int D>
 __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p) {
-  constexpr int V = D / kLanesPerRow;
+  constexpr int V = 8;
+  constexpr int kLanesPerRow = D / V;
   const int row = blockIdx.x * (kMergeThreads / kLanesPerRow) + threadIdx.x / kLanesPerRow;
   const int sub = threadIdx.x % kLanesPerRow;
   if (row >= p.num_seqs * p.num_q_heads) return;
   const int s = row / p.num_q_heads, hq = row - s * p.num_q_heads;
   const int np = p.seq_npart[s];
   const int64_t base = (int64_t)s * p.max_partials;
+  const _Float16* rows = static_cast<const _Float16*>(p.partial_out);
+  const float2* lse_scale = reinterpret_cast<const float2*>(p.partial_lse);
 
   // One online pass (running maximum, rescaled sum): the loads of successive partials do
   // not depend on each other, so unrolling keeps several of them in flight.
@@ -30,18 +36,17 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
 #pragma unroll 4
   for (int i = 0; i < np; ++i) {
     const int64_t pr = (base + i) * p.num_q_heads + hq;
-    const float l = p.partial_lse[pr];
-    float o[V];
-    const float* src = p.partial_out + pr * D + sub * V;
-#pragma unroll
-    for (int e = 0; e < V; ++e) o[e] = src[e];
+    const float2 ls = lse_scale[pr];
+    const f16x8 o = *reinterpret_cast<const f16x8*>(rows + pr * D + sub * V);
+    const float l = ls.x;
     if (!(l > -INFINITY)) continue;  // empty partial: weight 0, whatever its output holds
     const float m_new = fmaxf(m, l);
     const float keep = __expf(m - m_new);  // exp(-inf) = 0 on the first live partial
     const float w = __expf(l - m_new);
     wsum = wsum * keep + w;
+    const float ws = w * ls.y;
 #pragma unroll
-    for (int e = 0; e < V; ++e) acc[e] = acc[e] * keep + w * o[e];
+    for (int e = 0; e < V; ++e) acc[e] = acc[e] * keep + ws * (float)o[e];
     m = m_new;
   }
   const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
@@ -72,7 +77,7 @@ hipError_t launch_copy(const void* src, void* dst, size_t bytes, hipStream_t str
 
 hipError_t launch_merge(const MergeParams& p, hipStream_t stream) {
   const int rows = p.num_seqs * p.num_q_heads;
-  const int per_block = kMergeThreads / kLanesPerRow;
+  const int per_block = kMergeThreads / (p.head_dim / 8);
   const int grid = (rows + per_block - 1) / per_block;
   if (grid == 0) return hipSuccess;
   if (p.head_dim == 128)

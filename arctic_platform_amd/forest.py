@@ -32,8 +32,8 @@ class ForestMetadata:
     plan: _lib.FcaPlan
     layout: _lib.FcaMetaLayout
     meta: torch.Tensor  # int32 workspace on the device
-    partial_out: torch.Tensor  # fp32 [S * max_partials, Hq, D]
-    partial_lse: torch.Tensor  # fp32 [S * max_partials, Hq]
+    partial_out: torch.Tensor  # half [S * max_partials, Hq, D]: rows scaled by a power of two
+    partial_lse: torch.Tensor  # fp32 [S * max_partials, Hq, 2]: {lse, row scale}
     block_table: torch.Tensor
     seq_lens: torch.Tensor
 
@@ -174,12 +174,12 @@ def build_forest_metadata(
             plan=plan,
             layout=layout,
             meta=torch.zeros(nm.value // 4, dtype=torch.int32, device=dev),
-            partial_out=torch.empty(slots, num_q_heads, head_dim, dtype=torch.float32, device=dev),
-            partial_lse=torch.empty(slots, num_q_heads, dtype=torch.float32, device=dev),
+            partial_out=torch.empty(slots, num_q_heads, head_dim, dtype=torch.float16, device=dev),
+            partial_lse=torch.empty(slots, num_q_heads, 2, dtype=torch.float32, device=dev),
             block_table=block_table,
             seq_lens=seq_lens,
         )
-        assert md.partial_out.numel() * 4 == no.value and md.partial_lse.numel() * 4 == nl.value
+        assert md.partial_out.numel() * 2 == no.value and md.partial_lse.numel() * 4 == nl.value
     entry = lib.fca_update_metadata if update and same_workspace else lib.fca_build_metadata
     _lib.check(
         entry(

@@ -110,8 +110,11 @@ typedef struct fca_meta_layout {
 int fca_version(void);
 const char* fca_last_error(void);
 
-/* Workspace sizes for a plan: metadata (int32 arrays) and the two partial buffers
- * (fp32 [S * max_partials, Hq, D] and fp32 [S * max_partials, Hq]). */
+/* Workspace sizes for a plan: metadata (int32 arrays) and the two partial buffers.  A
+ * partial output row is D half-precision values times one power-of-two scale per row:
+ * partial_out is half [S * max_partials, Hq, D], partial_lse is fp32
+ * [S * max_partials, Hq, 2] = {natural-log lse, scale}.  Both are opaque to the caller:
+ * written by the passes, read by the merge. */
 int fca_workspace_bytes(const fca_plan* plan, size_t* meta_bytes, size_t* partial_out_bytes, size_t* partial_lse_bytes);
 int fca_meta_describe(const fca_plan* plan, fca_meta_layout* layout);
 
@@ -134,26 +137,26 @@ int fca_build_metadata(const fca_plan* plan, const int32_t* block_table_dev, int
 int fca_update_metadata(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,
                         const int32_t* seq_lens_dev, void* meta_dev, void* stream);
 
-/* Shared-prefix pass: work items of shared nodes only.  Writes normalised fp32 partial
+/* Shared-prefix pass: work items of shared nodes only.  Writes normalised partial
  * outputs and natural-log LSEs into the slots the metadata assigns. */
 int fca_prefix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev,
-                    float* partial_out_dev, float* partial_lse_dev, void* stream);
+                    void* partial_out_dev, float* partial_lse_dev, void* stream);
 /* Per-sequence suffix pass: work items of private leaves only (with max_levels = 0 this
  * is the non-cascade paged decode kernel). */
 int fca_suffix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev,
-                    float* partial_out_dev, float* partial_lse_dev, void* stream);
+                    void* partial_out_dev, float* partial_lse_dev, void* stream);
 /* Both classes of work items in one launch (what fca_decode_step runs before its merge). */
 int fca_forest_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev,
-                    float* partial_out_dev, float* partial_lse_dev, void* stream);
+                    void* partial_out_dev, float* partial_lse_dev, void* stream);
 /* Log-sum-exp merge of each sequence's partials (online max / rescaled sum as in
  * arctic_platform/model/implementations/qwen35/models/layers/lm_head.py:190-202).
  * out: [S, Hq, D] bf16 or f32; lse: fp32 [S, Hq], natural log, may be NULL. */
-int fca_merge(const fca_plan* plan, const void* meta_dev, const float* partial_out_dev,
+int fca_merge(const fca_plan* plan, const void* meta_dev, const void* partial_out_dev,
               const float* partial_lse_dev, void* out_dev, int64_t out_seq_stride, int64_t out_head_stride,
               int32_t out_dtype, float* lse_dev, void* stream);
 /* One layer's decode attention: prefix and suffix items in one launch, then the merge. */
 int fca_decode_step(const fca_plan* plan, const fca_tensors* t, void* meta_dev,
-                    float* partial_out_dev, float* partial_lse_dev, void* out_dev, int64_t out_seq_stride,
+                    void* partial_out_dev, float* partial_lse_dev, void* out_dev, int64_t out_seq_stride,
                     int64_t out_head_stride, int32_t out_dtype, float* lse_dev, void* stream);
 
 /* KV-cache append, the step before decode attention in every layer: scatter the new

@@ -44,8 +44,8 @@ def test_workspace_sizes(lib):
     nm, no, nl = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
     assert lib.fca_workspace_bytes(ctypes.byref(plan), ctypes.byref(nm), ctypes.byref(no), ctypes.byref(nl)) == 0
     assert nm.value == layout.total_int32 * 4
-    assert no.value == 512 * layout.max_partials * 32 * 128 * 4
-    assert nl.value == 512 * layout.max_partials * 32 * 4
+    assert no.value == 512 * layout.max_partials * 32 * 128 * 2  # half-precision rows
+    assert nl.value == 512 * layout.max_partials * 32 * 2 * 4  # {lse, scale}
 
 
 @pytest.mark.parametrize(
