@@ -26,7 +26,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the attention kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE
 # passes summarised in profiles/, keyed by (configuration, chunk_tokens, rows_per_item).
 # Counters cannot be read from inside this process; other shapes report null.
-MEASURED_TRAFFIC_BYTES = {(2, 1024, 32): 1_883_600_000}
+MEASURED_TRAFFIC_BYTES = {(2, 1024, 32): 1_865_600_000}
 METRIC = "cascade decode-attn µs/step & % of HBM peak, Qwen3-4B shape 512 seqs"
 
 
