@@ -41,6 +41,8 @@ CASES = [
     (6, 32, 8, 128, torch.float8_e4m3fn, 5, 2, (1, 80), (1, 60), 32, 64),  # deep tree, fp8, 64 rows
     (7, 64, 2, 128, torch.bfloat16, 2, 3, (1, 100), (1, 40), 1024, 32),  # GQA 32: one member per 32-row tile
     (8, 4, 4, 64, torch.bfloat16, 6, 2, (1, 40), (0, 20), 32, 32),  # deeper than the default level cap
+    (9, 32, 2, 64, torch.bfloat16, 3, 4, (1, 120), (1, 80), 64, 64),  # GQA 16, D 64, four members per 64-row tile
+    (10, 16, 2, 64, torch.float8_e4m3fn, 4, 3, (1, 100), (1, 60), 32, 64),  # fp8, D 64, 64 rows
 ]
 
 
