@@ -103,6 +103,8 @@ int run_attend(const fca_plan* p, const fca_tensors* t, void* meta, void* po, fl
   if (int rc = check_plan(p)) return rc;
   if (int rc = check_tensors(p, t)) return rc;
   if (!meta || !po || !pl) return fail(FCA_ERR_INVALID_ARG, "metadata and partial workspaces must be non-NULL");
+  if ((reinterpret_cast<uintptr_t>(po) & 15) || (reinterpret_cast<uintptr_t>(pl) & 15))
+    return fail(FCA_ERR_INVALID_ARG, "partial workspaces must be 16-byte aligned");
   const fca::AttendParams a = attend_params(p, t, meta, po, pl, select);
   hipError_t e = fca::launch_attend(a, *p, t->kv_dtype, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? FCA_OK : hip_fail(e, "attention pass launch");
@@ -114,6 +116,8 @@ int run_merge(const fca_plan* p, const void* meta, const void* po, const float* 
   if (!meta || !po || !pl || !out) return fail(FCA_ERR_INVALID_ARG, "metadata, partials and out must be non-NULL");
   if (out_dtype != FCA_BF16 && out_dtype != FCA_F32)
     return fail(FCA_ERR_UNSUPPORTED, "out dtype %d is not supported (bf16 or f32)", out_dtype);
+  if ((reinterpret_cast<uintptr_t>(po) & 15) || (reinterpret_cast<uintptr_t>(pl) & 15))
+    return fail(FCA_ERR_INVALID_ARG, "partial workspaces must be 16-byte aligned");
   const fca::MetaLayout L = fca::make_layout(*p);
   fca::MergeParams m{};
   m.seq_npart = static_cast<const int32_t*>(meta) + L.seq_npart;
@@ -128,6 +132,9 @@ int run_merge(const fca_plan* p, const void* meta, const void* po, const float* 
   m.head_dim = p->head_dim;
   m.max_partials = (int32_t)L.max_partials;
   m.out_dtype = out_dtype;
+  // whole 16-byte stores when every 8-channel group of out is 16-byte aligned
+  const int64_t esz = out_dtype == FCA_F32 ? 4 : 2;
+  m.vector_out = !(reinterpret_cast<uintptr_t>(out) & 15) && (oss * esz) % 16 == 0 && (ohs * esz) % 16 == 0;
   hipError_t e = fca::launch_merge(m, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? FCA_OK : hip_fail(e, "merge launch");
 }

@@ -154,6 +154,7 @@ struct MergeParams {
   int64_t out_seq_stride, out_head_stride;
   float* lse;
   int32_t num_seqs, num_q_heads, head_dim, max_partials, out_dtype;
+  int32_t vector_out;  // out rows allow 16-byte stores
 };
 
 struct AppendParams {

@@ -53,12 +53,27 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
   const int64_t o = (int64_t)s * p.out_seq_stride + (int64_t)hq * p.out_head_stride + sub * V;
   if (p.out_dtype == FCA_F32) {
     float* dst = reinterpret_cast<float*>(p.out) + o;
+    if (p.vector_out) {
+      reinterpret_cast<float4*>(dst)[0] = make_float4(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv);
+      reinterpret_cast<float4*>(dst)[1] = make_float4(acc[4] * inv, acc[5] * inv, acc[6] * inv, acc[7] * inv);
+    } else {
 #pragma unroll
-    for (int e = 0; e < V; ++e) dst[e] = acc[e] * inv;
+      for (int e = 0; e < V; ++e) dst[e] = acc[e] * inv;
+    }
   } else {
     __hip_bfloat16* dst = reinterpret_cast<__hip_bfloat16*>(p.out) + o;
+    if (p.vector_out) {
+      union {
+        __hip_bfloat16 h[V];
+        uint4 u;
+      } pack;
 #pragma unroll
-    for (int e = 0; e < V; ++e) dst[e] = __float2bfloat16(acc[e] * inv);
+      for (int e = 0; e < V; ++e) pack.h[e] = __float2bfloat16(acc[e] * inv);
+      *reinterpret_cast<uint4*>(dst) = pack.u;
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) dst[e] = __float2bfloat16(acc[e] * inv);
+    }
   }
   if (p.lse && sub == 0) p.lse[row] = wsum > 0.f ? m + __logf(wsum) : -INFINITY;
 }
