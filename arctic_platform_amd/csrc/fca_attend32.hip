@@ -21,7 +21,6 @@
 
 namespace fca {
 
-
 template <int D, bool FP8, bool STREAM>
 __global__ __launch_bounds__(kThreads, 1) void fca_attend32_kernel(AttendParams p) {
   constexpr int KS = D / 16;   // MFMA steps of the score product
