@@ -10,9 +10,14 @@ recipes/rl/skyrl/txt2sql/run_qwen3_8b_bird_grpo_arl.sh:98-111).  The engine itse
 not part of the reference tree, so the class and argument names below follow the engine's
 public plug-in convention from its documentation, not from code in the reference.
 
-Decode batches only (one query token per sequence).  Prefill and mixed batches belong to
-a stock backend on the same cache; they are rejected here with a clear error when the
-metadata is built, never in the middle of a layer.
+Decode batches: one query token per sequence, or a few (the verify step of speculative
+decoding, ``spec_model`` in the platform's config).  A sequence with several query tokens
+is handed to the kernels as that many sequences over the same block-table row, each one
+token longer than the one before it; the forest builder then finds their common blocks
+like any other shared prefix, so causal order among the new tokens needs no mask and no
+kernel of its own.  Prefill and mixed batches with long query runs belong to a stock
+backend on the same cache; they are rejected here with a clear error when the metadata is
+built, never in the middle of a layer.
 """
 
 from __future__ import annotations
@@ -40,6 +45,10 @@ class CommonAttentionMetadata:
     num_reqs: int
     max_query_len: int
     num_actual_tokens: int | None = None
+
+
+# longest run of query tokens per sequence that is still treated as decode
+MAX_DECODE_QUERY_LEN = 16
 
 
 @dataclasses.dataclass
@@ -117,13 +126,24 @@ class ForestCascadeMetadataBuilder:
 
     def build(self, common_prefix_len: int, common_attn_metadata: CommonAttentionMetadata) -> ForestCascadeMetadata:
         m = common_attn_metadata
-        if m.max_query_len != 1:
+        if m.max_query_len > MAX_DECODE_QUERY_LEN or m.max_query_len < 1:
             raise NotImplementedError(
-                "forest cascade attention handles decode batches (one query token per sequence); "
-                f"got max_query_len={m.max_query_len}: route prefill and mixed batches to a stock backend"
+                "forest cascade attention handles decode batches (up to "
+                f"{MAX_DECODE_QUERY_LEN} query tokens per sequence); got max_query_len={m.max_query_len}: "
+                "route prefill and mixed batches to a stock backend"
             )
         bt, sl = m.block_table_tensor[: m.num_reqs], m.seq_lens[: m.num_reqs]
-        key = (m.num_reqs, bt.shape[1])
+        num_tokens = m.num_reqs
+        if m.max_query_len > 1:
+            # one row per query token: the row of its sequence, cut off behind the token itself
+            starts = m.query_start_loc[: m.num_reqs + 1].to(torch.int64)
+            q_lens = starts[1:] - starts[:-1]
+            num_tokens = m.num_actual_tokens if m.num_actual_tokens is not None else int(starts[-1])
+            req = torch.repeat_interleave(torch.arange(m.num_reqs, device=bt.device), q_lens, output_size=num_tokens)
+            ahead = starts[1:][req] - 1 - torch.arange(num_tokens, device=bt.device)  # query tokens after this one
+            sl = (sl[req].to(torch.int64) - ahead).to(torch.int32)
+            bt = bt[req].contiguous()
+        key = (num_tokens, bt.shape[1], m.max_query_len > 1)
         since = self._steps_since_build.get(key, self.rebuild_every)
         update = key in self._workspaces and since + 1 < self.rebuild_every
         self._steps_since_build[key] = since + 1 if update else 0
@@ -137,12 +157,13 @@ class ForestCascadeMetadataBuilder:
             chunk_tokens=self.chunk_tokens,
             rows_per_item=self.rows_per_item,
             cascade=self.enabled,
-            max_levels=self.max_levels,
+            # the query tokens of a sequence share its private blocks: one more level
+            max_levels=min(self.max_levels + (1 if m.max_query_len > 1 else 0), 8),
             out=self._workspaces.get(key),
             update=update,
         )
         self._workspaces[key] = forest
-        return ForestCascadeMetadata(forest=forest, slot_mapping=m.slot_mapping[: m.num_reqs], num_decode_tokens=m.num_reqs)
+        return ForestCascadeMetadata(forest=forest, slot_mapping=m.slot_mapping[:num_tokens], num_decode_tokens=num_tokens)
 
 
 class ForestCascadeAttentionImpl:

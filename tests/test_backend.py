@@ -35,7 +35,7 @@ def test_config_string_and_rejections():
     with pytest.raises(ValueError):
         ForestCascadeMetadataBuilder(30, 8, 128, device="cpu")
     builder = ForestCascadeMetadataBuilder(32, 8, 128, device="cpu", forest_cascade_attn_configs="{}")
-    meta = CommonAttentionMetadata(None, None, None, None, num_reqs=4, max_query_len=7)
+    meta = CommonAttentionMetadata(None, None, None, None, num_reqs=4, max_query_len=64)  # a prefill chunk
     with pytest.raises(NotImplementedError, match="decode"):
         builder.build(0, meta)
 
@@ -94,3 +94,60 @@ def test_decode_loop_through_backend(gpu, index):
         assert_matches_oracle(out.view(w.num_seqs, hq, d), ref_lse.float(), ref_out, ref_lse, what=f"C{index} step {step}")
         assert meta.forest.header()["shared_nodes"] == 8
         assert meta.forest.header()["updates"] == step, "steps after the first are length-only updates"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("q_lens_kind", ["uniform3", "mixed"])
+def test_several_query_tokens_per_sequence(gpu, q_lens_kind):
+    """The verify step of speculative decoding: a sequence brings several query tokens, each
+    seeing the cache up to and including itself.  The adapter turns every query token into a
+    row of its own over the sequence's block table; outputs are checked against the oracle
+    run on exactly those rows."""
+    from arctic_platform_amd.workloads import make_config
+    from tests.helpers import assert_matches_oracle, oracle_for
+    import dataclasses
+
+    w = make_config(2, device=gpu, shrink=8)
+    hq, hkv, d = w.num_q_heads, w.num_kv_heads, w.head_dim
+    builder = ForestCascadeAttentionBackend.get_builder_cls()(hq, hkv, d, device=gpu, forest_cascade_attn_configs='{"chunk_tokens": 128}')
+    impl = ForestCascadeAttentionBackend.get_impl_cls()(hq, d, w.scale, hkv)
+    gen = torch.Generator().manual_seed(4)
+    S = w.num_seqs
+    if q_lens_kind == "uniform3":
+        q_lens = torch.full((S,), 3, dtype=torch.int64)
+    else:
+        q_lens = torch.randint(1, 6, (S,), generator=gen)
+    q_lens = torch.minimum(q_lens, w.seq_lens.cpu().long())  # a sequence cannot bring more tokens than it has
+    starts = torch.cat([torch.zeros(1, dtype=torch.int64), q_lens.cumsum(0)])
+    T = int(starts[-1])
+    q = torch.randn(T, hq * d, generator=gen).to(torch.bfloat16).to(gpu)
+    common = CommonAttentionMetadata(
+        query_start_loc=starts.to(torch.int32).to(gpu),
+        seq_lens=w.seq_lens,
+        block_table_tensor=w.block_table,
+        slot_mapping=torch.zeros(T, dtype=torch.int64, device=gpu),
+        num_reqs=S,
+        max_query_len=int(q_lens.max()),
+        num_actual_tokens=T,
+    )
+    layer = types.SimpleNamespace(k_scale=None, v_scale=None)
+    for step in range(2):  # the second call takes the update path on the same workspace
+        meta = builder.build(0, common)
+        out = impl.forward(layer, q, None, None, w.kv_cache, meta)
+        torch.cuda.synchronize()
+        meta.forest.check()
+        assert meta.forest.header()["updates"] == step
+        # the oracle on one row per query token
+        req = torch.repeat_interleave(torch.arange(S), q_lens)
+        ahead = starts[1:][req] - 1 - torch.arange(T)
+        rows = dataclasses.replace(
+            w,
+            q=q.view(T, hq, d),
+            block_table=w.block_table[req.to(gpu)],
+            seq_lens=(w.seq_lens.cpu().long()[req] - ahead).to(torch.int32).to(gpu),
+        )
+        ref_out, ref_lse = oracle_for(rows)
+        assert_matches_oracle(out.view(T, hq, d), ref_lse.float(), ref_out, ref_lse, what=f"{q_lens_kind} step {step}")
+    # the query tokens of a sequence share its private blocks: more shared nodes than groups
+    assert meta.forest.header()["shared_nodes"] > 8
+
