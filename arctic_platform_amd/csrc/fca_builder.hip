@@ -25,25 +25,34 @@ constexpr int kBuildThreads = 1024;
 constexpr unsigned long long kEmptyKey = ~0ull;
 
 // Exclusive prefix sum of in[0..n) into out[0..n) by the whole workgroup; returns the
-// total to every thread.  `in` may alias `out`.
+// total to every thread.  `in` may alias `out`.  Every thread sums a contiguous slice,
+// the slice sums are scanned inside each wave with lane shuffles and across the sixteen
+// waves through LDS: three barriers in all.
 __device__ int block_exclusive_scan(const int* in, int* out, int n, int* lds) {
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int per = (n + kBuildThreads - 1) / kBuildThreads;
   const int lo = min(tid * per, n), hi = min(lo + per, n);
   int sum = 0;
   for (int i = lo; i < hi; ++i) sum += in[i];
-  lds[tid] = sum;
-  __syncthreads();
-  for (int off = 1; off < kBuildThreads; off <<= 1) {
-    int v = tid >= off ? lds[tid - off] : 0;
-    __syncthreads();
-    lds[tid] += v;
-    __syncthreads();
+  int incl = sum;  // inclusive scan over the lanes of the wave
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int v = __shfl_up(incl, off);
+    if (lane >= off) incl += v;
   }
-  int run = tid ? lds[tid - 1] : 0;
-  const int total = lds[kBuildThreads - 1];
+  if (lane == 63) lds[wave] = incl;
+  __syncthreads();
+  int wave_base = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < kBuildThreads / 64; ++w) {
+    const int v = lds[w];
+    if (w < wave) wave_base += v;
+    total += v;
+  }
+  __syncthreads();  // lds is reused by the next call
+  int run = wave_base + incl - sum;
   for (int i = lo; i < hi; ++i) {
-    int v = in[i];
+    const int v = in[i];
     out[i] = run;
     run += v;
   }
@@ -112,6 +121,7 @@ __device__ inline int plan_fingerprint(const fca_plan& pl) {
 __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p) {
   __shared__ int lds_scan[kBuildThreads];
   __shared__ int lds_mismatch;
+  __shared__ int lds_any;
   __shared__ int lds_hist[2 * kSizeBuckets];
   __shared__ int lds_cursor[2 * kSizeBuckets];
   __shared__ unsigned long long lds_tokens;
@@ -199,6 +209,7 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
     __syncthreads();
 
     for (int level = 0; level < p.plan.max_levels; ++level) {
+      if (tid == 0) lds_any = 0;
       for (int i = tid; i < hsize; i += kBuildThreads) {
         hkeys[i] = kEmptyKey;
         hmin[i] = 0x7fffffff;
@@ -230,9 +241,11 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
         if (slot[s] >= 0) {
           leader[s] = hmin[slot[s]];
           lcp[s] = nfull[s] - pos[s];
+          if (leader[s] != s) lds_any = 1;  // somebody follows a leader: a group of two or more
         }
       }
       __syncthreads();
+      if (!lds_any) break;  // every key is alone: no shared node at this level or below
       // Common run with the leader = first position where the two rows differ.  Every group
       // of 16 lanes takes its own sequence (64 sequences in flight per pass) and scans 256
       // positions per round, 16 independent loads per lane and row.
