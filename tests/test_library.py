@@ -89,3 +89,34 @@ def test_operators_refuse_cpu_tensors():
         build_forest_metadata(
             torch.zeros(2, 4, dtype=torch.int32), torch.ones(2, dtype=torch.int32), num_q_heads=8, num_kv_heads=2, head_dim=64
         )
+
+
+def test_header_is_plain_c_and_links(tmp_path):
+    """include/zorro_fca.h compiles as C99 and as C++, and a C program that only sizes a
+    workspace links against the library and runs without a GPU."""
+    import shutil
+    import subprocess
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler")
+    src = tmp_path / "probe.c"
+    src.write_text(
+        '#include "zorro_fca.h"\n#include <stdio.h>\n'
+        "int main(void) {\n"
+        "  fca_plan p = {512, 320, 32, 8, 128, 16, 1024, 32, 4};\n"
+        "  size_t m = 0, o = 0, l = 0;\n"
+        "  if (fca_workspace_bytes(&p, &m, &o, &l) != 0) { puts(fca_last_error()); return 1; }\n"
+        '  printf("%d %zu %zu %zu\\n", fca_version(), m, o, l);\n'
+        "  p.head_dim = 96;\n"
+        "  return fca_workspace_bytes(&p, &m, &o, &l) == 0;  /* must be refused */\n"
+        "}\n"
+    )
+    inc, libdir = os.path.join(root, "include"), os.path.join(root, "arctic_platform_amd")
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-x", "c", os.path.join(inc, "zorro_fca.h")], check=True)
+    subprocess.run([shutil.which("g++") or gcc, "-std=c++17", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", os.path.join(inc, "zorro_fca.h")], check=True)
+    exe = tmp_path / "probe"
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", f"-I{inc}", str(src), f"-L{libdir}", "-lzorro_fca", f"-Wl,-rpath,{libdir}", "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    assert int(out[0]) >= 1 and int(out[2]) == 512 * (320 * 16 // 1024 + 5) * 32 * 128 * 2
