@@ -189,3 +189,16 @@ def test_many_small_items_drawn_from_the_counter(gpu, rows, dtype):
             first = (out.clone(), lse.clone())
         else:
             assert torch.equal(out, first[0]) and torch.equal(lse, first[1]), "launches on one metadata differ"
+    # the same under graph replay: the counter has to re-arm itself, nothing clears it
+    out_g = torch.empty_like(first[0])
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            forest_cascade_decode(w.q, w.kv_cache, md, w.scale, w.k_scale, w.v_scale, out=out_g, return_lse=False)
+    for replay in range(3):
+        out_g.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, first[0]), f"replay {replay} differs from the eager launch"
+        assert int(md.meta[md.layout.header + 3]) == 0
