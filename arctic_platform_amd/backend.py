@@ -119,6 +119,9 @@ class ForestCascadeMetadataBuilder:
         self.rebuild_every = max(1, int(cfg.get("rebuild_every", 32)))
         group = num_q_heads // num_kv_heads
         self.rows_per_item = int(cfg.get("rows_per_item", 64 if group > 32 else 32))
+        # several query tokens per sequence multiply the rows of every shared node: unless the
+        # configuration fixes the tile height, such steps use 64-row tiles
+        self.rows_multi_token = int(cfg.get("rows_per_item", 64))
         if group > self.rows_per_item:
             raise ValueError(f"{group} query heads per KV head do not fit rows_per_item={self.rows_per_item}")
         self._workspaces: dict = {}
@@ -155,7 +158,7 @@ class ForestCascadeMetadataBuilder:
             head_dim=self.head_dim,
             block_size=BLOCK_SIZE,
             chunk_tokens=self.chunk_tokens,
-            rows_per_item=self.rows_per_item,
+            rows_per_item=self.rows_multi_token if m.max_query_len > 1 else self.rows_per_item,
             cascade=self.enabled,
             # the query tokens of a sequence share its private blocks: one more level
             max_levels=min(self.max_levels + (1 if m.max_query_len > 1 else 0), 8),
