@@ -42,6 +42,7 @@ def parse_args():
     ap.add_argument("--rows", type=int, default=0, help="query rows per work item, 32 or 64 (0 = default)")
     ap.add_argument("--cpu-seqs", type=int, default=512, help="sequences in the CPU baseline sample (0 = skip)")
     ap.add_argument("--skip-noncascade", action="store_true")
+    ap.add_argument("--split-passes", action="store_true", help="also time the shared-prefix pass and the suffix pass as launches of their own (and leave them in the trace for the profiler)")
     ap.add_argument("--calibrate", action="store_true", help="also run the library's plain copy kernel over 1 GiB (counter yardstick)")
     return ap.parse_args()
 
@@ -174,6 +175,21 @@ def main():
     update_us = ev_time(refresh)
     merge_us = ev_time(lambda: ops.merge_partials(md, w.q, out=out, return_lse=False))
 
+    split = None
+    if args.split_passes:
+        shared_tokens = sum(n["num_blocks"] * 16 for n in md.nodes())
+        prefix_bytes = shared_tokens * w.kv_bytes_per_token
+        tp = ev_time(lambda: ops.prefix_pass(w.q, w.kv_cache, md, w.scale, w.k_scale, w.v_scale))
+        ts = ev_time(lambda: ops.suffix_pass(w.q, w.kv_cache, md, w.scale, w.k_scale, w.v_scale))
+        split = {
+            "prefix_pass_us": round(tp, 2),
+            "prefix_unique_kv_bytes": prefix_bytes,
+            "prefix_gbs": round(prefix_bytes / tp / 1e3, 1),
+            "suffix_pass_us": round(ts, 2),
+            "suffix_unique_kv_bytes": unique_bytes - prefix_bytes,
+            "suffix_gbs": round((unique_bytes - prefix_bytes) / ts / 1e3, 1),
+        }
+
     result = {
         "metric": METRIC,
         "value": round(step_us, 2),
@@ -220,6 +236,9 @@ def main():
             "launches_timed": len(kern_us),
         },
     }
+
+    if split is not None:
+        result["split_passes"] = split
 
     if args.calibrate:
         from arctic_platform_amd import _lib
