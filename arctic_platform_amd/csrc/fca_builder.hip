@@ -165,7 +165,9 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       for (int s = gid; s < S; s += kBuildThreads / 16) {
         const int len = p.seq_lens[s];
         const int shared_blocks = pos[s];
-        bool ok = len >= 0 && len <= p.plan.max_blocks * kBlock && len / kBlock >= shared_blocks;
+        // (a sequence that got shorter is a new request in an old slot: build anew, it may
+        // share more than its predecessor did)
+        bool ok = len >= tmp1[s] && len <= p.plan.max_blocks * kBlock && len / kBlock >= shared_blocks;
         if (ok) ok = row_fingerprint(p.block_table + s * p.bt_stride, shared_blocks, glane) == sig[s];
         if (!ok && glane == 0) lds_mismatch = 1;
       }

@@ -127,8 +127,8 @@ int fca_build_metadata(const fca_plan* plan, const int32_t* block_table_dev, int
 /* The same for the next scheduler step of a running decode loop, into a workspace that a
  * build (or an earlier update) has filled: sequences have grown and may have taken new
  * private blocks.  The forest is kept if every row still starts with the blocks its shared
- * nodes were built from (compared through a per-row fingerprint) and those are still full
- * blocks of the row; then only the private leaves and the work list are made again, at a
+ * nodes were built from (compared through a per-row fingerprint), those are still full
+ * blocks of the row and no sequence got shorter; then only the private leaves and the work list are made again, at a
  * fraction of the cost.  Otherwise, or on a workspace never built or built for another
  * plan, this is fca_build_metadata.  Either way the result is valid for the given rows; a
  * kept forest may miss sharing that only a new build would find.  Header slot 14 counts

@@ -90,6 +90,18 @@ def test_update_detects_a_changed_batch(gpu):
     assert md.header()["updates"] == 0
     assert _semantics(md) == _semantics(fresh)
 
+    # a slot reused by a new request that is shorter than its predecessor but longer than the
+    # predecessor's shared prefix: still a full build (the newcomer may share more)
+    sl1 = sl.clone()
+    sl1[7] = int(sl[7]) - 1
+    md = build_forest_metadata(bt, sl1, out=md, update=True, **kw)
+    torch.cuda.synchronize()
+    assert md.header()["updates"] == 0
+    md = build_forest_metadata(bt, sl1, out=md, update=True, **kw)
+    torch.cuda.synchronize()
+    assert md.header()["updates"] == 1
+    sl = sl1
+
     # bad length: the full build flags it
     sl2 = sl.clone()
     sl2[0] = -4
