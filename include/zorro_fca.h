@@ -20,9 +20,12 @@
  *     performs no host<->device synchronisation and allocates nothing;
  *   - the caller owns every buffer, including the metadata and partial workspaces whose
  *     sizes fca_workspace_bytes() reports;
- *   - the attention and merge calls only read the metadata workspace; the partial
- *     workspaces are written by the attention call and read by the merge, so two layers
- *     running concurrently on different streams need separate partial workspaces.
+ *   - the attention and merge calls read the metadata workspace; the attention call also
+ *     uses one self-resetting work counter in its header (zero before and after every
+ *     launch), and the partial workspaces are written by the attention call and read by
+ *     the merge.  Calls that use one set of workspaces must therefore not overlap in
+ *     time: stream order is enough; layers running concurrently on different streams need
+ *     their own metadata and partial workspaces.
  */
 #ifndef ZORRO_FCA_H
 #define ZORRO_FCA_H
