@@ -14,6 +14,9 @@ typedef int i32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
+// Workgroups a CU holds at once: a wave's register budget is 512 / this.
+template <int D>
+constexpr int kWorkgroupsPerCu = D == 64 ? 2 : 1;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 constexpr float kRescaleSlack = 8.f;  // log2 units: rescale when a row maximum rises by more than 2^8
