@@ -24,6 +24,7 @@ EXPORTS = (
     "fca_meta_describe",
     "fca_build_metadata",
     "fca_update_metadata",
+    "fca_build_metadata_rows",
     "fca_prefix_pass",
     "fca_suffix_pass",
     "fca_forest_pass",
@@ -58,7 +59,7 @@ class FcaTensors(ctypes.Structure):
         ("kv_block_stride", ctypes.c_int64),
         ("kv_head_stride", ctypes.c_int64),
         ("kv_dtype", ctypes.c_int32),
-        ("reserved", ctypes.c_int32),
+        ("kv_reread", ctypes.c_int32),
         ("block_table_dev", ctypes.c_void_p),
         ("block_table_stride", ctypes.c_int64),
         ("k_scale_dev", ctypes.c_void_p),
@@ -130,6 +131,7 @@ def load_library() -> ctypes.CDLL:
     lib.fca_meta_describe.argtypes = [P(FcaPlan), P(FcaMetaLayout)]
     lib.fca_build_metadata.argtypes = [P(FcaPlan), VP, I64, VP, VP, VP]
     lib.fca_update_metadata.argtypes = [P(FcaPlan), VP, I64, VP, VP, VP]
+    lib.fca_build_metadata_rows.argtypes = [P(FcaPlan), VP, I64, I32, VP, VP, VP, VP, I32, VP]
     attend = [P(FcaPlan), P(FcaTensors), VP, VP, VP, VP]
     lib.fca_prefix_pass.argtypes = attend
     lib.fca_suffix_pass.argtypes = attend

@@ -12,12 +12,17 @@ public plug-in convention from its documentation, not from code in the reference
 
 Decode batches: one query token per sequence, or a few (the verify step of speculative
 decoding, ``spec_model`` in the platform's config).  A sequence with several query tokens
-is handed to the kernels as that many sequences over the same block-table row, each one
+is handed to the kernels as that many query rows over the same block-table row, each one
 token longer than the one before it; the forest builder then finds their common blocks
 like any other shared prefix, so causal order among the new tokens needs no mask and no
-kernel of its own.  Prefill and mixed batches with long query runs belong to a stock
-backend on the same cache; they are rejected here with a clear error when the metadata is
-built, never in the middle of a layer.
+kernel of its own.
+
+Prefill chunks and mixed batches go the same way.  A run longer than
+``MAX_DECODE_QUERY_LEN`` tokens is cut into tiles, one per 16-token block of the cache:
+the rows of a tile are declared a group (``fca_build_metadata_rows``), read the KV before
+their block once for all of them through the shared-node items, and each reads its own
+block alone.  The response-over-shared-prompt attention of the trainer is the in-tree
+counterpart (arctic_platform/rl/zorro_train/qwen_attention_patcher.py:1117-1262).
 """
 
 from __future__ import annotations
@@ -47,7 +52,8 @@ class CommonAttentionMetadata:
     num_actual_tokens: int | None = None
 
 
-# longest run of query tokens per sequence that is still treated as decode
+# Longest run of query tokens per sequence whose rows are grouped by discovery (with the
+# rows of other sequences that share the prompt); longer runs are tiled per cache block.
 MAX_DECODE_QUERY_LEN = 16
 
 
@@ -129,14 +135,11 @@ class ForestCascadeMetadataBuilder:
 
     def build(self, common_prefix_len: int, common_attn_metadata: CommonAttentionMetadata) -> ForestCascadeMetadata:
         m = common_attn_metadata
-        if m.max_query_len > MAX_DECODE_QUERY_LEN or m.max_query_len < 1:
-            raise NotImplementedError(
-                "forest cascade attention handles decode batches (up to "
-                f"{MAX_DECODE_QUERY_LEN} query tokens per sequence); got max_query_len={m.max_query_len}: "
-                "route prefill and mixed batches to a stock backend"
-            )
+        if m.max_query_len < 1:
+            raise ValueError(f"max_query_len must be at least 1, got {m.max_query_len}")
         bt, sl = m.block_table_tensor[: m.num_reqs], m.seq_lens[: m.num_reqs]
         num_tokens = m.num_reqs
+        row_table = row_group = None
         if m.max_query_len > 1:
             # one row per query token: the row of its sequence, cut off behind the token itself
             starts = m.query_start_loc[: m.num_reqs + 1].to(torch.int64)
@@ -145,8 +148,14 @@ class ForestCascadeMetadataBuilder:
             req = torch.repeat_interleave(torch.arange(m.num_reqs, device=bt.device), q_lens, output_size=num_tokens)
             ahead = starts[1:][req] - 1 - torch.arange(num_tokens, device=bt.device)  # query tokens after this one
             sl = (sl[req].to(torch.int64) - ahead).to(torch.int32)
-            bt = bt[req].contiguous()
-        key = (num_tokens, bt.shape[1], m.max_query_len > 1)
+            row_table = req.to(torch.int32)
+            if m.max_query_len > MAX_DECODE_QUERY_LEN:
+                # tiles of the long runs: one group per (sequence, cache block of the token)
+                if m.num_reqs * bt.shape[1] >= 2**31:
+                    raise ValueError("batch too large for 32-bit group ids")
+                tile = req * bt.shape[1] + (sl.to(torch.int64) - 1).clamp_(min=0) // BLOCK_SIZE
+                row_group = torch.where(q_lens[req] > MAX_DECODE_QUERY_LEN, tile, -1).to(torch.int32)
+        key = (num_tokens, bt.shape[1], m.max_query_len > 1, row_group is not None)
         since = self._steps_since_build.get(key, self.rebuild_every)
         update = key in self._workspaces and since + 1 < self.rebuild_every
         self._steps_since_build[key] = since + 1 if update else 0
@@ -163,7 +172,9 @@ class ForestCascadeMetadataBuilder:
             # the query tokens of a sequence share its private blocks: one more level
             max_levels=min(self.max_levels + (1 if m.max_query_len > 1 else 0), 8),
             out=self._workspaces.get(key),
-            update=update,
+            update=update and row_group is None,
+            row_table=row_table,
+            row_group=row_group,
         )
         self._workspaces[key] = forest
         return ForestCascadeMetadata(forest=forest, slot_mapping=m.slot_mapping[:num_tokens], num_decode_tokens=num_tokens)

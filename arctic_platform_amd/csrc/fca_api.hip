@@ -96,6 +96,7 @@ fca::AttendParams attend_params(const fca_plan* p, const fca_tensors* t, void* m
   a.group = p->num_q_heads / p->num_kv_heads;
   a.max_partials = (int32_t)L.max_partials;
   a.select = select;
+  a.kv_reread = t->kv_reread;
   return a;
 }
 
@@ -180,8 +181,12 @@ int fca_meta_describe(const fca_plan* plan, fca_meta_layout* out) {
 }
 
 static int run_build(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,
-                     const int32_t* seq_lens_dev, void* meta_dev, int try_update, void* stream) {
+                     const int32_t* seq_lens_dev, void* meta_dev, int try_update, void* stream,
+                     int32_t table_rows = 0, const int32_t* row_table_dev = nullptr,
+                     const int32_t* row_group_dev = nullptr) {
   if (int rc = check_plan(plan)) return rc;
+  if (row_table_dev && table_rows < 1)
+    return fail(FCA_ERR_INVALID_ARG, "table_rows must be >= 1 when a row table is given, got %d", table_rows);
   if (!block_table_dev || !seq_lens_dev || !meta_dev)
     return fail(FCA_ERR_INVALID_ARG, "block_table, seq_lens and metadata workspace must be non-NULL");
   if (block_table_stride < plan->max_blocks)
@@ -197,6 +202,9 @@ static int run_build(const fca_plan* plan, const int32_t* block_table_dev, int64
   b.meta = static_cast<int32_t*>(meta_dev);
   b.L = fca::make_layout(*plan);
   b.try_update = try_update;
+  b.row_table = row_table_dev;
+  b.row_group = row_group_dev;
+  b.table_rows = table_rows;
   hipError_t e = fca::launch_build(b, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? FCA_OK : hip_fail(e, "metadata builder launch");
 }
@@ -209,6 +217,13 @@ int fca_build_metadata(const fca_plan* plan, const int32_t* block_table_dev, int
 int fca_update_metadata(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,
                         const int32_t* seq_lens_dev, void* meta_dev, void* stream) {
   return run_build(plan, block_table_dev, block_table_stride, seq_lens_dev, meta_dev, 1, stream);
+}
+
+int fca_build_metadata_rows(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,
+                            int32_t table_rows, const int32_t* row_table_dev, const int32_t* row_group_dev,
+                            const int32_t* row_lens_dev, void* meta_dev, int32_t update, void* stream) {
+  return run_build(plan, block_table_dev, block_table_stride, row_lens_dev, meta_dev, update ? 1 : 0, stream, table_rows,
+                   row_table_dev, row_group_dev);
 }
 
 int fca_prefix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev, void* partial_out_dev,

@@ -440,8 +440,9 @@ hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dty
   if (nrt == 1) return launch_attend32(p, plan, kv_dtype, grid, stream);
   // With sharing on, a launch reads every KV block once: stream it past the caches.  With
   // sharing off, sequences of a group read the same blocks again and again and the
-  // memory-side cache serves the repeats, so the loads stay ordinary.
-  const bool stream_kv = plan.max_levels > 0;
+  // memory-side cache serves the repeats, so the loads stay ordinary; likewise when query
+  // runs make successive tiles of a sequence read the same blocks.
+  const bool stream_kv = plan.max_levels > 0 && !p.kv_reread;
 #define FCA_LAUNCH(D_, F_, S_) \
   hipLaunchKernelGGL((fca_attend64_kernel<D_, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, p)
 #define FCA_PICK(D_, F_) \

@@ -367,8 +367,9 @@ hipError_t launch_attend32(const AttendParams& p, const fca_plan& plan, int kv_d
   const bool fp8 = kv_dtype == FCA_FP8_E4M3;
   // With sharing on, a launch reads every KV block once: stream it past the caches.  With
   // sharing off, sequences of a group read the same blocks again and again and the
-  // memory-side cache serves the repeats, so the loads stay ordinary.
-  const bool stream_kv = plan.max_levels > 0;
+  // memory-side cache serves the repeats, so the loads stay ordinary; likewise when query
+  // runs make successive tiles of a sequence read the same blocks.
+  const bool stream_kv = plan.max_levels > 0 && !p.kv_reread;
 #define FCA_LAUNCH(D_, F_, S_) \
   hipLaunchKernelGGL((fca_attend32_kernel<D_, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, p)
 #define FCA_PICK(D_, F_) \

@@ -10,6 +10,13 @@
 // the group's first member, members ascending) follow the trainer's host-side discovery,
 // arctic_platform/rl/zorro_train/zorro_train.py:242-285.
 //
+// Query rows need not be one per block-table row: with a row table, several rows (the
+// tokens of a query run) read one table row up to different lengths.  The caller may
+// declare groups among them; a declared group is keyed by its id at the first level
+// instead of by block id, and its run ends before the block that holds the last token of
+// its shortest row, so that every member keeps a private leaf.  This is how a long run is
+// cut into tiles that each read the KV before them once.
+//
 // Between two scheduler steps of a decode loop only the lengths change: every sequence
 // grows by a token and now and then takes a new private block.  The forest is a function
 // of the shared blocks alone, so an update keeps it as long as every row still carries
@@ -152,6 +159,15 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   int* members = meta + L.members;
   unsigned long long* sig = reinterpret_cast<unsigned long long*>(meta + L.s_sig);
   const int plan_sig = plan_fingerprint(p.plan);
+  // block-table row of query row s
+  auto table_row = [&](int s) -> int64_t {
+    if (!p.row_table) return s;
+    const int r = p.row_table[s];
+    return r >= 0 && r < p.table_rows ? r : 0;  // (out of range: flagged by the full build)
+  };
+  // rows the caller has grouped: the group's common run ends before the block that holds
+  // the last token of its shortest row, so every member keeps a leaf of its own
+  auto declared = [&](int s) { return p.row_group && p.row_group[s] >= 0; };
 
   // ---- update: is the forest of the last build on this workspace still the forest of
   // these rows?  (pos = first private block of a row, ord = chunks of its shared nodes:
@@ -168,7 +184,7 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
         // (a sequence that got shorter is a new request in an old slot: build anew, it may
         // share more than its predecessor did)
         bool ok = len >= tmp1[s] && len <= p.plan.max_blocks * kBlock && len / kBlock >= shared_blocks;
-        if (ok) ok = row_fingerprint(p.block_table + s * p.bt_stride, shared_blocks, glane) == sig[s];
+        if (ok) ok = row_fingerprint(p.block_table + table_row(s) * p.bt_stride, shared_blocks, glane) == sig[s];
         if (!ok && glane == 0) lds_mismatch = 1;
       }
     }
@@ -202,8 +218,9 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
         atomicOr(&hdr[H_ERROR], 1);
         len = max(0, min(len, p.plan.max_blocks * kBlock));
       }
+      if (p.row_table && (p.row_table[s] < 0 || p.row_table[s] >= p.table_rows)) atomicOr(&hdr[H_ERROR], 4);
       tmp1[s] = len;  // validated length, kept for the leaf pass
-      nfull[s] = p.plan.max_levels > 0 ? len / kBlock : 0;
+      nfull[s] = p.plan.max_levels > 0 ? (declared(s) ? max(len - 1, 0) / kBlock : len / kBlock) : 0;
       pos[s] = 0;
       par[s] = -1;
       ord[s] = 0;
@@ -227,8 +244,15 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       // parent is -2 dropped out of sharing at an earlier level.
       for (int s = tid; s < S; s += kBuildThreads) {
         if (par[s] == -2 || pos[s] >= nfull[s]) continue;
-        unsigned blk = (unsigned)p.block_table[s * p.bt_stride + pos[s]];
-        unsigned long long key = ((unsigned long long)(unsigned)(par[s] + 1) << 32) | blk;
+        // The key of a declared group (first level only) is its id; otherwise rows meet
+        // under (parent node, physical block id at the current position).
+        unsigned long long key;
+        if (level == 0 && declared(s)) {
+          key = (1ull << 63) | (unsigned)p.row_group[s];
+        } else {
+          const unsigned blk = (unsigned)p.block_table[table_row(s) * p.bt_stride + pos[s]];
+          key = ((unsigned long long)(unsigned)(par[s] + 1) << 32) | blk;
+        }
         int h = hash_key(key) & (hsize - 1);
         for (int probe = 0; probe < hsize; ++probe) {
           unsigned long long prev = atomicCAS(&hkeys[h], kEmptyKey, key);
@@ -258,10 +282,11 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
           const int t = leader[s];
           if (t < 0 || t == s) continue;
           const int lim = min(nfull[s], nfull[t]) - pos[s];
-          const int32_t* row_s = p.block_table + s * p.bt_stride + pos[s];
-          const int32_t* row_t = p.block_table + t * p.bt_stride + pos[s];
+          const int32_t* row_s = p.block_table + table_row(s) * p.bt_stride + pos[s];
+          const int32_t* row_t = p.block_table + table_row(t) * p.bt_stride + pos[s];
           int first = lim;
-          for (int j0 = 0; j0 < lim && first == lim; j0 += 16 * kPerLane) {
+          // (query rows of one sequence read the same table row: nothing to compare)
+          for (int j0 = 0; row_s != row_t && j0 < lim && first == lim; j0 += 16 * kPerLane) {
             int mine = lim;
 #pragma unroll
             for (int u = kPerLane - 1; u >= 0; --u) {
@@ -342,7 +367,7 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
     {
       const int gid = tid >> 4, glane = tid & 15;
       for (int s = gid; s < S; s += kBuildThreads / 16) {
-        const unsigned long long f = row_fingerprint(p.block_table + s * p.bt_stride, pos[s], glane);
+        const unsigned long long f = row_fingerprint(p.block_table + table_row(s) * p.bt_stride, pos[s], glane);
         if (glane == 0) sig[s] = f;
       }
       if (tid == 0) {
@@ -377,8 +402,9 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   // alternating directions, which balances a descending list well.
   const int total_nodes = node_base + S;
   auto node_fields = [&](int n, int& rep, int& blk, int& tokens, int& moff, int& mcnt, int& o) {
+    // (rep is what the attention kernels index the block table with)
     if (n < node_base) {
-      rep = meta[L.node_rep + n];
+      rep = (int)table_row(meta[L.node_rep + n]);
       blk = meta[L.node_blk + n];
       tokens = meta[L.node_nblk + n] * kBlock;
       moff = meta[L.node_moff + n];
@@ -386,7 +412,7 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       o = meta[L.node_ord + n];
     } else {
       const int s = n - node_base;
-      rep = s;
+      rep = (int)table_row(s);
       blk = pos[s];
       tokens = tmp1[s] - pos[s] * kBlock;
       moff = leaf_members + s;

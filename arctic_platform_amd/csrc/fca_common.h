@@ -124,6 +124,10 @@ struct BuildParams {
   int32_t* meta;
   MetaLayout L;
   int32_t try_update;  // keep the forest of the last build if the rows still carry it
+  // Query rows that are not one per block-table row (all NULL / 0 for the plain case):
+  const int32_t* row_table;  // block-table row of every query row, NULL = the row itself
+  const int32_t* row_group;  // >= 0: rows with the same value form one declared group, NULL = none
+  int32_t table_rows;        // rows of the block table, bounds row_table
 };
 
 struct AttendParams {
@@ -144,6 +148,7 @@ struct AttendParams {
   int32_t num_q_heads, num_kv_heads, group;  // group = Hq / Hkv
   int32_t max_partials;
   int32_t select;  // 0 all items, 1 shared only, 2 leaves only
+  int32_t kv_reread;  // a launch reads KV blocks more than once (query runs): keep the loads cacheable
 };
 
 struct MergeParams {

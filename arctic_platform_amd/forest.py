@@ -35,7 +35,15 @@ class ForestMetadata:
     partial_out: torch.Tensor  # half [S * max_partials, Hq, D]: rows scaled by a power of two
     partial_lse: torch.Tensor  # fp32 [S * max_partials, Hq, 2]: {lse, row scale}
     block_table: torch.Tensor
-    seq_lens: torch.Tensor
+    seq_lens: torch.Tensor  # per query row
+    row_table: torch.Tensor | None = None  # block-table row of every query row (None: the row itself)
+    row_group: torch.Tensor | None = None  # declared groups of query rows
+
+    @property
+    def kv_reread(self) -> bool:
+        """The tiles of a long query run read the same blocks one after the other: keep the
+        KV loads cacheable.  (Rows grouped by discovery alone read a block about once.)"""
+        return self.row_group is not None
 
     # ---- inspection (synchronises; not for the decode loop) -------------------------
     def header(self) -> dict:
@@ -56,6 +64,8 @@ class ForestMetadata:
             raise ValueError("a sequence length is negative or exceeds max_blocks * block_size")
         if err & 2:
             raise RuntimeError("work list overflowed its reserved size")
+        if err & 4:
+            raise ValueError("a row_table entry is outside the block table")
 
     def nodes(self) -> list:
         L, m = self.layout, self.meta.cpu()
@@ -131,8 +141,16 @@ def build_forest_metadata(
     max_levels: int = 4,
     out: ForestMetadata | None = None,
     update: bool = False,
+    row_table: torch.Tensor | None = None,
+    row_group: torch.Tensor | None = None,
 ) -> ForestMetadata:
     """Discover the shared-prefix forest of a decode batch on the device.
+
+    With ``row_table`` (int32 ``[R]``) the query rows are not the block-table rows: query row
+    ``r`` attends to the first ``seq_lens[r]`` tokens of table row ``row_table[r]`` (the tokens
+    of a query run: one row per token, each one token longer), ``seq_lens`` is ``[R]`` and
+    the result serves ``q`` of ``R`` rows.  ``row_group`` (int32 ``[R]``, -1 = none) declares
+    groups of rows that share their leading blocks (``fca_build_metadata_rows``).
 
     ``cascade=False`` turns sharing off: every sequence becomes one private node over its
     whole block-table row, which makes the same kernels a plain paged decode attention.
@@ -145,13 +163,19 @@ def build_forest_metadata(
         raise ValueError(f"block_size must be {BLOCK_SIZE}")
     if block_table.dtype != torch.int32 or seq_lens.dtype != torch.int32:
         raise TypeError("block_table and seq_lens must be int32")
-    if block_table.dim() != 2 or block_table.stride(1) != 1 or seq_lens.shape != (block_table.shape[0],):
-        raise ValueError("block_table must be [num_seqs, max_blocks] with contiguous rows and seq_lens [num_seqs]")
+    if row_table is None and row_group is not None:
+        raise ValueError("row_group needs a row_table")
+    num_rows = block_table.shape[0] if row_table is None else row_table.shape[0]
+    if block_table.dim() != 2 or block_table.stride(1) != 1 or seq_lens.shape != (num_rows,):
+        raise ValueError("block_table must be [num_seqs, max_blocks] with contiguous rows and seq_lens one per query row")
+    for name, t in (("row_table", row_table), ("row_group", row_group)):
+        if t is not None and (t.dtype != torch.int32 or t.shape != (num_rows,) or not t.is_contiguous() or not t.is_cuda):
+            raise ValueError(f"{name} must be a contiguous int32 device tensor with one entry per query row")
     if not block_table.is_cuda:
         raise RuntimeError("forest metadata is built on the GPU; block_table must be a device tensor")
     lib = _lib.load_library()
     plan = make_plan(
-        block_table.shape[0],
+        num_rows,
         block_table.shape[1],
         num_q_heads,
         num_kv_heads,
@@ -162,7 +186,7 @@ def build_forest_metadata(
     )
     same_workspace = out is not None and bytes(out.plan) == bytes(plan)
     if same_workspace:
-        md = dataclasses.replace(out, block_table=block_table, seq_lens=seq_lens)
+        md = dataclasses.replace(out, block_table=block_table, seq_lens=seq_lens, row_table=row_table, row_group=row_group)
     else:
         layout = _lib.FcaMetaLayout()
         _lib.check(lib.fca_meta_describe(ctypes.byref(plan), ctypes.byref(layout)))
@@ -178,8 +202,26 @@ def build_forest_metadata(
             partial_lse=torch.empty(slots, num_q_heads, 2, dtype=torch.float32, device=dev),
             block_table=block_table,
             seq_lens=seq_lens,
+            row_table=row_table,
+            row_group=row_group,
         )
         assert md.partial_out.numel() * 2 == no.value and md.partial_lse.numel() * 4 == nl.value
+    if row_table is not None:
+        _lib.check(
+            lib.fca_build_metadata_rows(
+                ctypes.byref(md.plan),
+                block_table.data_ptr(),
+                block_table.stride(0),
+                block_table.shape[0],
+                row_table.data_ptr(),
+                row_group.data_ptr() if row_group is not None else None,
+                seq_lens.data_ptr(),
+                md.meta.data_ptr(),
+                1 if update and same_workspace else 0,
+                _stream_ptr(block_table.device),
+            )
+        )
+        return md
     entry = lib.fca_update_metadata if update and same_workspace else lib.fca_build_metadata
     _lib.check(
         entry(

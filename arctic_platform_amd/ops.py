@@ -58,7 +58,7 @@ def _tensors(q, kv_cache, meta: ForestMetadata, scale, k_scale, v_scale) -> _lib
         kv_cache.stride(1),
         kv_cache.stride(2),
         kv_dtype,
-        0,
+        1 if meta.kv_reread else 0,
         meta.block_table.data_ptr(),
         meta.block_table.stride(0),
         k_scale.data_ptr() if k_scale is not None else None,

@@ -77,8 +77,11 @@ typedef struct fca_tensors {
   int64_t kv_block_stride;     /* elements between blocks of one plane */
   int64_t kv_head_stride;      /* elements between KV heads of one block */
   int32_t kv_dtype;            /* FCA_BF16 or FCA_FP8_E4M3 */
-  int32_t reserved;
-  const int32_t* block_table_dev; /* [S, max_blocks] physical block ids */
+  int32_t kv_reread;           /* 0: a launch reads every KV block about once (decode), loads bypass
+                                  the caches; non-zero: blocks are read again and again (query runs
+                                  built with fca_build_metadata_rows), loads stay cacheable */
+  const int32_t* block_table_dev; /* [S, max_blocks] physical block ids ([table_rows, max_blocks]
+                                  for metadata built with fca_build_metadata_rows) */
   int64_t block_table_stride;
   const float* k_scale_dev;    /* [Hkv] dequant scales for fp8 caches, or NULL (= 1) */
   const float* v_scale_dev;
@@ -91,7 +94,8 @@ typedef struct fca_tensors {
 typedef struct fca_meta_layout {
   int64_t header;        /* [16]: 0 items, 1 shared items, 2 nodes (shared), 3 work ticket
                             (self-resetting, owned by the attention kernel), 4 reserved,
-                            5 error flag, 6/7 unique tokens lo/hi, 8 levels found,
+                            5 error flags (1 bad length, 2 work list overflow, 4 bad row table
+                            entry), 6/7 unique tokens lo/hi, 8 levels found,
                             10-13 and 15 state for fca_update_metadata, 14 updates since the
                             last full build */
   int64_t seq_npart;     /* [S] partial slots used per sequence */
@@ -139,6 +143,29 @@ int fca_build_metadata(const fca_plan* plan, const int32_t* block_table_dev, int
  * group discovery (arctic_platform/rl/zorro_train/zorro_train.py:242-285 runs once per batch). */
 int fca_update_metadata(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,
                         const int32_t* seq_lens_dev, void* meta_dev, void* stream);
+
+/* Metadata for query rows that are not one per block-table row: a sequence that brings a
+ * run of query tokens (a prefill or a chunk of one, the verify step of speculative
+ * decoding) contributes one query row per token.  plan->num_seqs is the number of query
+ * rows R (rows of q and out); row r attends to the first row_lens_dev[r] tokens of
+ * block-table row row_table_dev[r] (< table_rows), which for token i of a sequence is the
+ * sequence's length up to and including that token, so causal order needs no mask.
+ * row_group_dev may be NULL.  A value >= 0 declares a group: rows with equal values share
+ * their leading blocks, and the builder makes one shared node of the run that ends before
+ * the block holding the last token of the group's shortest row (rows of one table row are
+ * not compared, others are, so a wrong declaration costs sharing, never correctness).
+ * Declared groups are how a long run is tiled: the tokens of one 16-token block form a
+ * group, read the KV before their block once for all of them, and each reads its own
+ * block alone.  Rows with -1 are grouped by discovery as in fca_build_metadata, and
+ * declared groups take part in discovery below their node.  update != 0 asks for the
+ * update of fca_update_metadata.  The attention calls then take the [table_rows,
+ * max_blocks] block table and kv_reread = 1.  Counterpart in the reference: the
+ * response-over-shared-prompt attention of the trainer, which rebuilds full sequences from
+ * de-duplicated prompts (arctic_platform/rl/zorro_train/zorro_train.py:160-235) and runs
+ * a varlen attention over them (rl/zorro_train/qwen_attention_patcher.py:1117-1262). */
+int fca_build_metadata_rows(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,
+                            int32_t table_rows, const int32_t* row_table_dev, const int32_t* row_group_dev,
+                            const int32_t* row_lens_dev, void* meta_dev, int32_t update, void* stream);
 
 /* Shared-prefix pass: work items of shared nodes only.  Writes normalised partial
  * outputs and natural-log LSEs into the slots the metadata assigns. */

@@ -11,6 +11,15 @@ and the comparison is applied recursively, which turns the flat groups into a fo
 A node is a maximal run of leading block-table positions whose physical ids are identical
 for a fixed set of two or more sequences.  Only full blocks can be shared.  What is left
 of a sequence below its deepest shared node is its private leaf.
+
+Query rows need not be block-table rows: with ``row_table`` query row r reads table row
+``row_table[r]`` up to ``seq_lens[r]`` tokens (the tokens of a query run).  ``row_group``
+declares first-level groups among such rows in place of the block-id comparison; for a
+declared row the last block it may share is the one before the block that holds its last
+token, so every member of a declared group keeps a private leaf (this is the tiling of a
+long run: the tokens of one block form a group).  The trainer's counterpart is the
+response-over-shared-prompt attention, which reads each unique prompt once for all its
+responses (arctic_platform/rl/zorro_train/qwen_attention_patcher.py:1117-1262).
 """
 
 from __future__ import annotations
@@ -20,15 +29,17 @@ from collections import OrderedDict
 BLOCK = 16
 
 
-def discover_forest(block_table, seq_lens, block_size=BLOCK, max_levels=8):
+def discover_forest(block_table, seq_lens, block_size=BLOCK, max_levels=8, row_table=None, row_group=None):
     """Returns (nodes, leaves).
 
     nodes: list of dict(members, blk_start, num_blocks, level, parent) for shared runs.
     leaves: per sequence dict(blk_start, tokens, parent): the private remainder.
     """
-    bt = [list(map(int, row)) for row in block_table]
+    table = [list(map(int, row)) for row in block_table]
     lens = [int(n) for n in seq_lens]
-    nfull = [n // block_size for n in lens]
+    bt = table if row_table is None else [table[int(r)] for r in row_table]
+    group_of = [-1] * len(lens) if row_group is None else [int(g) for g in row_group]
+    nfull = [(max(n - 1, 0) if g >= 0 else n) // block_size for n, g in zip(lens, group_of)]
     nodes = []
     leaf_start = [0] * len(lens)
     leaf_parent = [-1] * len(lens)
@@ -39,7 +50,8 @@ def discover_forest(block_table, seq_lens, block_size=BLOCK, max_levels=8):
         groups = OrderedDict()
         for s in members:
             if pos < nfull[s]:
-                groups.setdefault(bt[s][pos], []).append(s)
+                key = ("declared", group_of[s]) if level == 0 and group_of[s] >= 0 else bt[s][pos]
+                groups.setdefault(key, []).append(s)
         for group in groups.values():
             if len(group) < 2:
                 continue

@@ -35,8 +35,8 @@ def test_config_string_and_rejections():
     with pytest.raises(ValueError):
         ForestCascadeMetadataBuilder(30, 8, 128, device="cpu")
     builder = ForestCascadeMetadataBuilder(32, 8, 128, device="cpu", forest_cascade_attn_configs="{}")
-    meta = CommonAttentionMetadata(None, None, None, None, num_reqs=4, max_query_len=64)  # a prefill chunk
-    with pytest.raises(NotImplementedError, match="decode"):
+    meta = CommonAttentionMetadata(None, None, None, None, num_reqs=4, max_query_len=0)
+    with pytest.raises(ValueError, match="max_query_len"):
         builder.build(0, meta)
 
 

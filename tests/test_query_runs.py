@@ -1,0 +1,223 @@
+"""Query runs: several query tokens per sequence (prefill chunks, mixed batches).
+
+One query row per token over the sequence's block-table row; long runs are tiled by
+declaring the tokens of one cache block a group.  CPU tests pin the forest oracle's
+handling of declared groups by coverage invariants and a hand-built case; GPU tests
+compare the kernels with the flat fp64 oracle row by row.
+"""
+
+import random
+
+import pytest
+import torch
+
+from oracle.forest import canonical_nodes, discover_forest
+
+BLOCK = 16
+
+
+def run_rows(ctx_and_query, max_blocks, tile_min=2):
+    """Row arrays of a batch given (context tokens, query tokens) per sequence: the table
+    row, the causal length and the declared group of every query row.  Runs of at least
+    ``tile_min`` tokens are tiled per cache block; shorter ones are left to discovery."""
+    row_table, row_lens, row_group = [], [], []
+    for s, (ctx, ql) in enumerate(ctx_and_query):
+        for i in range(ql):
+            n = ctx + i + 1
+            row_table.append(s)
+            row_lens.append(n)
+            row_group.append(s * max_blocks + (n - 1) // BLOCK if ql >= tile_min else -1)
+    return row_table, row_lens, row_group
+
+
+def covered_tokens(nodes, leaves, row):
+    """Token ranges a row reads through its shared nodes and its leaf, as a sorted list."""
+    spans = [(n["blk_start"] * BLOCK, (n["blk_start"] + n["num_blocks"]) * BLOCK) for n in nodes if row in n["members"]]
+    leaf = leaves[row]
+    spans.append((leaf["blk_start"] * BLOCK, leaf["blk_start"] * BLOCK + leaf["tokens"]))
+    return sorted(spans)
+
+
+def assert_exact_cover(nodes, leaves, row_lens):
+    for r, n in enumerate(row_lens):
+        at = 0
+        for lo, hi in covered_tokens(nodes, leaves, r):
+            if hi == lo:
+                continue
+            assert lo == at, f"row {r}: gap or overlap at token {at} (next span starts at {lo})"
+            at = hi
+        assert at == n, f"row {r}: covered {at} tokens of {n}"
+
+
+def test_fresh_prefill_is_tiled_per_block():
+    # one sequence, 40 prompt tokens, nothing cached: blocks 0, 1 and half of block 2
+    table = [[7, 3, 9, 0]]
+    row_table, row_lens, row_group = run_rows([(0, 40)], max_blocks=4)
+    nodes, leaves = discover_forest(table, row_lens, row_table=row_table, row_group=row_group)
+    # tokens 16..31 share block 0, tokens 32..39 share blocks 0 and 1; tokens 0..15 share nothing
+    assert canonical_nodes(nodes) == sorted([(tuple(range(16, 32)), 0, 1), (tuple(range(32, 40)), 0, 2)])
+    assert [l["blk_start"] for l in leaves] == [0] * 16 + [1] * 16 + [2] * 8
+    assert [l["tokens"] for l in leaves] == list(range(1, 17)) * 2 + list(range(1, 9))
+    assert_exact_cover(nodes, leaves, row_lens)
+
+
+def test_chunked_prefill_continues_inside_a_block():
+    # 23 tokens cached, 30 more arrive: first tile is the rest of block 1 (tokens 23..31)
+    table = [[4, 5, 6, 8]]
+    row_table, row_lens, row_group = run_rows([(23, 30)], max_blocks=4)
+    nodes, leaves = discover_forest(table, row_lens, row_table=row_table, row_group=row_group)
+    assert canonical_nodes(nodes) == sorted(
+        [(tuple(range(0, 9)), 0, 1), (tuple(range(9, 25)), 0, 2), (tuple(range(25, 30)), 0, 3)]
+    )
+    assert_exact_cover(nodes, leaves, row_lens)
+
+
+def test_mixed_batch_keeps_discovery_for_single_tokens():
+    # sequences 0 and 1 decode one token each over a shared two-block prompt; sequence 2 is a prefill
+    table = [[1, 2, 10, 0], [1, 2, 11, 0], [20, 21, 22, 23]]
+    row_table, row_lens, row_group = run_rows([(36, 1), (40, 1), (0, 50)], max_blocks=4)
+    nodes, leaves = discover_forest(table, row_lens, row_table=row_table, row_group=row_group)
+    got = canonical_nodes(nodes)
+    assert ((0, 1), 0, 2) in got  # the decode rows share their prompt as before
+    assert (tuple(range(2 + 16, 2 + 32)), 0, 1) in got and (tuple(range(2 + 48, 2 + 50)), 0, 3) in got
+    assert_exact_cover(nodes, leaves, row_lens)
+
+
+def test_cover_invariant_on_random_batches():
+    rng = random.Random(5)
+    for _ in range(30):
+        nseq = rng.randint(1, 5)
+        max_blocks = 12
+        table = [[rng.randrange(1000) for _ in range(max_blocks)] for _ in range(nseq)]
+        if nseq > 1 and rng.random() < 0.5:  # two sequences with a common cached prompt
+            table[1][:3] = table[0][:3]
+        batch = []
+        for _ in range(nseq):
+            ql = rng.choice([1, 1, 2, 15, 16, 17, 33, 60])
+            ctx = rng.randint(48 if ql == 1 else 0, max_blocks * BLOCK - ql)
+            batch.append((ctx, ql))
+        row_table, row_lens, row_group = run_rows(batch, max_blocks, tile_min=rng.choice([2, 17]))
+        for levels in (1, 4):
+            nodes, leaves = discover_forest(table, row_lens, max_levels=levels, row_table=row_table, row_group=row_group)
+            assert_exact_cover(nodes, leaves, row_lens)
+            for n in nodes:  # the members of a node really hold the same blocks there
+                ids = {tuple(table[row_table[r]][n["blk_start"] : n["blk_start"] + n["num_blocks"]]) for r in n["members"]}
+                assert len(ids) == 1
+
+
+# ---------------------------------------------------------------------------------- GPU
+
+
+def _batch_on_gpu(gpu, seed, batch, hq, hkv, d, kv_dtype, share=()):
+    """Random cache and block tables for (context, query) pairs; ``share`` lists pairs of
+    sequences (a, b, blocks) whose first blocks are the same physical blocks."""
+    from arctic_platform_amd.kv_layout import kv_cache_shape
+
+    gen = torch.Generator().manual_seed(seed)
+    max_blocks = max((c + q + BLOCK - 1) // BLOCK for c, q in batch) + 1
+    nblocks = len(batch) * max_blocks + 3
+    perm = torch.randperm(nblocks, generator=gen).to(torch.int32)
+    table = perm[: len(batch) * max_blocks].view(len(batch), max_blocks).clone()
+    for a, b, n in share:
+        table[b, :n] = table[a, :n]
+    shape = kv_cache_shape(nblocks, BLOCK, hkv, d)
+    cache = torch.randn(shape, generator=gen)
+    k_scale = v_scale = None
+    if kv_dtype == torch.float8_e4m3fn:
+        k_scale = torch.rand(hkv, generator=gen) * 0.09 + 0.01
+        v_scale = torch.rand(hkv, generator=gen) * 0.09 + 0.01
+        cache = (cache * 20).clamp(-448, 448)
+    cache = cache.to(kv_dtype)
+    rows = sum(q for _, q in batch)
+    q = torch.randn(rows, hq, d, generator=gen).to(torch.bfloat16)
+    dev = lambda t: None if t is None else t.to(gpu)
+    return dev(table), dev(cache), dev(q), dev(k_scale), dev(v_scale), max_blocks
+
+
+CASES = [
+    # (seed, Hq, Hkv, D, kv dtype, rows per item, chunk, [(context, query)], shared prompts)
+    (1, 8, 2, 64, torch.bfloat16, 32, 64, [(0, 1), (0, 37), (0, 300), (23, 50), (100, 1), (64, 16)], ()),
+    (2, 32, 8, 128, torch.bfloat16, 64, 128, [(0, 200), (130, 70), (77, 1), (90, 1), (5, 3)], ((2, 3, 4),)),
+    (3, 16, 4, 128, torch.float8_e4m3fn, 64, 256, [(0, 129), (511, 33), (40, 1)], ()),
+    (4, 32, 4, 64, torch.bfloat16, 64, 32, [(16, 48), (0, 16), (15, 2)], ()),  # GQA 8: two row tiles per group
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", CASES, ids=[f"seed{c[0]}" for c in CASES])
+def test_query_runs_match_oracle(gpu, case):
+    from arctic_platform_amd.forest import build_forest_metadata
+    from arctic_platform_amd.ops import forest_cascade_decode
+    from oracle.attention import flat_decode_attention
+    from tests.helpers import assert_matches_oracle
+
+    seed, hq, hkv, d, kv_dtype, rows, chunk, batch, share = case
+    table, cache, q, k_scale, v_scale, max_blocks = _batch_on_gpu(gpu, seed, batch, hq, hkv, d, kv_dtype, share)
+    row_table, row_lens, row_group = run_rows(batch, max_blocks)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=gpu)
+    scale = d**-0.5
+    for levels in (4, 0):
+        md = build_forest_metadata(
+            table, i32(row_lens), num_q_heads=hq, num_kv_heads=hkv, head_dim=d, chunk_tokens=chunk, rows_per_item=rows,
+            max_levels=levels, row_table=i32(row_table), row_group=i32(row_group),
+        )
+        out, lse = forest_cascade_decode(q, cache, md, scale, k_scale, v_scale)
+        torch.cuda.synchronize()
+        md.check()
+        nodes, leaves = discover_forest(table.cpu().tolist(), row_lens, max_levels=levels, row_table=row_table, row_group=row_group)
+        assert canonical_nodes(md.nodes()) == canonical_nodes(nodes)
+        assert [l["tokens"] for l in md.leaves()] == [l["tokens"] for l in leaves]
+        # every item addresses the block table by table row
+        assert all(0 <= it["rep"] < len(batch) for it in md.items())
+        ref_out, ref_lse = flat_decode_attention(
+            q.cpu(), cache.cpu(), table.cpu()[torch.tensor(row_table)], torch.tensor(row_lens), scale,
+            None if k_scale is None else k_scale.cpu(), None if v_scale is None else v_scale.cpu(),
+        )
+        assert_matches_oracle(out, lse, ref_out, ref_lse, what=f"query runs {seed}, levels {levels}")
+
+
+@pytest.mark.gpu
+def test_bad_row_table_is_flagged_not_followed(gpu):
+    from arctic_platform_amd.forest import build_forest_metadata
+
+    table = torch.arange(8, dtype=torch.int32, device=gpu).view(2, 4)
+    lens = torch.tensor([5, 9, 20], dtype=torch.int32, device=gpu)
+    rows = torch.tensor([0, 7, 1], dtype=torch.int32, device=gpu)  # 7 is not a row of the table
+    md = build_forest_metadata(table, lens, num_q_heads=8, num_kv_heads=2, head_dim=64, row_table=rows)
+    torch.cuda.synchronize()
+    with pytest.raises(ValueError, match="row_table"):
+        md.check()
+
+
+@pytest.mark.gpu
+def test_prefill_and_decode_through_backend(gpu):
+    """A mixed step through the adapter: one sequence prefills 150 tokens, one continues a
+    chunked prefill, two decode; forward() writes the new K/V and attends."""
+    import types
+
+    from arctic_platform_amd.backend import CommonAttentionMetadata, ForestCascadeAttentionBackend
+    from oracle.attention import flat_decode_attention
+    from tests.helpers import assert_matches_oracle
+
+    hq, hkv, d = 16, 4, 128
+    batch = [(0, 150), (70, 40), (300, 1), (33, 1)]
+    table, cache, q, _, _, max_blocks = _batch_on_gpu(gpu, 11, batch, hq, hkv, d, torch.bfloat16)
+    builder = ForestCascadeAttentionBackend.get_builder_cls()(hq, hkv, d, device=gpu, forest_cascade_attn_configs='{"chunk_tokens": 64}')
+    impl = ForestCascadeAttentionBackend.get_impl_cls()(hq, d, d**-0.5, hkv)
+    qlens = torch.tensor([b[1] for b in batch])
+    starts = torch.cat([torch.zeros(1, dtype=torch.long), qlens.cumsum(0)]).to(torch.int32).to(gpu)
+    seq_lens = torch.tensor([c + n for c, n in batch], dtype=torch.int32, device=gpu)
+    row_table, row_lens, _ = run_rows(batch, max_blocks)
+    pos = torch.tensor(row_lens) - 1
+    slots = (table.cpu()[torch.tensor(row_table), pos // BLOCK].long() * BLOCK + pos % BLOCK).to(gpu)
+    gen = torch.Generator().manual_seed(12)
+    t = q.shape[0]
+    key = torch.randn(t, hkv * d, generator=gen).to(torch.bfloat16).to(gpu)
+    value = torch.randn(t, hkv * d, generator=gen).to(torch.bfloat16).to(gpu)
+    meta = builder.build(0, CommonAttentionMetadata(starts, seq_lens, table, slots, num_reqs=len(batch), max_query_len=150, num_actual_tokens=t))
+    out = impl.forward(types.SimpleNamespace(), q.view(t, hq * d), key, value, cache, meta)
+    torch.cuda.synchronize()
+    meta.forest.check()
+    ref_out, ref_lse = flat_decode_attention(q.cpu(), cache.cpu(), table.cpu()[torch.tensor(row_table)], torch.tensor(row_lens), d**-0.5)
+    got = out.view(t, hq, d)
+    assert_matches_oracle(got, ref_lse, ref_out, ref_lse, what="mixed step through the backend")
