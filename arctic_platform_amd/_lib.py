@@ -87,6 +87,8 @@ class FcaMetaLayout(ctypes.Structure):
             "max_items",
             "max_partials",
             "total_int32",
+            "node_tok",
+            "node_causal",
         )
     ]
 

@@ -177,6 +177,8 @@ int fca_meta_describe(const fca_plan* plan, fca_meta_layout* out) {
   out->max_items = L.max_items;
   out->max_partials = L.max_partials;
   out->total_int32 = L.total;
+  out->node_tok = L.node_tok;
+  out->node_causal = L.node_causal;
   return FCA_OK;
 }
 

@@ -109,7 +109,7 @@ __global__ __launch_bounds__(kThreads, kWorkgroupsPerCu<D>) void fca_attend64_ke
     const int4* rec =
         reinterpret_cast<const int4*>(meta + p.off_items + (int64_t)(first + it) * kItemInts + opaque_zero);
     r0 = rec[0];  // rep, blk_start, tok_len, member_off
-    r1 = rec[1];  // member_cnt, ord, node, -
+    r1 = rec[1];  // member_cnt, ord, node, tokens the first member sees (causal last chunk) or 0
   };
   // Per-lane data that hangs off a record: one block id of the chunk per lane (a chunk has
   // at most 64 blocks) and the member sequence of this lane's query row(s).
@@ -194,7 +194,11 @@ __global__ __launch_bounds__(kThreads, kWorkgroupsPerCu<D>) void fca_attend64_ke
       const bool two_tiles = rows > 32;
       const int nblk = (tok_len + kBlock - 1) / kBlock;
       const int ntiles = (tok_len + kTile - 1) / kTile;
-      const int nfull = tok_len / kTile;  // tiles with all 32 tokens live; at most one ragged tile follows
+      // Last chunk of a query-run tile: member i sees the first `sees + i` tokens of the chunk
+      // (its own token and what is before it).  All members end inside the last tile, which
+      // then takes the masking path even when the chunk fills it.
+      const int sees = __builtin_amdgcn_readfirstlane(r1.w);
+      const int nfull = (tok_len - (sees > 0 ? 1 : 0)) / kTile;  // tiles without masking; at most one masked tile follows
       const int last = ntiles - 1;
       int64_t prow[NRT];  // partial row this lane's query row is written to, -1 for a dead row
 #pragma unroll
@@ -261,9 +265,11 @@ __global__ __launch_bounds__(kThreads, kWorkgroupsPerCu<D>) void fca_attend64_ke
           }
           // register r holds token 16 * (r / 8) + 8 * h + r % 8 of the tile
           if constexpr (RAGGED) {
+            // every score register of a lane belongs to the lane's own query row
+            const int row_lim = sees > 0 ? min(tok_len, sees + row_member[rt]) : tok_len;
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-              if (tok0 + 16 * (r >> 3) + 8 * h + (r & 7) >= tok_len) sr[r] = -INFINITY;
+              if (tok0 + 16 * (r >> 3) + 8 * h + (r & 7) >= row_lim) sr[r] = -INFINITY;
           }
           float mx = sr[0];
 #pragma unroll

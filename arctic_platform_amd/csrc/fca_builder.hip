@@ -153,6 +153,8 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   int* slot = meta + L.s_slot;
   int* tmp0 = meta + L.s_tmp0;
   int* tmp1 = meta + L.s_tmp1;
+  int* cbad = meta + L.s_nitems;  // per leader: some member breaks the pattern of a query-run tile
+  int* cmax = cbad + S;           // per leader: largest member row minus the leader's row
   unsigned long long* hkeys = reinterpret_cast<unsigned long long*>(meta + L.hash_keys);
   int* hmin = meta + L.hash_min;
   const int hsize = (int)L.hash_size;
@@ -165,8 +167,13 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
     const int r = p.row_table[s];
     return r >= 0 && r < p.table_rows ? r : 0;  // (out of range: flagged by the full build)
   };
-  // rows the caller has grouped: the group's common run ends before the block that holds
-  // the last token of its shortest row, so every member keeps a leaf of its own
+  // Rows the caller has grouped.  The common run of a declared group ends before the block
+  // that holds the last token of its shortest row.  If the members are successive rows
+  // reading one table row, each one token longer than the one before it, with their last
+  // tokens in one block (a tile of a query run), the node takes that block in as well and
+  // is marked causal: its last chunk tells the attention kernel the first member's length,
+  // and the kernel hides from every row the tokens behind its own.  Such members have no
+  // leaf.  Any other declared group keeps a private leaf per member from that block on.
   auto declared = [&](int s) { return p.row_group && p.row_group[s] >= 0; };
 
   // ---- update: is the forest of the last build on this workspace still the forest of
@@ -238,16 +245,20 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
         cnt[s] = 0;
         leader[s] = -1;
         slot[s] = -1;
+        cbad[s] = 0;
+        cmax[s] = 0;
       }
       __syncthreads();
       // Key every sequence that still has a full block at its position.  A sequence whose
       // parent is -2 dropped out of sharing at an earlier level.
       for (int s = tid; s < S; s += kBuildThreads) {
-        if (par[s] == -2 || pos[s] >= nfull[s]) continue;
+        if (par[s] == -2) continue;
+        const bool by_id = level == 0 && declared(s);
+        if (by_id ? tmp1[s] < 1 : pos[s] >= nfull[s]) continue;
         // The key of a declared group (first level only) is its id; otherwise rows meet
         // under (parent node, physical block id at the current position).
         unsigned long long key;
-        if (level == 0 && declared(s)) {
+        if (by_id) {
           key = (1ull << 63) | (unsigned)p.row_group[s];
         } else {
           const unsigned blk = (unsigned)p.block_table[table_row(s) * p.bt_stride + pos[s]];
@@ -301,9 +312,16 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       }
       __syncthreads();
       for (int s = tid; s < S; s += kBuildThreads) {
-        if (leader[s] >= 0) {
-          atomicMin(&run[leader[s]], lcp[s]);
-          atomicAdd(&cnt[leader[s]], 1);
+        const int t = leader[s];
+        if (t >= 0) {
+          atomicMin(&run[t], lcp[s]);
+          atomicAdd(&cnt[t], 1);
+          if (level == 0 && declared(s)) {
+            const bool tile = table_row(s) == table_row(t) && tmp1[s] == tmp1[t] + (s - t) &&
+                              (tmp1[s] - 1) / kBlock == (tmp1[t] - 1) / kBlock;
+            if (!tile) atomicOr(&cbad[t], 1);
+            atomicMax(&cmax[t], s - t);
+          }
         }
       }
       __syncthreads();
@@ -320,15 +338,20 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       for (int s = tid; s < S; s += kBuildThreads) {
         if (leader[s] == s && cnt[s] >= 2) {
           const int id = node_base + tmp0[s];
+          // a tile of a query run: members s, s + 1, ... without a gap, all fitting the pattern
+          const bool causal = level == 0 && declared(s) && !cbad[s] && cmax[s] + 1 == cnt[s];
+          const int ntok = causal ? tmp1[s] + cnt[s] - 1 : run[s] * kBlock;
           meta[L.node_rep + id] = s;
           meta[L.node_blk + id] = pos[s];
-          meta[L.node_nblk + id] = run[s];
+          meta[L.node_nblk + id] = run[s] + (causal ? 1 : 0);
+          meta[L.node_tok + id] = ntok;
+          meta[L.node_causal + id] = causal ? 1 : 0;
           meta[L.node_level + id] = level;
           meta[L.node_moff + id] = member_base + nodeof[s];
           meta[L.node_mcnt + id] = cnt[s];
           meta[L.node_ord + id] = ord[s];
           tmp0[s] = id;
-          atomicAdd(&lds_tokens, (unsigned long long)run[s] * kBlock);
+          atomicAdd(&lds_tokens, (unsigned long long)ntok);
         }
       }
       __syncthreads();
@@ -346,7 +369,7 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       for (int s = tid; s < S; s += kBuildThreads) {
         const int t = leader[s];
         if (t >= 0 && cnt[t] >= 2) {
-          lcp[s] = run[t];  // advance amount, applied after the barrier (pos[t] is read by others)
+          lcp[s] = 1;  // advances past the node, after the barrier (pos[t] is read by others)
           par[s] = tmp0[t];
         } else {
           lcp[s] = 0;
@@ -355,8 +378,9 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       }
       __syncthreads();
       for (int s = tid; s < S; s += kBuildThreads) {
-        pos[s] += lcp[s];
-        ord[s] += num_chunks_for(lcp[s] * kBlock, chunk);
+        if (!lcp[s]) continue;
+        pos[s] += meta[L.node_nblk + par[s]];
+        ord[s] += num_chunks_for(meta[L.node_tok + par[s]], chunk);
       }
       node_base += new_nodes;
       member_base += new_members;
@@ -385,7 +409,7 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   // shared nodes [0, node_base), then leaf of sequence s at node_base + s.
   const int leaf_members = member_base;
   for (int s = tid; s < S; s += kBuildThreads) {
-    const int tokens = tmp1[s] - pos[s] * kBlock;
+    const int tokens = max(0, tmp1[s] - pos[s] * kBlock);  // (none below a causal node)
     meta[L.seq_leaf_blk + s] = pos[s];
     meta[L.seq_npart + s] = ord[s] + num_chunks_for(tokens, chunk);
     members[leaf_members + s] = s;
@@ -401,12 +425,15 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   // class in descending size order: the attention kernel deals the list to its waves in
   // alternating directions, which balances a descending list well.
   const int total_nodes = node_base + S;
-  auto node_fields = [&](int n, int& rep, int& blk, int& tokens, int& moff, int& mcnt, int& o) {
+  // first_len: length of the first member of a causal node, 0 for any other node
+  auto node_fields = [&](int n, int& rep, int& blk, int& tokens, int& moff, int& mcnt, int& o, int& first_len) {
+    first_len = 0;
     // (rep is what the attention kernels index the block table with)
     if (n < node_base) {
       rep = (int)table_row(meta[L.node_rep + n]);
       blk = meta[L.node_blk + n];
-      tokens = meta[L.node_nblk + n] * kBlock;
+      tokens = meta[L.node_tok + n];
+      if (meta[L.node_causal + n]) first_len = tmp1[meta[L.node_rep + n]];
       moff = meta[L.node_moff + n];
       mcnt = meta[L.node_mcnt + n];
       o = meta[L.node_ord + n];
@@ -414,7 +441,7 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       const int s = n - node_base;
       rep = (int)table_row(s);
       blk = pos[s];
-      tokens = tmp1[s] - pos[s] * kBlock;
+      tokens = max(0, tmp1[s] - pos[s] * kBlock);
       moff = leaf_members + s;
       mcnt = 1;
       o = ord[s];
@@ -425,8 +452,8 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
     return cls * kSizeBuckets + (kSizeBuckets - 1 - sb);
   };
   for (int n = tid; n < total_nodes; n += kBuildThreads) {
-    int rep, blk, tokens, moff, mcnt, o;
-    node_fields(n, rep, blk, tokens, moff, mcnt, o);
+    int rep, blk, tokens, moff, mcnt, o, first_len;
+    node_fields(n, rep, blk, tokens, moff, mcnt, o, first_len);
     const int clen = chunk_len_for(tokens, chunk);
     const int nch = num_chunks_for(tokens, chunk);
     const int ntile = (mcnt + members_per_item - 1) / members_per_item;
@@ -456,8 +483,8 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   __syncthreads();
   int32_t* items = meta + L.items;
   for (int n = tid; n < total_nodes; n += kBuildThreads) {
-    int rep, blk, tokens, moff, mcnt, o;
-    node_fields(n, rep, blk, tokens, moff, mcnt, o);
+    int rep, blk, tokens, moff, mcnt, o, first_len;
+    node_fields(n, rep, blk, tokens, moff, mcnt, o, first_len);
     const int clen = chunk_len_for(tokens, chunk);
     const int nch = num_chunks_for(tokens, chunk);
     const int ntile = (mcnt + members_per_item - 1) / members_per_item;
@@ -469,8 +496,12 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       for (int r = 0; r < ntile; ++r) {
         if (at + r >= (int)L.max_items) break;
         int4* rec = reinterpret_cast<int4*>(items + (int64_t)(at + r) * kItemInts);
+        // Last chunk of a causal node: tokens of the chunk the item's first member sees;
+        // member i of the item sees i more.  Every member's own block lies in the last tile
+        // of this chunk (chunks are whole tiles and a tile holds whole blocks).
+        const int sees = first_len && c == nch - 1 ? first_len + r * members_per_item - c * clen : 0;
         rec[0] = make_int4(rep, blk + c * (clen / kBlock), tl, moff + r * members_per_item);
-        rec[1] = make_int4(min(members_per_item, mcnt - r * members_per_item), o + c, n, 0);
+        rec[1] = make_int4(min(members_per_item, mcnt - r * members_per_item), o + c, n, sees);
       }
     }
   }

@@ -41,6 +41,8 @@ struct MetaLayout {
   int64_t header;
   int64_t seq_npart, seq_leaf_blk;
   int64_t node_rep, node_blk, node_nblk, node_level, node_moff, node_mcnt, node_ord;
+  int64_t node_tok;     // KV tokens of the node: blocks * 16, or up to its last member's token (causal node)
+  int64_t node_causal;  // 1: the members are successive tokens of one query run and the node includes their own block
   int64_t members;
   int64_t items;
   // builder scratch
@@ -77,6 +79,8 @@ inline __host__ MetaLayout make_layout(const fca_plan& p) {
   L.node_moff = take(S);
   L.node_mcnt = take(S);
   L.node_ord = take(S);
+  L.node_tok = take(S);
+  L.node_causal = take(S);
   L.members = take(S * (FCA_MAX_LEVELS + 1));
   L.items = take(L.max_items * kItemInts);
   L.s_pos = take(S);

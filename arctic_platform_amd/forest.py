@@ -80,6 +80,8 @@ class ForestMetadata:
                     rep=int(m[L.node_rep + i]),
                     blk_start=int(m[L.node_blk + i]),
                     num_blocks=int(m[L.node_nblk + i]),
+                    tokens=int(m[L.node_tok + i]),
+                    causal=bool(m[L.node_causal + i]),
                     level=int(m[L.node_level + i]),
                     ord=int(m[L.node_ord + i]),
                 )
@@ -91,7 +93,7 @@ class ForestMetadata:
         s = self.plan.num_seqs
         lens = self.seq_lens.cpu().tolist()
         blk = m[L.seq_leaf_blk : L.seq_leaf_blk + s].tolist()
-        return [dict(blk_start=blk[i], tokens=lens[i] - blk[i] * BLOCK_SIZE) for i in range(s)]
+        return [dict(blk_start=blk[i], tokens=max(0, lens[i] - blk[i] * BLOCK_SIZE)) for i in range(s)]
 
     def seq_num_partials(self) -> list:
         L = self.layout
@@ -113,6 +115,7 @@ class ForestMetadata:
                     members=members[r[3] : r[3] + r[4]].tolist(),
                     ord=r[5],
                     node=r[6],
+                    sees=r[7],
                     shared=i < shared,
                 )
             )

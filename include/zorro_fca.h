@@ -90,7 +90,9 @@ typedef struct fca_tensors {
 
 /* Offsets (in int32 units) of the arrays inside a built metadata workspace, for
  * inspection and tests.  Item records are 8 x int32:
- * {rep_seq, blk_start, tok_len, member_off, member_cnt, ord, node, 0}. */
+ * {rep_row, blk_start, tok_len, member_off, member_cnt, ord, node, sees}; rep_row is the
+ * block-table row the item reads, sees is 0 except in the last chunk of a causal node,
+ * where member i of the item attends to the first sees + i tokens of the chunk. */
 typedef struct fca_meta_layout {
   int64_t header;        /* [16]: 0 items, 1 shared items, 2 nodes (shared), 3 work ticket
                             (self-resetting, owned by the attention kernel), 4 reserved,
@@ -112,6 +114,9 @@ typedef struct fca_meta_layout {
   int64_t max_items;
   int64_t max_partials;  /* partial slots reserved per sequence */
   int64_t total_int32;
+  int64_t node_tok;      /* [S] KV tokens of the node: num blocks * 16, or, for a causal node, up to
+                            the last token of its last member */
+  int64_t node_causal;   /* [S] 1: the node is a tile of a query run (fca_build_metadata_rows) */
 } fca_meta_layout;
 
 int fca_version(void);
@@ -155,9 +160,13 @@ int fca_update_metadata(const fca_plan* plan, const int32_t* block_table_dev, in
  * the block holding the last token of the group's shortest row (rows of one table row are
  * not compared, others are, so a wrong declaration costs sharing, never correctness).
  * Declared groups are how a long run is tiled: the tokens of one 16-token block form a
- * group, read the KV before their block once for all of them, and each reads its own
- * block alone.  Rows with -1 are grouped by discovery as in fca_build_metadata, and
- * declared groups take part in discovery below their node.  update != 0 asks for the
+ * group.  When the members of a group are successive rows over one table row, each one
+ * token longer than the one before it and all ending in one block, the node takes that
+ * block in as well (a causal node): the group reads all its KV once, the kernels hide from
+ * every row the tokens behind its own, and the rows have no private part.  Other declared
+ * groups read the KV before that block once and each row reads the rest alone.  Rows with
+ * -1 are grouped by discovery as in fca_build_metadata, and declared groups that are not
+ * causal take part in discovery below their node.  update != 0 asks for the
  * update of fca_update_metadata.  The attention calls then take the [table_rows,
  * max_blocks] block table and kv_reread = 1.  Counterpart in the reference: the
  * response-over-shared-prompt attention of the trainer, which rebuilds full sequences from

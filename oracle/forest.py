@@ -16,8 +16,11 @@ Query rows need not be block-table rows: with ``row_table`` query row r reads ta
 ``row_table[r]`` up to ``seq_lens[r]`` tokens (the tokens of a query run).  ``row_group``
 declares first-level groups among such rows in place of the block-id comparison; for a
 declared row the last block it may share is the one before the block that holds its last
-token, so every member of a declared group keeps a private leaf (this is the tiling of a
-long run: the tokens of one block form a group).  The trainer's counterpart is the
+token.  A declared group whose members are successive rows over one table row, each one
+token longer than the one before it and all ending in one block, is a tile of a query run:
+its node takes that block in too, holds ``tokens`` = the last member's length, is marked
+``causal`` (each member attends only up to its own token) and leaves its members no leaf.
+Members of any other declared group keep a private leaf from that block on.  The trainer's counterpart is the
 response-over-shared-prompt attention, which reads each unique prompt once for all its
 responses (arctic_platform/rl/zorro_train/qwen_attention_patcher.py:1117-1262).
 """
@@ -32,8 +35,8 @@ BLOCK = 16
 def discover_forest(block_table, seq_lens, block_size=BLOCK, max_levels=8, row_table=None, row_group=None):
     """Returns (nodes, leaves).
 
-    nodes: list of dict(members, blk_start, num_blocks, level, parent) for shared runs.
-    leaves: per sequence dict(blk_start, tokens, parent): the private remainder.
+    nodes: list of dict(members, blk_start, num_blocks, tokens, causal, level, parent) for
+    shared runs.  leaves: per sequence dict(blk_start, tokens, parent): the private remainder.
     """
     table = [list(map(int, row)) for row in block_table]
     lens = [int(n) for n in seq_lens]
@@ -49,9 +52,11 @@ def discover_forest(block_table, seq_lens, block_size=BLOCK, max_levels=8, row_t
             return
         groups = OrderedDict()
         for s in members:
-            if pos < nfull[s]:
-                key = ("declared", group_of[s]) if level == 0 and group_of[s] >= 0 else bt[s][pos]
-                groups.setdefault(key, []).append(s)
+            if level == 0 and group_of[s] >= 0:
+                if lens[s] >= 1:
+                    groups.setdefault(("declared", group_of[s]), []).append(s)
+            elif pos < nfull[s]:
+                groups.setdefault(bt[s][pos], []).append(s)
         for group in groups.values():
             if len(group) < 2:
                 continue
@@ -60,16 +65,31 @@ def discover_forest(block_table, seq_lens, block_size=BLOCK, max_levels=8, row_t
             run = 0
             while run < limit and all(bt[s][pos + run] == bt[first][pos + run] for s in group):
                 run += 1
+            tokens, causal = run * block_size, False
+            if level == 0 and group_of[first] >= 0:
+                trow = (lambda s: s) if row_table is None else (lambda s: int(row_table[s]))
+                causal = all(
+                    s == first + i
+                    and trow(s) == trow(first)
+                    and lens[s] == lens[first] + i
+                    and (lens[s] - 1) // block_size == (lens[first] - 1) // block_size
+                    for i, s in enumerate(group)
+                )
+                if causal:
+                    run, tokens = run + 1, lens[group[-1]]
             node_id = len(nodes)
-            nodes.append(dict(members=list(group), blk_start=pos, num_blocks=run, level=level, parent=parent))
+            nodes.append(
+                dict(members=list(group), blk_start=pos, num_blocks=run, tokens=tokens, causal=causal, level=level, parent=parent)
+            )
             for s in group:
                 leaf_start[s] = pos + run
                 leaf_parent[s] = node_id
-            descend(group, pos + run, level + 1, node_id)
+            if not causal:
+                descend(group, pos + run, level + 1, node_id)
 
     descend(list(range(len(lens))), 0, 0, -1)
     leaves = [
-        dict(blk_start=leaf_start[s], tokens=lens[s] - leaf_start[s] * block_size, parent=leaf_parent[s])
+        dict(blk_start=leaf_start[s], tokens=max(0, lens[s] - leaf_start[s] * block_size), parent=leaf_parent[s])
         for s in range(len(lens))
     ]
     return nodes, leaves
@@ -97,4 +117,4 @@ def canonical_nodes(nodes):
 
 
 def unique_tokens(nodes, leaves, block_size=BLOCK):
-    return sum(n["num_blocks"] * block_size for n in nodes) + sum(l["tokens"] for l in leaves)
+    return sum(n.get("tokens", n["num_blocks"] * block_size) for n in nodes) + sum(l["tokens"] for l in leaves)

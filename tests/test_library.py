@@ -31,7 +31,7 @@ def test_exports_every_declared_symbol(lib):
 
 def test_struct_sizes_match_header():
     assert ctypes.sizeof(_lib.FcaPlan) == 9 * 4
-    assert ctypes.sizeof(_lib.FcaMetaLayout) == 15 * 8
+    assert ctypes.sizeof(_lib.FcaMetaLayout) == 17 * 8
     assert ctypes.sizeof(_lib.FcaTensors) == 104
 
 

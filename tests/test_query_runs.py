@@ -1,8 +1,9 @@
 """Query runs: several query tokens per sequence (prefill chunks, mixed batches).
 
 One query row per token over the sequence's block-table row; long runs are tiled by
-declaring the tokens of one cache block a group.  CPU tests pin the forest oracle's
-handling of declared groups by coverage invariants and a hand-built case; GPU tests
+declaring the tokens of one cache block a group, which becomes a causal node: the group
+reads its KV once and every row stops at its own token.  CPU tests pin the forest oracle's
+handling of declared groups by coverage invariants and hand-built cases; GPU tests
 compare the kernels with the flat fp64 oracle row by row.
 """
 
@@ -30,9 +31,16 @@ def run_rows(ctx_and_query, max_blocks, tile_min=2):
     return row_table, row_lens, row_group
 
 
-def covered_tokens(nodes, leaves, row):
-    """Token ranges a row reads through its shared nodes and its leaf, as a sorted list."""
-    spans = [(n["blk_start"] * BLOCK, (n["blk_start"] + n["num_blocks"]) * BLOCK) for n in nodes if row in n["members"]]
+def covered_tokens(nodes, leaves, row, row_len):
+    """Token ranges a row reads through its shared nodes and its leaf, as a sorted list.  A
+    causal node ends, for each member, at the member's own last token."""
+    spans = []
+    for n in nodes:
+        if row in n["members"]:
+            end = n["blk_start"] * BLOCK + n["tokens"]
+            assert n["causal"] or n["tokens"] == n["num_blocks"] * BLOCK
+            assert not n["causal"] or (n["num_blocks"] - 1) * BLOCK < n["tokens"] <= n["num_blocks"] * BLOCK
+            spans.append((n["blk_start"] * BLOCK, min(end, row_len) if n["causal"] else end))
     leaf = leaves[row]
     spans.append((leaf["blk_start"] * BLOCK, leaf["blk_start"] * BLOCK + leaf["tokens"]))
     return sorted(spans)
@@ -41,7 +49,7 @@ def covered_tokens(nodes, leaves, row):
 def assert_exact_cover(nodes, leaves, row_lens):
     for r, n in enumerate(row_lens):
         at = 0
-        for lo, hi in covered_tokens(nodes, leaves, r):
+        for lo, hi in covered_tokens(nodes, leaves, r, n):
             if hi == lo:
                 continue
             assert lo == at, f"row {r}: gap or overlap at token {at} (next span starts at {lo})"
@@ -54,10 +62,12 @@ def test_fresh_prefill_is_tiled_per_block():
     table = [[7, 3, 9, 0]]
     row_table, row_lens, row_group = run_rows([(0, 40)], max_blocks=4)
     nodes, leaves = discover_forest(table, row_lens, row_table=row_table, row_group=row_group)
-    # tokens 16..31 share block 0, tokens 32..39 share blocks 0 and 1; tokens 0..15 share nothing
-    assert canonical_nodes(nodes) == sorted([(tuple(range(16, 32)), 0, 1), (tuple(range(32, 40)), 0, 2)])
-    assert [l["blk_start"] for l in leaves] == [0] * 16 + [1] * 16 + [2] * 8
-    assert [l["tokens"] for l in leaves] == list(range(1, 17)) * 2 + list(range(1, 9))
+    # one causal node per block of the run, holding everything up to the tile's last token
+    assert canonical_nodes(nodes) == sorted(
+        [(tuple(range(0, 16)), 0, 1), (tuple(range(16, 32)), 0, 2), (tuple(range(32, 40)), 0, 3)]
+    )
+    assert sorted(n["tokens"] for n in nodes) == [16, 32, 40] and all(n["causal"] for n in nodes)
+    assert [l["tokens"] for l in leaves] == [0] * 40
     assert_exact_cover(nodes, leaves, row_lens)
 
 
@@ -67,9 +77,26 @@ def test_chunked_prefill_continues_inside_a_block():
     row_table, row_lens, row_group = run_rows([(23, 30)], max_blocks=4)
     nodes, leaves = discover_forest(table, row_lens, row_table=row_table, row_group=row_group)
     assert canonical_nodes(nodes) == sorted(
-        [(tuple(range(0, 9)), 0, 1), (tuple(range(9, 25)), 0, 2), (tuple(range(25, 30)), 0, 3)]
+        [(tuple(range(0, 9)), 0, 2), (tuple(range(9, 25)), 0, 3), (tuple(range(25, 30)), 0, 4)]
     )
+    assert sorted(n["tokens"] for n in nodes) == [32, 48, 53]
     assert_exact_cover(nodes, leaves, row_lens)
+
+
+def test_declared_group_that_is_no_tile_keeps_private_leaves():
+    # two sequences over one cached prompt of three blocks, declared a group by the caller
+    table = [[1, 2, 3, 10], [1, 2, 3, 11]]
+    nodes, leaves = discover_forest(table, [52, 60], row_table=[0, 1], row_group=[5, 5])
+    assert canonical_nodes(nodes) == [((0, 1), 0, 3)] and not nodes[0]["causal"] and nodes[0]["tokens"] == 48
+    assert [l["tokens"] for l in leaves] == [4, 12]
+    # same rows, but the shorter one ends inside the third block: that block stays private
+    nodes, leaves = discover_forest(table, [40, 60], row_table=[0, 1], row_group=[5, 5])
+    assert canonical_nodes(nodes) == [((0, 1), 0, 2)]
+    assert [l["tokens"] for l in leaves] == [8, 28]
+    # one table row, lengths that are not successive: no tile either
+    nodes, leaves = discover_forest([[1, 2, 3, 4]], [50, 52], row_table=[0, 0], row_group=[0, 0])
+    assert canonical_nodes(nodes) == [((0, 1), 0, 3)] and not nodes[0]["causal"]
+    assert_exact_cover(nodes, leaves, [50, 52])
 
 
 def test_mixed_batch_keeps_discovery_for_single_tokens():
@@ -79,7 +106,7 @@ def test_mixed_batch_keeps_discovery_for_single_tokens():
     nodes, leaves = discover_forest(table, row_lens, row_table=row_table, row_group=row_group)
     got = canonical_nodes(nodes)
     assert ((0, 1), 0, 2) in got  # the decode rows share their prompt as before
-    assert (tuple(range(2 + 16, 2 + 32)), 0, 1) in got and (tuple(range(2 + 48, 2 + 50)), 0, 3) in got
+    assert (tuple(range(2 + 16, 2 + 32)), 0, 2) in got and (tuple(range(2 + 48, 2 + 50)), 0, 4) in got
     assert_exact_cover(nodes, leaves, row_lens)
 
 
@@ -166,6 +193,8 @@ def test_query_runs_match_oracle(gpu, case):
         md.check()
         nodes, leaves = discover_forest(table.cpu().tolist(), row_lens, max_levels=levels, row_table=row_table, row_group=row_group)
         assert canonical_nodes(md.nodes()) == canonical_nodes(nodes)
+        by_members = lambda ns: sorted((tuple(n["members"]), n["tokens"], n["causal"]) for n in ns)
+        assert by_members(md.nodes()) == by_members(nodes)
         assert [l["tokens"] for l in md.leaves()] == [l["tokens"] for l in leaves]
         # every item addresses the block table by table row
         assert all(0 <= it["rep"] < len(batch) for it in md.items())
@@ -174,6 +203,35 @@ def test_query_runs_match_oracle(gpu, case):
             None if k_scale is None else k_scale.cpu(), None if v_scale is None else v_scale.cpu(),
         )
         assert_matches_oracle(out, lse, ref_out, ref_lse, what=f"query runs {seed}, levels {levels}")
+
+
+@pytest.mark.gpu
+def test_declared_groups_that_are_no_tiles(gpu):
+    """Groups the caller declares across table rows (an explicit tree spec) and groups whose
+    lengths do not form a run: shared node before the members' own blocks, private leaves."""
+    from arctic_platform_amd.forest import build_forest_metadata
+    from arctic_platform_amd.ops import forest_cascade_decode
+    from oracle.attention import flat_decode_attention
+    from tests.helpers import assert_matches_oracle
+
+    hq, hkv, d = 8, 2, 64
+    batch = [(50, 1), (70, 1), (90, 1), (10, 9)]
+    table, cache, q, _, _, max_blocks = _batch_on_gpu(gpu, 21, batch, hq, hkv, d, torch.bfloat16, share=((0, 1, 3), (0, 2, 3)))
+    row_table = [0, 1, 2] + [3] * 9
+    row_lens = [51, 71, 91] + [11, 13, 12, 14, 15, 16, 17, 18, 19]  # two rows of the run swapped
+    row_group = [4, 4, 4] + [9] * 9
+    q = q[: len(row_table)]
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=gpu)
+    md = build_forest_metadata(table, i32(row_lens), num_q_heads=hq, num_kv_heads=hkv, head_dim=d, chunk_tokens=32, row_table=i32(row_table), row_group=i32(row_group))
+    out, lse = forest_cascade_decode(q, cache, md, d**-0.5)
+    torch.cuda.synchronize()
+    md.check()
+    nodes, leaves = discover_forest(table.cpu().tolist(), row_lens, max_levels=4, row_table=row_table, row_group=row_group)
+    assert canonical_nodes(md.nodes()) == canonical_nodes(nodes)
+    assert ((0, 1, 2), 0, 3) in canonical_nodes(nodes) and not any(n["causal"] for n in md.nodes())
+    assert [l["tokens"] for l in md.leaves()] == [l["tokens"] for l in leaves]
+    ref_out, ref_lse = flat_decode_attention(q.cpu(), cache.cpu(), table.cpu()[torch.tensor(row_table)], torch.tensor(row_lens), d**-0.5)
+    assert_matches_oracle(out, lse, ref_out, ref_lse, what="declared groups that are no tiles")
 
 
 @pytest.mark.gpu
