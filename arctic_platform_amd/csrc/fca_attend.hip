@@ -54,7 +54,7 @@ namespace fca {
 // first tile are requested before the current item's partial is written out, so the
 // memory pipe does not drain at item boundaries.
 template <int D, bool FP8, bool STREAM>
-__global__ __launch_bounds__(kThreads, kWorkgroupsPerCu<D>) void fca_attend64_kernel(AttendParams p) {
+__global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 64)) void fca_attend64_kernel(AttendParams p) {
   constexpr int NRT = 2;       // row tiles of 32 query rows
   constexpr int KS = D / 16;   // MFMA steps of the score product
   constexpr int NDB = D / 32;  // 32-channel blocks of the output
@@ -434,13 +434,13 @@ hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dty
   const bool fp8 = kv_dtype == FCA_FP8_E4M3;
   const int nrt = plan.rows_per_item / 32;
   // Four independent waves per workgroup.  At head size 128 a wave uses the whole register
-  // file of its SIMD, so one workgroup per CU; at head size 64 two fit, and the second
-  // wave per SIMD hides the arithmetic latency of a tile, which is what limits a head that
-  // small (fp8 most of all).
+  // file of its SIMD, so one workgroup per CU; at head size 64 two fit (32-row bf16 aside),
+  // and the second wave per SIMD hides the arithmetic latency of a tile, which is what
+  // limits a head that small (fp8 most of all).
   const int64_t max_tickets = (int64_t)plan.num_seqs *
                               ((int64_t)plan.max_blocks * kBlock / plan.chunk_tokens + plan.max_levels + 1) *
                               plan.num_kv_heads;
-  int grid = cached_cu_count() * (plan.head_dim == 64 ? kWorkgroupsPerCu<64> : kWorkgroupsPerCu<128>);
+  int grid = cached_cu_count() * workgroups_per_cu(plan.head_dim, fp8, plan.rows_per_item);
   if ((int64_t)grid * kWaves > max_tickets) grid = (int)((max_tickets + kWaves - 1) / kWaves);
   if (grid < 1) grid = 1;
   if (nrt == 1) return launch_attend32(p, plan, kv_dtype, grid, stream);

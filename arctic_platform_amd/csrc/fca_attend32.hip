@@ -22,7 +22,7 @@
 namespace fca {
 
 template <int D, bool FP8, bool STREAM>
-__global__ __launch_bounds__(kThreads, kWorkgroupsPerCu<D>) void fca_attend32_kernel(AttendParams p) {
+__global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_attend32_kernel(AttendParams p) {
   constexpr int KS = D / 16;   // MFMA steps of the score product
   constexpr int NDB = D / 32;  // 32-channel blocks of the output
   using KT = KTile<D, FP8>;

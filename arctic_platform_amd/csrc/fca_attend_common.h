@@ -14,9 +14,13 @@ typedef int i32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
-// Workgroups a CU holds at once: a wave's register budget is 512 / this.
-template <int D>
-constexpr int kWorkgroupsPerCu = D == 64 ? 2 : 1;
+// Workgroups a CU holds at once: a wave's register budget is 512 / this.  Two where the
+// kernel fits 256 registers without scratch and gains from the second wave per SIMD: head
+// size 64 with 64-row tiles or fp8.  (The 32-row bf16 kernel at head size 64 would need two
+// registers of scratch and gains under 2 %.)
+constexpr int workgroups_per_cu(int head_dim, bool fp8, int rows_per_item) {
+  return head_dim == 64 && (fp8 || rows_per_item == 64) ? 2 : 1;
+}
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 constexpr float kRescaleSlack = 8.f;  // log2 units: rescale when a row maximum rises by more than 2^8
