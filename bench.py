@@ -44,6 +44,8 @@ def parse_args():
     ap.add_argument("--skip-noncascade", action="store_true")
     ap.add_argument("--split-passes", action="store_true", help="also time the shared-prefix pass and the suffix pass as launches of their own (and leave them in the trace for the profiler)")
     ap.add_argument("--calibrate", action="store_true", help="also run the library's plain copy kernel over 1 GiB (counter yardstick)")
+    ap.add_argument("--query-runs", default="", metavar="NxL", help="instead of a decode configuration: N sequences that each bring a run of L query tokens (a prefill chunk), e.g. 4x2048")
+    ap.add_argument("--context", type=int, default=0, help="tokens already cached in front of every query run")
     return ap.parse_args()
 
 
@@ -109,6 +111,13 @@ def cpu_baseline(torch, w, nseq):
         times.append(time.perf_counter() - t0)
     sample_s = median(times[1:]) if len(times) > 1 else times[0]
     scale_up = float(w.seq_lens.sum()) / float(lens.sum())
+    # for context: the same sample through the CPU restatement of the cascade (shared nodes
+    # read once for all their members, then the merge), discovery included
+    from oracle.cascade import cascade_decode_attention
+
+    t0 = time.perf_counter()
+    cascade_decode_attention(q, cache, table, lens, w.scale, ks, vs, dtype=torch.float32)
+    cascade_s = time.perf_counter() - t0
     return {
         "value": sample_s * scale_up * 1e6,
         "unit": "us/step",
@@ -116,13 +125,108 @@ def cpu_baseline(torch, w, nseq):
         "kind": "port",
         "sample": f"first {nseq} of {w.num_seqs} sequences ({int(lens.sum())} of {int(w.seq_lens.sum())} gathered tokens), "
         f"flat fp32 attention on torch-CPU, {sample_s:.2f} s measured, scaled by tokens x{scale_up:.2f}",
+        "cascade_restatement_us": cascade_s * scale_up * 1e6,
     }
+
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def main_query_runs(args):
+    """Prefill-shaped work on the same kernels: every sequence brings a run of query tokens;
+    one query row per token, the tokens of one cache block form a causal node.  A step is
+    one layer's attention call over all rows; flops are counted causally."""
+    import torch
+
+    from arctic_platform_amd import ops
+    from arctic_platform_amd.forest import build_forest_metadata
+    from arctic_platform_amd.kv_layout import kv_cache_shape
+    from oracle.attention import flat_decode_attention
+
+    nseq, ql = (int(v) for v in args.query_runs.lower().split("x"))
+    ctx, hq, hkv, d = args.context, 32, 8, 128
+    dev = torch.device("cuda:0")
+    gen = torch.Generator().manual_seed(4242)
+    max_blocks = (ctx + ql + 15) // 16
+    table = torch.randperm(nseq * max_blocks, generator=gen).to(torch.int32).view(nseq, max_blocks).to(dev)
+    caches = [torch.randn(kv_cache_shape(nseq * max_blocks, 16, hkv, d), generator=gen).to(torch.bfloat16).to(dev)]
+    caches += [caches[0].clone() for _ in range(max(1, args.kv_copies) - 1)]
+    rows_total = nseq * ql
+    q = torch.randn(rows_total, hq, d, generator=gen).to(torch.bfloat16).to(dev)
+    seq = torch.arange(nseq, device=dev).repeat_interleave(ql)
+    lens = (ctx + 1 + torch.arange(ql, device=dev).repeat(nseq)).to(torch.int32)
+    row_table = seq.to(torch.int32)
+    row_group = (seq * max_blocks + (lens - 1) // 16).to(torch.int32)
+    chunk, rows = args.chunk or 1024, args.rows or 64
+    kw = dict(num_q_heads=hq, num_kv_heads=hkv, head_dim=d, chunk_tokens=chunk, rows_per_item=rows, row_table=row_table, row_group=row_group)
+    md = build_forest_metadata(table, lens, **kw)
+    torch.cuda.synchronize()
+    md.check()
+    out = torch.empty_like(q)
+    scale = d**-0.5
+
+    def step(i, events=None):
+        cache = caches[i % len(caches)]
+        if i % args.layers == 0:
+            build_forest_metadata(table, lens, out=md, **kw)
+            if events is not None:
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                ops.forest_pass(q, cache, md, scale)
+                b.record()
+                ops.merge_partials(md, q, out=out, return_lse=False)
+                events.append((a, b))
+                return
+        ops.forest_cascade_decode(q, cache, md, scale, out=out, return_lse=False)
+
+    steps, warmup = min(args.steps, 144), min(args.warmup, 36)
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    events = []
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i, events)
+    torch.cuda.synchronize()
+    step_us = (time.perf_counter() - t0) / steps * 1e6
+    kern = sum(a.elapsed_time(b) * 1e3 for a, b in events) / len(events)
+    flops = 4.0 * d * hq * float(lens.double().sum())
+
+    # CPU baseline and a parity spot check on a sample of rows
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    torch.set_num_threads(cores)
+    sample = list(range(0, rows_total, max(1, rows_total // 256)))[:256]
+    idx = torch.tensor(sample)
+    t0 = time.perf_counter()
+    ref_out, _ = flat_decode_attention(q[idx.to(dev)].cpu(), caches[0].cpu(), table.cpu()[row_table.cpu()[idx].long()], lens.cpu()[idx], scale, dtype=torch.float32)
+    cpu_s = time.perf_counter() - t0
+    err = float((out[idx.to(dev)].cpu().float() - ref_out).abs().max())
+    scale_up = float(lens.double().sum()) / float(lens.cpu()[idx].double().sum())
+    hdr = md.header()
+    print(json.dumps({
+        "metric": "query-run (prefill) attention µs/step, causal, Qwen3-4B heads",
+        "value": round(step_us, 2), "unit": "us/step", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(step_us / 1e3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 MFMA / f32 accumulate", "data": "synthetic",
+        "config": {"workload": f"{nseq} sequences x {ql} query tokens after {ctx} cached, Hq {hq} / Hkv {hkv} / D {d}, bf16, one causal node per cache block of a run",
+                   "query_rows": rows_total, "chunk_tokens": chunk, "rows_per_item": rows, "work_items": hdr["items"],
+                   "layers_per_metadata_build": args.layers, "causal_flops": flops},
+        "roofline": {"kernel": "fca_attend64_kernel" if rows == 64 else "fca_attend32_kernel", "bound": "mfma",
+                     "achieved": round(flops / kern / 1e6, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(flops / kern / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None, "launches_timed": len(events)},
+        "breakdown_us": {"attention_kernel": round(kern, 2)},
+        "cpu_baseline": {"value": cpu_s * scale_up * 1e6, "unit": "us/step", "cores": cores, "kind": "port",
+                         "sample": f"{len(sample)} of {rows_total} query rows, flat fp32 attention on torch-CPU, {cpu_s:.2f} s measured, scaled by gathered tokens x{scale_up:.1f}"},
+        "max_abs_err_vs_oracle_sample": err,
+    }))
 
 
 def main():
     args = parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path uses no collectives and the boxes have one GPU; run with --gpus 1")
+    if args.query_runs:
+        return main_query_runs(args)
     import torch
 
     from arctic_platform_amd import ops
