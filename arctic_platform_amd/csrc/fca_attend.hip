@@ -7,10 +7,10 @@
 // Work item = (node chunk, tile of members) x KV head.  Every wavefront is its own worker:
 // it walks its share of the size-ordered work list, streams each chunk's 32-token tiles
 // with private online-softmax state and writes one normalised partial per item.  There is
-// no workgroup barrier.  The kernel runs one wave per SIMD with the whole 512-entry
-// register file: registers, not LDS, are the staging buffer for K and V, because the cache
-// already stores tiles in MFMA operand order and a tile in flight needs a place to land
-// either way.
+// no workgroup barrier.  At head size 128 the kernels run one wave per SIMD with the whole
+// 512-entry register file (two waves where a smaller head leaves room): registers, not
+// LDS, are the staging buffer for K and V, because the cache already stores tiles in MFMA
+// operand order and a tile in flight needs a place to land either way.
 //
 // Per tile and wave, with tokens on the MFMA M dimension (the transposed product):
 //   St[32 tok x 32 rows] = K[32 x D] . Qt[D x 32]       D/16 x mfma_f32_32x32x16_bf16
@@ -21,6 +21,11 @@
 // orders of these two products: every operand is one contiguous 16-byte global load per
 // lane.  The K rows are fed in the token order that makes the softmax output registers
 // line up with the B operand of the second product, so P never leaves registers.
+//
+// Query runs (several query tokens of one sequence, one query row each) need a mask only
+// where a tile of such rows meets its own tokens: the last tile of the last chunk of a
+// causal node, where the item record says how many tokens the first member sees and every
+// further member sees one more.  Everything else is the unmasked decode product.
 //
 // Semantics (softmax scale, GQA head mapping h -> h / (Hq/Hkv), no mask for the decode
 // token) follow arctic_platform/model/implementations/qwen35/models/qwen3_5_moe/
