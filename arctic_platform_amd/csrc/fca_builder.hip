@@ -83,38 +83,105 @@ __device__ inline unsigned long long mix64(unsigned long long k) {
   return k;
 }
 
-// Fingerprint of the first n block ids of a row, computed by a group of 16 lanes (every
-// lane returns it): the sum over positions j of (id_j ^ c) * w_j in 64 bits, with an odd
-// 32-bit weight per position.  A change of one id moves the sum by a non-zero multiple of
-// an odd number, an exchange of two ids by a product of two non-zero numbers below 2^32:
-// neither can be zero modulo 2^64.  One multiply-add per element, eight loads in
-// flight per lane.
+// Lanes that work on one row together (row comparison, fingerprints).
+constexpr int kRowLanes = 8;
+
+// Fingerprint of the first n block ids of a row, computed by a group of kRowLanes lanes
+// (every lane returns it): the sum over positions j of (id_j ^ c) * w_j in 64 bits, with an
+// odd 32-bit weight per position.  A change of one id moves the sum by a non-zero multiple
+// of an odd number, an exchange of two ids by a product of two non-zero numbers below 2^32:
+// neither can be zero modulo 2^64.  One multiply-add per element.  A 16-byte aligned row is
+// read four ids per load, eight loads in flight per lane (256 positions per round trip of
+// the group); loads past the end are clamped and not counted.
 __device__ inline unsigned long long row_fingerprint(const int32_t* row, int n, int glane) {
   unsigned long long acc = 0;
-  constexpr int kUnroll = 8;  // 128 positions per round trip of the group
+  constexpr int kUnroll = 8;
   auto term = [](int id, unsigned j) {
     return (unsigned long long)((unsigned)id ^ 0xa5a5a5a5u) * ((j * 0x9e3779b1u) | 1u);
   };
-  int j0 = 0;
-  for (; j0 + 16 * kUnroll <= n; j0 += 16 * kUnroll) {
-    int v[kUnroll];
+  int done = 0;  // positions covered by the vector part
+  if ((reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+    const int4* row4 = reinterpret_cast<const int4*>(row);
+    const int nv = n >> 2;
+    for (int j0 = 0; j0 < nv; j0 += kRowLanes * kUnroll) {
+      int4 v[kUnroll];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) v[u] = row[j0 + u * 16 + glane];
+      for (int u = 0; u < kUnroll; ++u) v[u] = row4[min(j0 + u * kRowLanes + glane, nv - 1)];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) acc += term(v[u], (unsigned)(j0 + u * 16 + glane));
+      for (int u = 0; u < kUnroll; ++u) {
+        const int j = j0 + u * kRowLanes + glane;
+        if (j < nv)
+          acc += term(v[u].x, 4u * j) + term(v[u].y, 4u * j + 1) + term(v[u].z, 4u * j + 2) + term(v[u].w, 4u * j + 3);
+      }
+    }
+    done = nv << 2;
   }
-  if (j0 < n) {  // the rest in one round trip: loads past the end are clamped and not counted
+  for (int j0 = done; j0 < n; j0 += kRowLanes * kUnroll) {
     int v[kUnroll];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) v[u] = row[min(j0 + u * 16 + glane, n - 1)];
+    for (int u = 0; u < kUnroll; ++u) v[u] = row[min(j0 + u * kRowLanes + glane, n - 1)];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-      const int j = j0 + u * 16 + glane;
+      const int j = j0 + u * kRowLanes + glane;
       if (j < n) acc += term(v[u], (unsigned)j);
     }
   }
-  for (int off = 8; off; off >>= 1) acc += __shfl_xor(acc, off, 16);
+  for (int off = kRowLanes / 2; off; off >>= 1) acc += __shfl_xor(acc, off, kRowLanes);
   return acc;
+}
+
+// First position below lim at which two rows differ (lim if none), found by a group of
+// kRowLanes lanes; every lane returns it.  Where both rows are 16-byte aligned together
+// they are compared four ids per load, eight loads per row in flight per lane (256
+// positions per round trip of the group), and the scan stops at the first round that holds
+// a difference.
+__device__ inline int first_difference(const int32_t* a, const int32_t* b, int lim, int glane) {
+  constexpr int kUnroll = 8;
+  auto group_min = [](int v) {
+    for (int off = kRowLanes / 2; off; off >>= 1) v = min(v, __shfl_xor(v, off, kRowLanes));
+    return v;
+  };
+  // scalar compare of [lo, hi): a few positions at the ends, or everything for rows that
+  // never reach a 16-byte boundary together
+  auto scalar_part = [&](int lo, int hi) {
+    int first = lim;
+    for (int j0 = lo; j0 < hi && first == lim; j0 += kRowLanes * kUnroll) {
+      int mine = lim;
+#pragma unroll
+      for (int u = kUnroll - 1; u >= 0; --u) {
+        const int j = j0 + u * kRowLanes + glane;
+        if (j < hi && a[j] != b[j]) mine = j;
+      }
+      first = group_min(mine);
+    }
+    return first;
+  };
+  const uintptr_t ua = reinterpret_cast<uintptr_t>(a), ub = reinterpret_cast<uintptr_t>(b);
+  if ((ua & 15) != (ub & 15)) return scalar_part(0, lim);
+  const int head = min(lim, (int)(((16 - (ua & 15)) & 15) >> 2));  // positions before the boundary
+  int first = scalar_part(0, head);
+  if (first != lim) return first;
+  const int4* a4 = reinterpret_cast<const int4*>(a + head);
+  const int4* b4 = reinterpret_cast<const int4*>(b + head);
+  const int nv = (lim - head) >> 2;
+  for (int j0 = 0; j0 < nv && first == lim; j0 += kRowLanes * kUnroll) {
+    int mine = lim;
+#pragma unroll
+    for (int u = kUnroll - 1; u >= 0; --u) {
+      const int j = j0 + u * kRowLanes + glane;
+      if (j < nv) {
+        const int4 x = a4[j], y = b4[j];
+        const int at = head + 4 * j;
+        if (x.w != y.w) mine = at + 3;
+        if (x.z != y.z) mine = at + 2;
+        if (x.y != y.y) mine = at + 1;
+        if (x.x != y.x) mine = at;
+      }
+    }
+    first = group_min(mine);
+  }
+  if (first != lim) return first;
+  return scalar_part(head + 4 * nv, lim);
 }
 
 __device__ inline int plan_fingerprint(const fca_plan& pl) {
@@ -129,6 +196,7 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   __shared__ int lds_scan[kBuildThreads];
   __shared__ int lds_mismatch;
   __shared__ int lds_any;
+  __shared__ int lds_listed;
   __shared__ int lds_hist[2 * kSizeBuckets];
   __shared__ int lds_cursor[2 * kSizeBuckets];
   __shared__ unsigned long long lds_tokens;
@@ -184,8 +252,8 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
     if (tid == 0) lds_mismatch = (hdr[H_BUILT] != kBuiltMagic || hdr[H_PLAN_SIG] != plan_sig) ? 1 : 0;
     __syncthreads();
     if (!lds_mismatch) {
-      const int gid = tid >> 4, glane = tid & 15;
-      for (int s = gid; s < S; s += kBuildThreads / 16) {
+      const int gid = tid / kRowLanes, glane = tid % kRowLanes;
+      for (int s = gid; s < S; s += kBuildThreads / kRowLanes) {
         const int len = p.seq_lens[s];
         const int shared_blocks = pos[s];
         // (a sequence that got shorter is a new request in an old slot: build anew, it may
@@ -283,30 +351,30 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       }
       __syncthreads();
       if (!lds_any) break;  // every key is alone: no shared node at this level or below
-      // Common run with the leader = first position where the two rows differ.  Every group
-      // of 16 lanes takes its own sequence (64 sequences in flight per pass) and scans 256
-      // positions per round, 16 independent loads per lane and row.
+      // Common run with the leader = first position where the two rows differ.  Followers
+      // that read the leader's own table row (query rows of one sequence) have nothing to
+      // compare; the others are listed (in a scratch array that is free here) and every group of
+      // kRowLanes lanes takes one listed sequence at a time (128 in flight per pass).
+      if (tid == 0) lds_listed = 0;
+      __syncthreads();
+      for (int s = tid; s < S; s += kBuildThreads) {
+        const int t = leader[s];
+        if (t < 0 || t == s) continue;
+        if (table_row(s) == table_row(t))
+          lcp[s] = min(lcp[s], min(nfull[s], nfull[t]) - pos[s]);
+        else
+          tmp0[atomicAdd(&lds_listed, 1)] = s;
+      }
+      __syncthreads();
       {
-        const int gid = tid >> 4, glane = tid & 15;
-        constexpr int kGroups = kBuildThreads / 16, kPerLane = 16;
-        for (int s = gid; s < S; s += kGroups) {
-          const int t = leader[s];
-          if (t < 0 || t == s) continue;
+        const int gid = tid / kRowLanes, glane = tid % kRowLanes;
+        const int listed = lds_listed;
+        for (int i = gid; i < listed; i += kBuildThreads / kRowLanes) {
+          const int s = tmp0[i], t = leader[s];
           const int lim = min(nfull[s], nfull[t]) - pos[s];
           const int32_t* row_s = p.block_table + table_row(s) * p.bt_stride + pos[s];
           const int32_t* row_t = p.block_table + table_row(t) * p.bt_stride + pos[s];
-          int first = lim;
-          // (query rows of one sequence read the same table row: nothing to compare)
-          for (int j0 = 0; row_s != row_t && j0 < lim && first == lim; j0 += 16 * kPerLane) {
-            int mine = lim;
-#pragma unroll
-            for (int u = kPerLane - 1; u >= 0; --u) {
-              const int j = j0 + u * 16 + glane;
-              if (j < lim && row_s[j] != row_t[j]) mine = j;
-            }
-            for (int off = 8; off; off >>= 1) mine = min(mine, __shfl_xor(mine, off, 16));
-            first = mine;
-          }
+          const int first = first_difference(row_s, row_t, lim, glane);
           if (glane == 0) lcp[s] = min(lcp[s], first);
         }
       }
@@ -387,10 +455,12 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       __syncthreads();
     }
     // What a later update starts from: fingerprints of the shared part of every row and
-    // the totals of the shared nodes.
-    {
-      const int gid = tid >> 4, glane = tid & 15;
-      for (int s = gid; s < S; s += kBuildThreads / 16) {
+    // the totals of the shared nodes.  With declared groups there is nothing to keep: the
+    // rows of a query run move on with every step, so the workspace stays marked as not
+    // built and an update on it is a full build.
+    if (!p.row_group) {
+      const int gid = tid / kRowLanes, glane = tid % kRowLanes;
+      for (int s = gid; s < S; s += kBuildThreads / kRowLanes) {
         const unsigned long long f = row_fingerprint(p.block_table + table_row(s) * p.bt_stride, pos[s], glane);
         if (glane == 0) sig[s] = f;
       }
@@ -408,12 +478,18 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   // Private leaves and per-sequence partial counts.  Node index space for the work list:
   // shared nodes [0, node_base), then leaf of sequence s at node_base + s.
   const int leaf_members = member_base;
-  for (int s = tid; s < S; s += kBuildThreads) {
-    const int tokens = max(0, tmp1[s] - pos[s] * kBlock);  // (none below a causal node)
-    meta[L.seq_leaf_blk + s] = pos[s];
-    meta[L.seq_npart + s] = ord[s] + num_chunks_for(tokens, chunk);
-    members[leaf_members + s] = s;
-    atomicAdd(&lds_tokens, (unsigned long long)tokens);
+  {
+    unsigned long long leaf_tokens = 0;
+    for (int s = tid; s < S; s += kBuildThreads) {
+      const int tokens = max(0, tmp1[s] - pos[s] * kBlock);  // (none below a causal node)
+      meta[L.seq_leaf_blk + s] = pos[s];
+      meta[L.seq_npart + s] = ord[s] + num_chunks_for(tokens, chunk);
+      members[leaf_members + s] = s;
+      leaf_tokens += (unsigned long long)tokens;
+    }
+    // one atomic per wave
+    for (int off = 32; off; off >>= 1) leaf_tokens += __shfl_xor(leaf_tokens, off);
+    if ((tid & 63) == 0 && leaf_tokens) atomicAdd(&lds_tokens, leaf_tokens);
   }
   if (tid < 2 * kSizeBuckets) {
     lds_hist[tid] = 0;
