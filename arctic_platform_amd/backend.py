@@ -11,18 +11,17 @@ not part of the reference tree, so the class and argument names below follow the
 public plug-in convention from its documentation, not from code in the reference.
 
 Decode batches: one query token per sequence, or a few (the verify step of speculative
-decoding, ``spec_model`` in the platform's config).  A sequence with several query tokens
-is handed to the kernels as that many query rows over the same block-table row, each one
-token longer than the one before it; the forest builder then finds their common blocks
-like any other shared prefix, so causal order among the new tokens needs no mask and no
-kernel of its own.
-
-Prefill chunks and mixed batches go the same way.  A run longer than
-``MAX_DECODE_QUERY_LEN`` tokens is cut into tiles, one per 16-token block of the cache:
-the rows of a tile are declared a group (``fca_build_metadata_rows``), read the KV before
-their block once for all of them through the shared-node items, and each reads its own
-block alone.  The response-over-shared-prompt attention of the trainer is the in-tree
-counterpart (arctic_platform/rl/zorro_train/qwen_attention_patcher.py:1117-1262).
+decoding, ``spec_model`` in the platform's config), prefill chunks and mixed batches.  A
+sequence with several query tokens is handed to the kernels as that many query rows over
+the same block-table row, each one token longer than the one before it
+(``fca_build_metadata_rows``).  The run is cut into tiles, one per 16-token block of the
+cache, by declaring the rows of a tile a group.  The forest builder first finds what the
+sequence shares with other sequences (a cached prompt): all rows of all those sequences
+read that once.  Below it every tile becomes a causal node: its rows read the rest of
+the sequence, up to and including their own block, once for all of them, and the kernels
+hide from each row the tokens behind its own.  The response-over-shared-prompt attention of
+the trainer is the in-tree counterpart
+(arctic_platform/rl/zorro_train/qwen_attention_patcher.py:1117-1262).
 """
 
 from __future__ import annotations
@@ -52,8 +51,7 @@ class CommonAttentionMetadata:
     num_actual_tokens: int | None = None
 
 
-# Longest run of query tokens per sequence whose rows are grouped by discovery (with the
-# rows of other sequences that share the prompt); longer runs are tiled per cache block.
+# Query runs up to this length count as decode for the choice of the row-tile height.
 MAX_DECODE_QUERY_LEN = 16
 
 
@@ -149,12 +147,11 @@ class ForestCascadeMetadataBuilder:
             ahead = starts[1:][req] - 1 - torch.arange(num_tokens, device=bt.device)  # query tokens after this one
             sl = (sl[req].to(torch.int64) - ahead).to(torch.int32)
             row_table = req.to(torch.int32)
-            if m.max_query_len > MAX_DECODE_QUERY_LEN:
-                # tiles of the long runs: one group per (sequence, cache block of the token)
-                if m.num_reqs * bt.shape[1] >= 2**31:
-                    raise ValueError("batch too large for 32-bit group ids")
-                tile = req * bt.shape[1] + (sl.to(torch.int64) - 1).clamp_(min=0) // BLOCK_SIZE
-                row_group = torch.where(q_lens[req] > MAX_DECODE_QUERY_LEN, tile, -1).to(torch.int32)
+            # tiles of the runs: one group per (sequence, cache block of the token)
+            if m.num_reqs * bt.shape[1] >= 2**31:
+                raise ValueError("batch too large for 32-bit group ids")
+            tile = req * bt.shape[1] + (sl.to(torch.int64) - 1).clamp_(min=0) // BLOCK_SIZE
+            row_group = torch.where(q_lens[req] > 1, tile, -1).to(torch.int32)
         key = (num_tokens, bt.shape[1], m.max_query_len > 1, row_group is not None)
         since = self._steps_since_build.get(key, self.rebuild_every)
         update = key in self._workspaces and since + 1 < self.rebuild_every
@@ -169,12 +166,13 @@ class ForestCascadeMetadataBuilder:
             chunk_tokens=self.chunk_tokens,
             rows_per_item=self.rows_multi_token if m.max_query_len > 1 else self.rows_per_item,
             cascade=self.enabled,
-            # the query tokens of a sequence share its private blocks: one more level
-            max_levels=min(self.max_levels + (1 if m.max_query_len > 1 else 0), 8),
+            max_levels=self.max_levels,
             out=self._workspaces.get(key),
             update=update and row_group is None,
             row_table=row_table,
             row_group=row_group,
+            # short runs read a block about once per launch, like plain decode
+            kv_reread=m.max_query_len > MAX_DECODE_QUERY_LEN,
         )
         self._workspaces[key] = forest
         return ForestCascadeMetadata(forest=forest, slot_mapping=m.slot_mapping[:num_tokens], num_decode_tokens=num_tokens)

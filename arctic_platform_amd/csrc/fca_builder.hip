@@ -12,10 +12,14 @@
 //
 // Query rows need not be one per block-table row: with a row table, several rows (the
 // tokens of a query run) read one table row up to different lengths.  The caller may
-// declare groups among them; a declared group is keyed by its id at the first level
-// instead of by block id, and its run ends before the block that holds the last token of
-// its shortest row, so that every member keeps a private leaf.  This is how a long run is
-// cut into tiles that each read the KV before them once.
+// declare groups among them.  Declared rows take part in discovery like any other row,
+// except that their last block (the one their own token is in) is never shared there and
+// that a group of nothing but declared rows of one table row is left alone.  After
+// discovery the declared rows meet once more under (node they ended in, group id): a group
+// that is a tile of a query run becomes a causal node from there to its last token, any
+// other declared group a plain node over what its members have in common.  This is how a
+// run is cut into tiles that each read their private KV once, below whatever its sequence
+// shares with others.
 //
 // Between two scheduler steps of a decode loop only the lengths change: every sequence
 // grows by a token and now and then takes a new private block.  The forest is a function
@@ -239,9 +243,10 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   // that holds the last token of its shortest row.  If the members are successive rows
   // reading one table row, each one token longer than the one before it, with their last
   // tokens in one block (a tile of a query run), the node takes that block in as well and
-  // is marked causal: its last chunk tells the attention kernel the first member's length,
-  // and the kernel hides from every row the tokens behind its own.  Such members have no
-  // leaf.  Any other declared group keeps a private leaf per member from that block on.
+  // is marked causal: its last chunk tells the attention kernel how many of its tokens the
+  // first member sees, and the kernel hides from every row the tokens behind its own.
+  // Such members have no leaf.  Any other declared group keeps a private leaf per member
+  // from that block on.
   auto declared = [&](int s) { return p.row_group && p.row_group[s] >= 0; };
 
   // ---- update: is the forest of the last build on this workspace still the forest of
@@ -302,7 +307,17 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
     }
     __syncthreads();
 
-    for (int level = 0; level < p.plan.max_levels; ++level) {
+    // Discovery level by level; then, if the caller has declared groups, one more pass in
+    // which the declared rows meet under (node they ended in, group id).  A row that drops
+    // out of discovery keeps its parent in par as -(parent + 3), so -2 stands for "none".
+    const bool have_groups = p.row_group != nullptr && p.plan.max_levels > 0;
+    auto parent_of = [&](int s) { return par[s] <= -2 ? -par[s] - 3 : par[s]; };
+    bool group_pass = false;
+    for (int level = 0;; ++level) {
+      if (!group_pass && level >= p.plan.max_levels) {
+        if (!have_groups) break;
+        group_pass = true;
+      }
       if (tid == 0) lds_any = 0;
       for (int i = tid; i < hsize; i += kBuildThreads) {
         hkeys[i] = kEmptyKey;
@@ -317,17 +332,14 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
         cmax[s] = 0;
       }
       __syncthreads();
-      // Key every sequence that still has a full block at its position.  A sequence whose
-      // parent is -2 dropped out of sharing at an earlier level.
+      // Key every sequence that still has a full block at its position and has not dropped
+      // out of sharing at an earlier level: rows meet under (parent node, physical block id
+      // at the current position).  In the pass for declared groups: every declared row.
       for (int s = tid; s < S; s += kBuildThreads) {
-        if (par[s] == -2) continue;
-        const bool by_id = level == 0 && declared(s);
-        if (by_id ? tmp1[s] < 1 : pos[s] >= nfull[s]) continue;
-        // The key of a declared group (first level only) is its id; otherwise rows meet
-        // under (parent node, physical block id at the current position).
+        if (group_pass ? !declared(s) || tmp1[s] < 1 : par[s] <= -2 || pos[s] >= nfull[s]) continue;
         unsigned long long key;
-        if (by_id) {
-          key = (1ull << 63) | (unsigned)p.row_group[s];
+        if (group_pass) {
+          key = (1ull << 63) | ((unsigned long long)(unsigned)(parent_of(s) + 1) << 32) | (unsigned)p.row_group[s];
         } else {
           const unsigned blk = (unsigned)p.block_table[table_row(s) * p.bt_stride + pos[s]];
           key = ((unsigned long long)(unsigned)(par[s] + 1) << 32) | blk;
@@ -350,7 +362,11 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
         }
       }
       __syncthreads();
-      if (!lds_any) break;  // every key is alone: no shared node at this level or below
+      if (!lds_any) {  // every key is alone: no shared node at this level or below
+        if (group_pass || !have_groups) break;
+        group_pass = true;
+        continue;
+      }
       // Common run with the leader = first position where the two rows differ.  Followers
       // that read the leader's own table row (query rows of one sequence) have nothing to
       // compare; the others are listed (in a scratch array that is free here) and every group of
@@ -384,31 +400,51 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
         if (t >= 0) {
           atomicMin(&run[t], lcp[s]);
           atomicAdd(&cnt[t], 1);
-          if (level == 0 && declared(s)) {
+          if (group_pass) {
+            // does the group look like a tile of a query run?
             const bool tile = table_row(s) == table_row(t) && tmp1[s] == tmp1[t] + (s - t) &&
                               (tmp1[s] - 1) / kBlock == (tmp1[t] - 1) / kBlock;
             if (!tile) atomicOr(&cbad[t], 1);
             atomicMax(&cmax[t], s - t);
+          } else if (have_groups) {
+            // does the group hold anything but declared rows of the leader's table row?
+            if (!declared(s) || table_row(s) != table_row(t)) atomicOr(&cbad[t], 1);
           }
         }
       }
       __syncthreads();
+      // Which leaders make a node (kept in `slot`, which is free by now: 0 none, 1 plain, 2
+      // causal).  Discovery leaves a group alone that is nothing but declared rows of one
+      // table row, i.e. the rows of one query run: the pass for declared groups tiles them.
+      // There, a group whose members are rows s, s + 1, ... without a gap, each one token
+      // longer and all ending in one block, is such a tile and becomes a causal node.
       for (int s = tid; s < S; s += kBuildThreads) {
-        const bool is_node = leader[s] == s && cnt[s] >= 2;
-        tmp0[s] = is_node ? 1 : 0;
-        nodeof[s] = is_node ? cnt[s] : 0;
+        int kind = 0;
+        if (leader[s] == s && cnt[s] >= 2) {
+          if (group_pass)
+            kind = !cbad[s] && cmax[s] + 1 == cnt[s] ? 2 : (run[s] > 0 ? 1 : 0);
+          else
+            kind = !have_groups || cbad[s] ? 1 : 0;
+        }
+        if (leader[s] == s) slot[s] = kind;
+        tmp0[s] = kind ? 1 : 0;
+        nodeof[s] = kind ? cnt[s] : 0;
       }
       __syncthreads();
       const int new_nodes = block_exclusive_scan(tmp0, tmp0, S, lds_scan);
-      if (new_nodes == 0) break;
+      if (new_nodes == 0) {
+        if (group_pass || !have_groups) break;
+        group_pass = true;
+        continue;
+      }
       const int new_members = block_exclusive_scan(nodeof, nodeof, S, lds_scan);
       ++levels;
       for (int s = tid; s < S; s += kBuildThreads) {
-        if (leader[s] == s && cnt[s] >= 2) {
+        if (leader[s] == s && slot[s]) {
           const int id = node_base + tmp0[s];
-          // a tile of a query run: members s, s + 1, ... without a gap, all fitting the pattern
-          const bool causal = level == 0 && declared(s) && !cbad[s] && cmax[s] + 1 == cnt[s];
-          const int ntok = causal ? tmp1[s] + cnt[s] - 1 : run[s] * kBlock;
+          // a causal node runs from the group's position to the last member's last token
+          const bool causal = slot[s] == 2;
+          const int ntok = causal ? tmp1[s] + cnt[s] - 1 - pos[s] * kBlock : run[s] * kBlock;
           meta[L.node_rep + id] = s;
           meta[L.node_blk + id] = pos[s];
           meta[L.node_nblk + id] = run[s] + (causal ? 1 : 0);
@@ -428,7 +464,7 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       // adjacent rows, so the scan is a handful of steps.
       for (int s = tid; s < S; s += kBuildThreads) {
         const int t = leader[s];
-        if (t < 0 || cnt[t] < 2) continue;
+        if (t < 0 || !slot[t]) continue;
         int below = 0;
         for (int j = t; j < s; ++j) below += leader[j] == t ? 1 : 0;
         members[meta[L.node_moff + tmp0[t]] + below] = s;
@@ -436,12 +472,12 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       __syncthreads();
       for (int s = tid; s < S; s += kBuildThreads) {
         const int t = leader[s];
-        if (t >= 0 && cnt[t] >= 2) {
+        if (t >= 0 && slot[t]) {
           lcp[s] = 1;  // advances past the node, after the barrier (pos[t] is read by others)
           par[s] = tmp0[t];
         } else {
           lcp[s] = 0;
-          par[s] = -2;
+          if (par[s] > -2) par[s] = -(par[s] + 3);  // out of discovery from here on
         }
       }
       __syncthreads();
@@ -453,6 +489,7 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       node_base += new_nodes;
       member_base += new_members;
       __syncthreads();
+      if (group_pass) break;
     }
     // What a later update starts from: fingerprints of the shared part of every row and
     // the totals of the shared nodes.  With declared groups there is nothing to keep: the
@@ -509,7 +546,7 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       rep = (int)table_row(meta[L.node_rep + n]);
       blk = meta[L.node_blk + n];
       tokens = meta[L.node_tok + n];
-      if (meta[L.node_causal + n]) first_len = tmp1[meta[L.node_rep + n]];
+      if (meta[L.node_causal + n]) first_len = tmp1[meta[L.node_rep + n]] - blk * kBlock;
       moff = meta[L.node_moff + n];
       mcnt = meta[L.node_mcnt + n];
       o = meta[L.node_ord + n];

@@ -81,7 +81,7 @@ inline __host__ MetaLayout make_layout(const fca_plan& p) {
   L.node_ord = take(S);
   L.node_tok = take(S);
   L.node_causal = take(S);
-  L.members = take(S * (FCA_MAX_LEVELS + 1));
+  L.members = take(S * (FCA_MAX_LEVELS + 2));  // discovery levels, the pass for declared groups, leaves
   L.items = take(L.max_items * kItemInts);
   L.s_pos = take(S);
   L.s_par = take(S);

@@ -38,12 +38,9 @@ class ForestMetadata:
     seq_lens: torch.Tensor  # per query row
     row_table: torch.Tensor | None = None  # block-table row of every query row (None: the row itself)
     row_group: torch.Tensor | None = None  # declared groups of query rows
-
-    @property
-    def kv_reread(self) -> bool:
-        """The tiles of a long query run read the same blocks one after the other: keep the
-        KV loads cacheable.  (Rows grouped by discovery alone read a block about once.)"""
-        return self.row_group is not None
+    # The tiles of a long query run read the same blocks one after the other: the attention
+    # calls then keep their KV loads cacheable (fca_tensors.kv_reread).
+    kv_reread: bool = False
 
     # ---- inspection (synchronises; not for the decode loop) -------------------------
     def header(self) -> dict:
@@ -146,6 +143,7 @@ def build_forest_metadata(
     update: bool = False,
     row_table: torch.Tensor | None = None,
     row_group: torch.Tensor | None = None,
+    kv_reread: bool | None = None,
 ) -> ForestMetadata:
     """Discover the shared-prefix forest of a decode batch on the device.
 
@@ -154,6 +152,8 @@ def build_forest_metadata(
     of a query run: one row per token, each one token longer), ``seq_lens`` is ``[R]`` and
     the result serves ``q`` of ``R`` rows.  ``row_group`` (int32 ``[R]``, -1 = none) declares
     groups of rows that share their leading blocks (``fca_build_metadata_rows``).
+    ``kv_reread`` says whether a launch reads KV blocks again and again (long query runs,
+    many tiles per sequence); the default assumes so when groups are declared.
 
     ``cascade=False`` turns sharing off: every sequence becomes one private node over its
     whole block-table row, which makes the same kernels a plain paged decode attention.
@@ -190,6 +190,7 @@ def build_forest_metadata(
     same_workspace = out is not None and bytes(out.plan) == bytes(plan)
     if same_workspace:
         md = dataclasses.replace(out, block_table=block_table, seq_lens=seq_lens, row_table=row_table, row_group=row_group)
+        md.kv_reread = row_group is not None if kv_reread is None else bool(kv_reread)
     else:
         layout = _lib.FcaMetaLayout()
         _lib.check(lib.fca_meta_describe(ctypes.byref(plan), ctypes.byref(layout)))
@@ -207,6 +208,7 @@ def build_forest_metadata(
             seq_lens=seq_lens,
             row_table=row_table,
             row_group=row_group,
+            kv_reread=row_group is not None if kv_reread is None else bool(kv_reread),
         )
         assert md.partial_out.numel() * 2 == no.value and md.partial_lse.numel() * 4 == nl.value
     if row_table is not None:

@@ -109,7 +109,7 @@ typedef struct fca_meta_layout {
   int64_t node_moff;     /* [S] offset into members */
   int64_t node_mcnt;     /* [S] number of members */
   int64_t node_ord;      /* [S] partial ordinal of the node's first chunk */
-  int64_t members;       /* [S * (FCA_MAX_LEVELS + 1)] sequence ids; leaves last */
+  int64_t members;       /* [S * (FCA_MAX_LEVELS + 2)] sequence ids; leaves last */
   int64_t items;         /* [max_items * 8] */
   int64_t max_items;
   int64_t max_partials;  /* partial slots reserved per sequence */

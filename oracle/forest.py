@@ -14,13 +14,15 @@ of a sequence below its deepest shared node is its private leaf.
 
 Query rows need not be block-table rows: with ``row_table`` query row r reads table row
 ``row_table[r]`` up to ``seq_lens[r]`` tokens (the tokens of a query run).  ``row_group``
-declares first-level groups among such rows in place of the block-id comparison; for a
-declared row the last block it may share is the one before the block that holds its last
-token.  A declared group whose members are successive rows over one table row, each one
-token longer than the one before it and all ending in one block, is a tile of a query run:
-its node takes that block in too, holds ``tokens`` = the last member's length, is marked
-``causal`` (each member attends only up to its own token) and leaves its members no leaf.
-Members of any other declared group keep a private leaf from that block on.  The trainer's counterpart is the
+declares groups among such rows.  A declared row takes part in the discovery above, but
+the last block it may share there is the one before the block that holds its last token,
+and a group made of nothing but declared rows of one table row is left alone.  After
+discovery the declared rows meet under (node they ended in, group id).  A group whose
+members are successive rows over one table row, each one token longer than the one before
+it and all ending in one block, is a tile of a query run: its node runs from where
+discovery left the rows to the last member's last token (``tokens``), is marked ``causal``
+(each member attends only up to its own token) and leaves its members no leaf.  Any other
+declared group gets a plain node over what its members still have in common.  The trainer's counterpart is the
 response-over-shared-prompt attention, which reads each unique prompt once for all its
 responses (arctic_platform/rl/zorro_train/qwen_attention_patcher.py:1117-1262).
 """
@@ -40,54 +42,71 @@ def discover_forest(block_table, seq_lens, block_size=BLOCK, max_levels=8, row_t
     """
     table = [list(map(int, row)) for row in block_table]
     lens = [int(n) for n in seq_lens]
-    bt = table if row_table is None else [table[int(r)] for r in row_table]
+    trow = list(range(len(lens))) if row_table is None else [int(r) for r in row_table]
+    bt = [table[r] for r in trow]
     group_of = [-1] * len(lens) if row_group is None else [int(g) for g in row_group]
     nfull = [(max(n - 1, 0) if g >= 0 else n) // block_size for n, g in zip(lens, group_of)]
     nodes = []
     leaf_start = [0] * len(lens)
     leaf_parent = [-1] * len(lens)
 
+    def common_run(group, pos):
+        limit = min(nfull[s] for s in group) - pos
+        first = group[0]
+        run = 0
+        while run < limit and all(bt[s][pos + run] == bt[first][pos + run] for s in group):
+            run += 1
+        return run
+
+    def add_node(group, pos, run, tokens, causal, level, parent):
+        nodes.append(dict(members=list(group), blk_start=pos, num_blocks=run, tokens=tokens, causal=causal, level=level, parent=parent))
+        for s in group:
+            leaf_start[s] = pos + run
+            leaf_parent[s] = len(nodes) - 1
+        return len(nodes) - 1
+
     def descend(members, pos, level, parent):
         if level >= max_levels:
             return
         groups = OrderedDict()
         for s in members:
-            if level == 0 and group_of[s] >= 0:
-                if lens[s] >= 1:
-                    groups.setdefault(("declared", group_of[s]), []).append(s)
-            elif pos < nfull[s]:
+            if pos < nfull[s]:
                 groups.setdefault(bt[s][pos], []).append(s)
         for group in groups.values():
             if len(group) < 2:
                 continue
-            limit = min(nfull[s] for s in group) - pos
-            first = group[0]
-            run = 0
-            while run < limit and all(bt[s][pos + run] == bt[first][pos + run] for s in group):
-                run += 1
-            tokens, causal = run * block_size, False
-            if level == 0 and group_of[first] >= 0:
-                trow = (lambda s: s) if row_table is None else (lambda s: int(row_table[s]))
-                causal = all(
-                    s == first + i
-                    and trow(s) == trow(first)
-                    and lens[s] == lens[first] + i
-                    and (lens[s] - 1) // block_size == (lens[first] - 1) // block_size
-                    for i, s in enumerate(group)
-                )
-                if causal:
-                    run, tokens = run + 1, lens[group[-1]]
-            node_id = len(nodes)
-            nodes.append(
-                dict(members=list(group), blk_start=pos, num_blocks=run, tokens=tokens, causal=causal, level=level, parent=parent)
-            )
-            for s in group:
-                leaf_start[s] = pos + run
-                leaf_parent[s] = node_id
-            if not causal:
-                descend(group, pos + run, level + 1, node_id)
+            if all(group_of[s] >= 0 and trow[s] == trow[group[0]] for s in group):
+                continue  # the rows of one query run: tiled by their declared groups below
+            run = common_run(group, pos)
+            node_id = add_node(group, pos, run, run * block_size, False, level, parent)
+            descend(group, pos + run, level + 1, node_id)
 
     descend(list(range(len(lens))), 0, 0, -1)
+
+    # declared groups, below whatever discovery found
+    if max_levels > 0:
+        declared = OrderedDict()
+        for s in range(len(lens)):
+            if group_of[s] >= 0 and lens[s] >= 1:
+                declared.setdefault((leaf_parent[s], group_of[s]), []).append(s)
+        for (parent, _), group in declared.items():
+            if len(group) < 2:
+                continue
+            first, pos = group[0], leaf_start[group[0]]
+            level = nodes[parent]["level"] + 1 if parent >= 0 else 0
+            tile = all(
+                s == first + i
+                and trow[s] == trow[first]
+                and lens[s] == lens[first] + i
+                and (lens[s] - 1) // block_size == (lens[first] - 1) // block_size
+                for i, s in enumerate(group)
+            )
+            run = common_run(group, pos)
+            if tile:
+                add_node(group, pos, run + 1, lens[group[-1]] - pos * block_size, True, level, parent)
+            elif run > 0:
+                add_node(group, pos, run, run * block_size, False, level, parent)
+
     leaves = [
         dict(blk_start=leaf_start[s], tokens=max(0, lens[s] - leaf_start[s] * block_size), parent=leaf_parent[s])
         for s in range(len(lens))

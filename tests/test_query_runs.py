@@ -38,6 +38,9 @@ def covered_tokens(nodes, leaves, row, row_len):
     for n in nodes:
         if row in n["members"]:
             end = n["blk_start"] * BLOCK + n["tokens"]
+            if n["parent"] >= 0:  # a node starts where its parent ends
+                up = nodes[n["parent"]]
+                assert row in up["members"] and n["blk_start"] == up["blk_start"] + up["num_blocks"]
             assert n["causal"] or n["tokens"] == n["num_blocks"] * BLOCK
             assert not n["causal"] or (n["num_blocks"] - 1) * BLOCK < n["tokens"] <= n["num_blocks"] * BLOCK
             spans.append((n["blk_start"] * BLOCK, min(end, row_len) if n["causal"] else end))
@@ -110,6 +113,25 @@ def test_mixed_batch_keeps_discovery_for_single_tokens():
     assert_exact_cover(nodes, leaves, row_lens)
 
 
+def test_runs_below_a_prompt_shared_between_sequences():
+    # two samples of one prompt (blocks 1, 2, 3 cached and shared), each verifying three
+    # speculated tokens at lengths 50..52 and 58..60; a third sequence alone
+    table = [[1, 2, 3, 10], [1, 2, 3, 11], [7, 8, 9, 0]]
+    row_table, row_lens, row_group = run_rows([(49, 3), (57, 3), (20, 1)], max_blocks=4)
+    nodes, leaves = discover_forest(table, row_lens, row_table=row_table, row_group=row_group)
+    by_members = {tuple(n["members"]): n for n in nodes}
+    # all six rows read the prompt once ...
+    shared = by_members[(0, 1, 2, 3, 4, 5)]
+    assert (shared["blk_start"], shared["num_blocks"], shared["causal"]) == (0, 3, False)
+    # ... and below it each sequence's rows form one causal tile over its fourth block
+    for members, last_len in (((0, 1, 2), 52), ((3, 4, 5), 60)):
+        n = by_members[members]
+        assert n["causal"] and (n["blk_start"], n["num_blocks"], n["tokens"]) == (3, 1, last_len - 48)
+        assert nodes[n["parent"]] is shared and n["level"] == 1
+    assert len(nodes) == 3 and [l["tokens"] for l in leaves] == [0] * 6 + [21]
+    assert_exact_cover(nodes, leaves, row_lens)
+
+
 def test_cover_invariant_on_random_batches():
     rng = random.Random(5)
     for _ in range(30):
@@ -167,6 +189,9 @@ CASES = [
     (2, 32, 8, 128, torch.bfloat16, 64, 128, [(0, 200), (130, 70), (77, 1), (90, 1), (5, 3)], ((2, 3, 4),)),
     (3, 16, 4, 128, torch.float8_e4m3fn, 64, 256, [(0, 129), (511, 33), (40, 1)], ()),
     (4, 32, 4, 64, torch.bfloat16, 64, 32, [(16, 48), (0, 16), (15, 2)], ()),  # GQA 8: two row tiles per group
+    # speculative verify: four samples of one 100-token prompt and two of another, 2 to 5 query tokens each
+    (5, 32, 8, 128, torch.bfloat16, 64, 64, [(130, 4), (141, 4), (97, 5), (163, 2), (80, 3), (95, 3), (40, 1)], ((0, 1, 6), (0, 2, 6), (0, 3, 6), (4, 5, 4))),
+    (6, 8, 2, 64, torch.float8_e4m3fn, 32, 32, [(130, 4), (141, 4), (97, 5), (70, 20)], ((0, 1, 6), (0, 2, 6), (0, 3, 3))),
 ]
 
 
