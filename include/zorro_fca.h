@@ -155,22 +155,28 @@ int fca_update_metadata(const fca_plan* plan, const int32_t* block_table_dev, in
  * rows R (rows of q and out); row r attends to the first row_lens_dev[r] tokens of
  * block-table row row_table_dev[r] (< table_rows), which for token i of a sequence is the
  * sequence's length up to and including that token, so causal order needs no mask.
- * row_group_dev may be NULL.  A value >= 0 declares a group: rows with equal values share
- * their leading blocks, and the builder makes one shared node of the run that ends before
- * the block holding the last token of the group's shortest row (rows of one table row are
- * not compared, others are, so a wrong declaration costs sharing, never correctness).
- * Declared groups are how a long run is tiled: the tokens of one 16-token block form a
- * group.  When the members of a group are successive rows over one table row, each one
- * token longer than the one before it and all ending in one block, the node takes that
- * block in as well (a causal node): the group reads all its KV once, the kernels hide from
- * every row the tokens behind its own, and the rows have no private part.  Other declared
- * groups read the KV before that block once and each row reads the rest alone.  Rows with
- * -1 are grouped by discovery as in fca_build_metadata, and declared groups that are not
- * causal take part in discovery below their node.  update != 0 asks for the
- * update of fca_update_metadata.  The attention calls then take the [table_rows,
- * max_blocks] block table and kv_reread = 1.  Counterpart in the reference: the
- * response-over-shared-prompt attention of the trainer, which rebuilds full sequences from
- * de-duplicated prompts (arctic_platform/rl/zorro_train/zorro_train.py:160-235) and runs
+ * row_group_dev may be NULL.  A value >= 0 declares a group, which is how a run is cut
+ * into tiles: give the tokens of one 16-token cache block of one sequence one id.
+ * All rows first go through the discovery of fca_build_metadata (rows with -1 exactly as
+ * there).  A declared row never shares the block its own token is in through discovery,
+ * and a group that discovery finds among declared rows of one table row alone is left
+ * alone, so what discovery keeps is what a sequence shares with other sequences (a
+ * cached prompt): all rows of all those sequences read it once.  Then the declared rows
+ * meet under (node they ended in, group id).  When the members of a group are successive
+ * rows over one table row, each one token longer than the one before it and all ending in
+ * one block, the group becomes a causal node from there to its last token: it reads the
+ * rest of its KV, its own block included, once, the kernels hide from every row the
+ * tokens behind its own, and the rows have no private part.  Any other declared group
+ * (rows over different table rows: an explicit tree) becomes a plain node over the blocks
+ * its members still have in common (rows of one table row are not compared, others are,
+ * so a wrong declaration costs sharing, never correctness), and each row reads the rest
+ * alone.  A build with declared groups leaves nothing for an update to keep, so an update
+ * on such a workspace is a full build; update != 0 otherwise asks for the update of
+ * fca_update_metadata.  The attention calls take the [table_rows, max_blocks] block
+ * table, and kv_reread = 1 when runs are long (many tiles read the same blocks).
+ * Counterpart in the reference: the response-over-shared-prompt attention of the trainer,
+ * which rebuilds full sequences from de-duplicated prompts
+ * (arctic_platform/rl/zorro_train/zorro_train.py:160-235) and runs
  * a varlen attention over them (rl/zorro_train/qwen_attention_patcher.py:1117-1262). */
 int fca_build_metadata_rows(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,
                             int32_t table_rows, const int32_t* row_table_dev, const int32_t* row_group_dev,
