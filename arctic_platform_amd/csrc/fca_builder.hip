@@ -196,6 +196,16 @@ __device__ inline int plan_fingerprint(const fca_plan& pl) {
   return (int)(k & 0x7fffffff);
 }
 
+// Runs of equal keys over the adjacent lanes of a wave (adjacent lanes hold adjacent rows,
+// and the rows of a group usually are adjacent): the lane a lane's run starts at.  One lane
+// per run then speaks for all of them, which turns up to 64 atomics on one address into
+// one.  Every lane of the wave must call this.
+__device__ inline int run_head_lane(unsigned long long key, int lane) {
+  const unsigned long long prev = __shfl_up(key, 1);
+  const unsigned long long heads = __ballot(lane == 0 || prev != key);
+  return 63 - __clzll((long long)(heads & ((2ull << lane) - 1)));
+}
+
 __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p) {
   __shared__ int lds_scan[kBuildThreads];
   __shared__ int lds_mismatch;
@@ -206,6 +216,7 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   __shared__ unsigned long long lds_tokens;
 
   const int tid = threadIdx.x;
+  const int lane = tid & 63;
   const int S = p.plan.num_seqs;
   const int chunk = p.plan.chunk_tokens;
   const int group = p.plan.num_q_heads / p.plan.num_kv_heads;
@@ -335,23 +346,34 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       // Key every sequence that still has a full block at its position and has not dropped
       // out of sharing at an earlier level: rows meet under (parent node, physical block id
       // at the current position).  In the pass for declared groups: every declared row.
-      for (int s = tid; s < S; s += kBuildThreads) {
-        if (group_pass ? !declared(s) || tmp1[s] < 1 : par[s] <= -2 || pos[s] >= nfull[s]) continue;
-        unsigned long long key;
-        if (group_pass) {
-          key = (1ull << 63) | ((unsigned long long)(unsigned)(parent_of(s) + 1) << 32) | (unsigned)p.row_group[s];
-        } else {
-          const unsigned blk = (unsigned)p.block_table[table_row(s) * p.bt_stride + pos[s]];
-          key = ((unsigned long long)(unsigned)(par[s] + 1) << 32) | blk;
+      // The first lane of every run of equal keys in a wave enters the key and its own row,
+      // the smallest of the run, for all of them.
+      for (int base = 0; base < S; base += kBuildThreads) {
+        const int s = base + tid;
+        const bool keyed =
+            s < S && !(group_pass ? !declared(s) || tmp1[s] < 1 : par[s] <= -2 || pos[s] >= nfull[s]);
+        unsigned long long key = kEmptyKey - 1 - (unsigned)lane;  // no key: a run of its own
+        if (keyed) {
+          if (group_pass) {
+            key = (1ull << 63) | ((unsigned long long)(unsigned)(parent_of(s) + 1) << 32) | (unsigned)p.row_group[s];
+          } else {
+            const unsigned blk = (unsigned)p.block_table[table_row(s) * p.bt_stride + pos[s]];
+            key = ((unsigned long long)(unsigned)(par[s] + 1) << 32) | blk;
+          }
         }
-        int h = hash_key(key) & (hsize - 1);
-        for (int probe = 0; probe < hsize; ++probe) {
-          unsigned long long prev = atomicCAS(&hkeys[h], kEmptyKey, key);
-          if (prev == kEmptyKey || prev == key) break;
-          h = (h + 1) & (hsize - 1);
+        const int head = run_head_lane(key, lane);
+        int h = -1;
+        if (keyed && head == lane) {
+          h = hash_key(key) & (hsize - 1);
+          for (int probe = 0; probe < hsize; ++probe) {
+            unsigned long long prev = atomicCAS(&hkeys[h], kEmptyKey, key);
+            if (prev == kEmptyKey || prev == key) break;
+            h = (h + 1) & (hsize - 1);
+          }
+          atomicMin(&hmin[h], s);
         }
-        slot[s] = h;
-        atomicMin(&hmin[h], s);
+        h = __shfl(h, head);
+        if (keyed) slot[s] = h;
       }
       __syncthreads();
       for (int s = tid; s < S; s += kBuildThreads) {
@@ -395,21 +417,39 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
         }
       }
       __syncthreads();
-      for (int s = tid; s < S; s += kBuildThreads) {
-        const int t = leader[s];
+      // Per leader: the shortest common run, the member count, the largest distance of a
+      // member's row from the leader's, and a flag (below).  The last lane of every run of
+      // equal leaders in a wave reports for the run.
+      for (int base = 0; base < S; base += kBuildThreads) {
+        const int s = base + tid;
+        const int t = s < S ? leader[s] : -1;
+        int shortest = 0x7fffffff, flag = 0;
         if (t >= 0) {
-          atomicMin(&run[t], lcp[s]);
-          atomicAdd(&cnt[t], 1);
+          shortest = lcp[s];
           if (group_pass) {
             // does the group look like a tile of a query run?
-            const bool tile = table_row(s) == table_row(t) && tmp1[s] == tmp1[t] + (s - t) &&
-                              (tmp1[s] - 1) / kBlock == (tmp1[t] - 1) / kBlock;
-            if (!tile) atomicOr(&cbad[t], 1);
-            atomicMax(&cmax[t], s - t);
+            flag = !(table_row(s) == table_row(t) && tmp1[s] == tmp1[t] + (s - t) &&
+                     (tmp1[s] - 1) / kBlock == (tmp1[t] - 1) / kBlock);
           } else if (have_groups) {
             // does the group hold anything but declared rows of the leader's table row?
-            if (!declared(s) || table_row(s) != table_row(t)) atomicOr(&cbad[t], 1);
+            flag = !declared(s) || table_row(s) != table_row(t);
           }
+        }
+        const unsigned long long key = t >= 0 ? (unsigned long long)(unsigned)t : kEmptyKey - 1 - (unsigned)lane;
+        const int head = run_head_lane(key, lane);
+        for (int off = 1; off < 64; off <<= 1) {  // minimum and flag from the run's first lane up to this one
+          const int other_shortest = __shfl_up(shortest, off), other_flag = __shfl_up(flag, off);
+          if (lane - off >= head) {
+            shortest = min(shortest, other_shortest);
+            flag |= other_flag;
+          }
+        }
+        const int next_head = __shfl_down(head, 1);
+        if (t >= 0 && (lane == 63 || next_head != head)) {
+          atomicMin(&run[t], shortest);
+          atomicAdd(&cnt[t], lane - head + 1);
+          atomicMax(&cmax[t], s - t);
+          if (flag) atomicOr(&cbad[t], 1);
         }
       }
       __syncthreads();
@@ -460,13 +500,15 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       }
       __syncthreads();
       // Member lists in ascending sequence order: rank = members of the same leader below s.
-      // One thread per sequence scans [leader, s); the members of a group are usually
-      // adjacent rows, so the scan is a handful of steps.
+      // Where the members are not adjacent rows, one thread per sequence scans [leader, s).
       for (int s = tid; s < S; s += kBuildThreads) {
         const int t = leader[s];
         if (t < 0 || !slot[t]) continue;
-        int below = 0;
-        for (int j = t; j < s; ++j) below += leader[j] == t ? 1 : 0;
+        int below = s - t;  // members in adjacent rows (the usual case): the distance is the rank
+        if (cmax[t] + 1 != cnt[t]) {
+          below = 0;
+          for (int j = t; j < s; ++j) below += leader[j] == t ? 1 : 0;
+        }
         members[meta[L.node_moff + tmp0[t]] + below] = s;
       }
       __syncthreads();
