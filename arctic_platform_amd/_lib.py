@@ -25,6 +25,7 @@ EXPORTS = (
     "fca_build_metadata",
     "fca_update_metadata",
     "fca_build_metadata_rows",
+    "fca_rows_from_query_runs",
     "fca_prefix_pass",
     "fca_suffix_pass",
     "fca_forest_pass",
@@ -134,6 +135,7 @@ def load_library() -> ctypes.CDLL:
     lib.fca_build_metadata.argtypes = [P(FcaPlan), VP, I64, VP, VP, VP]
     lib.fca_update_metadata.argtypes = [P(FcaPlan), VP, I64, VP, VP, VP]
     lib.fca_build_metadata_rows.argtypes = [P(FcaPlan), VP, I64, I32, VP, VP, VP, VP, I32, VP]
+    lib.fca_rows_from_query_runs.argtypes = [VP, VP, I32, I32, I32, VP, VP, VP, VP]
     attend = [P(FcaPlan), P(FcaTensors), VP, VP, VP, VP]
     lib.fca_prefix_pass.argtypes = attend
     lib.fca_suffix_pass.argtypes = attend

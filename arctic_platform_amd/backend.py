@@ -33,7 +33,7 @@ import torch
 
 from .cache import append_kv
 from .config import ModelConfig, validate_fca_support
-from .forest import ForestMetadata, build_forest_metadata
+from .forest import ForestMetadata, build_forest_metadata, rows_from_query_runs
 from .kv_layout import BLOCK_SIZE, kv_cache_shape
 from .ops import forest_cascade_decode
 
@@ -139,19 +139,16 @@ class ForestCascadeMetadataBuilder:
         num_tokens = m.num_reqs
         row_table = row_group = None
         if m.max_query_len > 1:
-            # one row per query token: the row of its sequence, cut off behind the token itself
-            starts = m.query_start_loc[: m.num_reqs + 1].to(torch.int64)
-            q_lens = starts[1:] - starts[:-1]
+            # one row per query token: the row of its sequence, cut off behind the token itself;
+            # the tokens of a run that fall into one cache block form a tile
+            starts = m.query_start_loc[: m.num_reqs + 1]
             num_tokens = m.num_actual_tokens if m.num_actual_tokens is not None else int(starts[-1])
-            req = torch.repeat_interleave(torch.arange(m.num_reqs, device=bt.device), q_lens, output_size=num_tokens)
-            ahead = starts[1:][req] - 1 - torch.arange(num_tokens, device=bt.device)  # query tokens after this one
-            sl = (sl[req].to(torch.int64) - ahead).to(torch.int32)
-            row_table = req.to(torch.int32)
-            # tiles of the runs: one group per (sequence, cache block of the token)
-            if m.num_reqs * bt.shape[1] >= 2**31:
-                raise ValueError("batch too large for 32-bit group ids")
-            tile = req * bt.shape[1] + (sl.to(torch.int64) - 1).clamp_(min=0) // BLOCK_SIZE
-            row_group = torch.where(q_lens[req] > 1, tile, -1).to(torch.int32)
+            rows_key = (num_tokens, "rows")
+            if rows_key not in self._workspaces:
+                self._workspaces[rows_key] = tuple(torch.empty(num_tokens, dtype=torch.int32, device=bt.device) for _ in range(3))
+            row_table, sl, row_group = rows_from_query_runs(
+                starts.to(torch.int32).contiguous(), sl.contiguous(), num_tokens, bt.shape[1], out=self._workspaces[rows_key]
+            )
         key = (num_tokens, bt.shape[1], m.max_query_len > 1, row_group is not None)
         since = self._steps_since_build.get(key, self.rebuild_every)
         update = key in self._workspaces and since + 1 < self.rebuild_every

@@ -228,6 +228,21 @@ int fca_build_metadata_rows(const fca_plan* plan, const int32_t* block_table_dev
                    row_table_dev, row_group_dev);
 }
 
+int fca_rows_from_query_runs(const int32_t* query_start_loc_dev, const int32_t* seq_lens_dev, int32_t num_reqs,
+                             int32_t num_rows, int32_t max_blocks, int32_t* row_table_dev, int32_t* row_lens_dev,
+                             int32_t* row_group_dev, void* stream) {
+  if (num_reqs < 1 || num_rows < 0 || max_blocks < 1)
+    return fail(FCA_ERR_INVALID_ARG, "num_reqs and max_blocks must be >= 1 and num_rows >= 0");
+  if ((int64_t)num_reqs * max_blocks > 0x7fffffffLL)
+    return fail(FCA_ERR_UNSUPPORTED, "num_reqs * max_blocks exceeds 32-bit group ids");
+  if (num_rows == 0) return FCA_OK;
+  if (!query_start_loc_dev || !seq_lens_dev || !row_table_dev || !row_lens_dev || !row_group_dev)
+    return fail(FCA_ERR_INVALID_ARG, "query_start_loc, seq_lens and the three row arrays must be non-NULL");
+  hipError_t e = fca::launch_rows(query_start_loc_dev, seq_lens_dev, num_reqs, num_rows, max_blocks, row_table_dev,
+                                  row_lens_dev, row_group_dev, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? FCA_OK : hip_fail(e, "query-row kernel launch");
+}
+
 int fca_prefix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev, void* partial_out_dev,
                     float* partial_lse_dev, void* stream) {
   return run_attend(plan, t, meta_dev, partial_out_dev, partial_lse_dev, 1, stream);

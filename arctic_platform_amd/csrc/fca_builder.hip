@@ -662,6 +662,35 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   }
 }
 
+// Query rows of a step from the engine's per-request arrays: one thread per query token
+// finds its request by bisection over the cumulative query lengths.
+__global__ __launch_bounds__(256) void fca_rows_kernel(const int32_t* __restrict__ query_start_loc,
+                                                       const int32_t* __restrict__ seq_lens, int num_reqs, int num_rows,
+                                                       int max_blocks, int32_t* __restrict__ row_table,
+                                                       int32_t* __restrict__ row_lens, int32_t* __restrict__ row_group) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= num_rows) return;
+  int lo = 0, hi = num_reqs - 1;  // last request whose first token is at or before r
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (query_start_loc[mid] <= r) lo = mid; else hi = mid - 1;
+  }
+  const int first = query_start_loc[lo], end = query_start_loc[lo + 1];
+  // the sequence length counts the whole run: this token sees all but the tokens after it
+  const int len = seq_lens[lo] - (end - 1 - r);
+  row_table[r] = lo;
+  row_lens[r] = len;
+  // a run of two or more tokens is tiled per cache block of the token
+  row_group[r] = end - first > 1 ? lo * max_blocks + max(len - 1, 0) / kBlock : -1;
+}
+
+hipError_t launch_rows(const int32_t* query_start_loc, const int32_t* seq_lens, int num_reqs, int num_rows, int max_blocks,
+                       int32_t* row_table, int32_t* row_lens, int32_t* row_group, hipStream_t stream) {
+  hipLaunchKernelGGL(fca_rows_kernel, dim3((num_rows + 255) / 256), dim3(256), 0, stream, query_start_loc, seq_lens,
+                     num_reqs, num_rows, max_blocks, row_table, row_lens, row_group);
+  return hipGetLastError();
+}
+
 hipError_t launch_build(const BuildParams& p, hipStream_t stream) {
   hipLaunchKernelGGL(fca_build_kernel, dim3(1), dim3(kBuildThreads), 0, stream, p);
   return hipGetLastError();

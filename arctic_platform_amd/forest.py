@@ -119,6 +119,29 @@ class ForestMetadata:
         return out
 
 
+def rows_from_query_runs(query_start_loc: torch.Tensor, seq_lens: torch.Tensor, num_rows: int, max_blocks: int, out=None):
+    """Row table, row lengths and tile group ids of a step with query runs, one entry per
+    query token (``fca_rows_from_query_runs``; one launch, no synchronisation).  ``out`` may
+    hold three int32 tensors of at least ``num_rows`` entries to write into."""
+    num_reqs = seq_lens.shape[0]
+    if query_start_loc.dtype != torch.int32 or seq_lens.dtype != torch.int32:
+        raise TypeError("query_start_loc and seq_lens must be int32")
+    if query_start_loc.shape[0] < num_reqs + 1 or not (query_start_loc.is_contiguous() and seq_lens.is_contiguous()):
+        raise ValueError("query_start_loc must be contiguous with num_reqs + 1 entries, seq_lens contiguous")
+    if not seq_lens.is_cuda:
+        raise RuntimeError("query rows are made on the GPU; seq_lens must be a device tensor")
+    if out is None:
+        out = tuple(torch.empty(num_rows, dtype=torch.int32, device=seq_lens.device) for _ in range(3))
+    row_table, row_lens, row_group = (t[:num_rows] for t in out)
+    _lib.check(
+        _lib.load_library().fca_rows_from_query_runs(
+            query_start_loc.data_ptr(), seq_lens.data_ptr(), num_reqs, num_rows, max_blocks,
+            row_table.data_ptr(), row_lens.data_ptr(), row_group.data_ptr(), _stream_ptr(seq_lens.device),
+        )
+    )
+    return row_table, row_lens, row_group
+
+
 def make_plan(
     num_seqs, max_blocks, num_q_heads, num_kv_heads, head_dim, *, chunk_tokens=512, rows_per_item=32, max_levels=4
 ) -> _lib.FcaPlan:

@@ -182,6 +182,18 @@ int fca_build_metadata_rows(const fca_plan* plan, const int32_t* block_table_dev
                             int32_t table_rows, const int32_t* row_table_dev, const int32_t* row_group_dev,
                             const int32_t* row_lens_dev, void* meta_dev, int32_t update, void* stream);
 
+/* The three row arrays of fca_build_metadata_rows from what an engine keeps per request:
+ * query_start_loc_dev [num_reqs + 1] (cumulative query tokens, num_rows at the end) and
+ * seq_lens_dev [num_reqs] (tokens in the cache including the whole run).  Token i of a run
+ * of q tokens gets its request as table row, length seq_len - (q - 1 - i), and, for
+ * q >= 2, the group id request * max_blocks + (block its own token is in); single tokens
+ * get -1.  One launch, no host synchronisation.  In the reference this bookkeeping is
+ * host code on the trainer's side (cu_seqlens per response and per unique prompt,
+ * arctic_platform/rl/zorro_train/zorro_train.py:2059-2127). */
+int fca_rows_from_query_runs(const int32_t* query_start_loc_dev, const int32_t* seq_lens_dev, int32_t num_reqs,
+                             int32_t num_rows, int32_t max_blocks, int32_t* row_table_dev, int32_t* row_lens_dev,
+                             int32_t* row_group_dev, void* stream);
+
 /* Shared-prefix pass: work items of shared nodes only.  Writes normalised partial
  * outputs and natural-log LSEs into the slots the metadata assigns. */
 int fca_prefix_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev,

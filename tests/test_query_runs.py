@@ -260,6 +260,27 @@ def test_declared_groups_that_are_no_tiles(gpu):
 
 
 @pytest.mark.gpu
+def test_row_arrays_from_query_start_loc(gpu):
+    """The device-side bookkeeping (request, causal length and tile id of every query token)
+    against the plain loops of run_rows, bit for bit."""
+    from arctic_platform_amd.forest import rows_from_query_runs
+
+    rng = random.Random(9)
+    for max_blocks in (7, 64):
+        batch = []
+        for _ in range(rng.randint(1, 40)):
+            ql = rng.choice([1, 1, 1, 2, 5, 16, 17, 40])
+            batch.append((rng.randint(0, max_blocks * BLOCK - ql), ql))
+        want = run_rows(batch, max_blocks)
+        starts = torch.tensor([0] + [q for _, q in batch]).cumsum(0).to(torch.int32).to(gpu)
+        seq_lens = torch.tensor([c + q for c, q in batch], dtype=torch.int32, device=gpu)
+        got = rows_from_query_runs(starts, seq_lens, len(want[0]), max_blocks)
+        torch.cuda.synchronize()
+        for g, w in zip(got, want):
+            assert g.cpu().tolist() == w
+
+
+@pytest.mark.gpu
 def test_bad_row_table_is_flagged_not_followed(gpu):
     from arctic_platform_amd.forest import build_forest_metadata
 
