@@ -281,6 +281,53 @@ def test_row_arrays_from_query_start_loc(gpu):
 
 
 @pytest.mark.gpu
+def test_query_runs_under_graph_replay(gpu):
+    """Row arrays + build + attention of a mixed step captured in a HIP graph: nothing in it
+    allocates or waits for the host, and every replay on changed inputs (same buffers)
+    equals the eager result."""
+    from arctic_platform_amd.forest import build_forest_metadata, rows_from_query_runs
+    from arctic_platform_amd.ops import forest_cascade_decode
+
+    hq, hkv, d = 16, 4, 64
+    batch = [(40, 50), (100, 1), (7, 3), (64, 1), (0, 33)]
+    table, cache, q, _, _, max_blocks = _batch_on_gpu(gpu, 31, batch, hq, hkv, d, torch.bfloat16, share=((1, 3, 3),))
+    rows = q.shape[0]
+    starts = torch.tensor([0] + [n for _, n in batch]).cumsum(0).to(torch.int32).to(gpu)
+    seq_lens = torch.tensor([c + n for c, n in batch], dtype=torch.int32, device=gpu)
+    kw = dict(num_q_heads=hq, num_kv_heads=hkv, head_dim=d, chunk_tokens=32, rows_per_item=64)
+    bufs = tuple(torch.empty(rows, dtype=torch.int32, device=gpu) for _ in range(3))
+    out = torch.empty_like(q)
+
+    def step(md):
+        rt, rl, rg = rows_from_query_runs(starts, seq_lens, rows, max_blocks, out=bufs)
+        md = build_forest_metadata(table, rl, out=md, row_table=rt, row_group=rg, **kw)
+        forest_cascade_decode(q, cache, md, d**-0.5, out=out, return_lse=False)
+        return md
+
+    md = step(None)  # allocates the workspaces, outside the graph
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            step(md)
+    gen = torch.Generator(device=gpu).manual_seed(5)
+    for replay in range(4):
+        q.copy_(torch.randn(q.shape, generator=gen, device=gpu).to(q.dtype))
+        if replay >= 2:  # the same runs one token further back in their sequences
+            seq_lens.copy_(torch.tensor([c + n - 1 for c, n in batch], dtype=torch.int32, device=gpu))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        rt, rl, rg = rows_from_query_runs(starts, seq_lens, rows, max_blocks)
+        md_e = build_forest_metadata(table, rl, row_table=rt, row_group=rg, **kw)
+        want = forest_cascade_decode(q, cache, md_e, d**-0.5, return_lse=False)
+        torch.cuda.synchronize()
+        md_e.check()
+        assert torch.equal(got, want), f"replay {replay} differs from eager"
+
+
+@pytest.mark.gpu
 def test_bad_row_table_is_flagged_not_followed(gpu):
     from arctic_platform_amd.forest import build_forest_metadata
 
