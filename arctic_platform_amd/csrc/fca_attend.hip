@@ -443,7 +443,7 @@ hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dty
   // and the second wave per SIMD hides the arithmetic latency of a tile, which is what
   // limits a head that small (fp8 most of all).
   const int64_t max_tickets = (int64_t)plan.num_seqs *
-                              ((int64_t)plan.max_blocks * kBlock / plan.chunk_tokens + plan.max_levels + 1) *
+                              ((int64_t)plan.max_blocks * kBlock / plan.chunk_tokens + plan.max_levels + 2) *
                               plan.num_kv_heads;
   int grid = cached_cu_count() * workgroups_per_cu(plan.head_dim, fp8, plan.rows_per_item);
   if ((int64_t)grid * kWaves > max_tickets) grid = (int)((max_tickets + kWaves - 1) / kWaves);

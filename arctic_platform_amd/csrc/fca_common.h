@@ -67,7 +67,9 @@ inline __host__ MetaLayout make_layout(const fca_plan& p) {
     off = align_up(off + n, 4);  // keep every array 16-byte aligned
     return at;
   };
-  L.max_partials = (int64_t)p.max_blocks * kBlock / p.chunk_tokens + p.max_levels + 1;
+  // chunks of the nodes on a row's path: at most tokens / chunk plus one per node, and a path
+  // holds at most max_levels discovered nodes, one node of a declared group and the leaf
+  L.max_partials = (int64_t)p.max_blocks * kBlock / p.chunk_tokens + p.max_levels + 2;
   L.max_items = S * L.max_partials;
   L.header = take(kHeaderInts);
   L.seq_npart = take(S);

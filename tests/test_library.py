@@ -39,7 +39,7 @@ def test_workspace_sizes(lib):
     plan = make_plan(512, 320, 32, 8, 128, chunk_tokens=512, max_levels=4)
     layout = _lib.FcaMetaLayout()
     assert lib.fca_meta_describe(ctypes.byref(plan), ctypes.byref(layout)) == 0
-    assert layout.max_partials == 320 * 16 // 512 + 4 + 1
+    assert layout.max_partials == 320 * 16 // 512 + 4 + 2  # chunks + discovered levels + declared group + leaf
     assert layout.max_items == 512 * layout.max_partials
     nm, no, nl = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
     assert lib.fca_workspace_bytes(ctypes.byref(plan), ctypes.byref(nm), ctypes.byref(no), ctypes.byref(nl)) == 0
@@ -119,4 +119,4 @@ def test_header_is_plain_c_and_links(tmp_path):
     exe = tmp_path / "probe"
     subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", f"-I{inc}", str(src), f"-L{libdir}", "-lzorro_fca", f"-Wl,-rpath,{libdir}", "-o", str(exe)], check=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
-    assert int(out[0]) >= 1 and int(out[2]) == 512 * (320 * 16 // 1024 + 5) * 32 * 128 * 2
+    assert int(out[0]) >= 1 and int(out[2]) == 512 * (320 * 16 // 1024 + 6) * 32 * 128 * 2
