@@ -562,7 +562,9 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
     for (int s = tid; s < S; s += kBuildThreads) {
       const int tokens = max(0, tmp1[s] - pos[s] * kBlock);  // (none below a causal node)
       meta[L.seq_leaf_blk + s] = pos[s];
-      meta[L.seq_npart + s] = ord[s] + num_chunks_for(tokens, chunk);
+      const int npart = ord[s] + num_chunks_for(tokens, chunk);
+      meta[L.seq_npart + s] = npart;
+      if (npart > (int)L.max_partials) atomicOr(&hdr[H_ERROR], 8);  // (cannot happen: see make_layout)
       members[leaf_members + s] = s;
       leaf_tokens += (unsigned long long)tokens;
     }

@@ -63,6 +63,8 @@ class ForestMetadata:
             raise RuntimeError("work list overflowed its reserved size")
         if err & 4:
             raise ValueError("a row_table entry is outside the block table")
+        if err & 8:
+            raise RuntimeError("a row needs more partial slots than the plan reserves")
 
     def nodes(self) -> list:
         L, m = self.layout, self.meta.cpu()

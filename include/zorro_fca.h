@@ -97,7 +97,8 @@ typedef struct fca_meta_layout {
   int64_t header;        /* [16]: 0 items, 1 shared items, 2 nodes (shared), 3 work ticket
                             (self-resetting, owned by the attention kernel), 4 reserved,
                             5 error flags (1 bad length, 2 work list overflow, 4 bad row table
-                            entry), 6/7 unique tokens lo/hi, 8 levels found,
+                            entry, 8 partial slots of a row overflow), 6/7 unique tokens lo/hi,
+                            8 levels found,
                             10-13 and 15 state for fca_update_metadata, 14 updates since the
                             last full build */
   int64_t seq_npart;     /* [S] partial slots used per sequence */

@@ -260,6 +260,40 @@ def test_declared_groups_that_are_no_tiles(gpu):
 
 
 @pytest.mark.gpu
+def test_longest_path_fills_the_partial_slots_exactly(gpu):
+    """Two discovered levels, a node of a declared group below them and a leaf, every one a
+    chunk of its own: the rows use every partial slot the plan reserves."""
+    from arctic_platform_amd.forest import build_forest_metadata
+    from arctic_platform_amd.ops import forest_cascade_decode
+    from oracle.attention import flat_decode_attention
+    from tests.helpers import assert_matches_oracle
+
+    hq, hkv, d = 8, 2, 64
+    batch = [(59, 1), (62, 1), (40, 1), (33, 1)]  # four single-token rows over four-block tables
+    table, cache, q, _, _, max_blocks = _batch_on_gpu(gpu, 41, batch, hq, hkv, d, torch.bfloat16)
+    table = table[:, :4].contiguous()
+    table[1:, 0] = table[0, 0]  # everybody shares the first block,
+    table[1:3, 1] = table[0, 1]  # rows 0, 1 and 2 the second,
+    table[1, 2] = table[0, 2]  # rows 0 and 1 the third: one level more than discovery may take
+    row_lens = [60, 63, 41, 34]
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=gpu)
+    md = build_forest_metadata(
+        table, i32(row_lens), num_q_heads=hq, num_kv_heads=hkv, head_dim=d, chunk_tokens=1024, max_levels=2,
+        row_table=i32([0, 1, 2, 3]), row_group=i32([7, 7, -1, -1]),
+    )
+    out, lse = forest_cascade_decode(q, cache, md, d**-0.5)
+    torch.cuda.synchronize()
+    md.check()
+    nodes, leaves = discover_forest(table.cpu().tolist(), row_lens, max_levels=2, row_table=[0, 1, 2, 3], row_group=[7, 7, -1, -1])
+    assert canonical_nodes(md.nodes()) == canonical_nodes(nodes)
+    assert canonical_nodes(nodes) == sorted([((0, 1, 2, 3), 0, 1), ((0, 1, 2), 1, 1), ((0, 1), 2, 1)])
+    assert [l["tokens"] for l in md.leaves()] == [12, 15, 9, 18]
+    assert md.seq_num_partials()[:2] == [md.layout.max_partials] * 2 == [4, 4]
+    ref_out, ref_lse = flat_decode_attention(q.cpu(), cache.cpu(), table.cpu(), torch.tensor(row_lens), d**-0.5)
+    assert_matches_oracle(out, lse, ref_out, ref_lse, what="longest path")
+
+
+@pytest.mark.gpu
 def test_row_arrays_from_query_start_loc(gpu):
     """The device-side bookkeeping (request, causal length and tile id of every query token)
     against the plain loops of run_rows, bit for bit."""
