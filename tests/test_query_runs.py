@@ -154,6 +154,42 @@ def test_cover_invariant_on_random_batches():
                 assert len(ids) == 1
 
 
+def test_cpu_cascade_with_causal_nodes_equals_flat_attention():
+    """The decomposition the kernels run (shared nodes, causal tiles with every member
+    stopping at its own token, leaves, log-sum-exp merge), restated on the CPU in fp64,
+    equals flat attention row by row."""
+    from arctic_platform_amd.kv_layout import pack_blocks
+    from oracle.attention import flat_decode_attention
+    from oracle.cascade import cascade_decode_attention
+
+    rng = random.Random(3)
+    gen = torch.Generator().manual_seed(3)
+    hq, hkv, d, max_blocks = 4, 2, 64, 6
+    for trial in range(6):
+        nseq = rng.randint(2, 4)
+        nblocks = nseq * max_blocks
+        table = torch.randperm(nblocks, generator=gen).to(torch.int32).view(nseq, max_blocks)
+        if trial % 2:
+            table[1, :2] = table[0, :2]  # a cached prompt shared by the first two sequences
+        k = torch.randn(nblocks, BLOCK, hkv, d, generator=gen, dtype=torch.float64)
+        v = torch.randn(nblocks, BLOCK, hkv, d, generator=gen, dtype=torch.float64)
+        cache = pack_blocks(k, v, torch.float64)
+        batch = []
+        for s in range(nseq):
+            ql = rng.choice([1, 2, 5, 17, 30])
+            batch.append((rng.randint(32 if trial % 2 and s < 2 else 0, max_blocks * BLOCK - ql), ql))
+        row_table, row_lens, row_group = run_rows(batch, max_blocks)
+        q = torch.randn(len(row_table), hq, d, generator=gen, dtype=torch.float64)
+        lens = torch.tensor(row_lens, dtype=torch.int32)
+        ref_out, ref_lse = flat_decode_attention(q, cache, table[torch.tensor(row_table)], lens, 0.125)
+        for chunk in (None, 32):
+            out, lse, nodes, _ = cascade_decode_attention(
+                q, cache, table, lens, 0.125, chunk_tokens=chunk, row_table=row_table, row_group=row_group
+            )
+            assert torch.allclose(out, ref_out, rtol=0, atol=1e-10) and torch.allclose(lse, ref_lse, rtol=0, atol=1e-10)
+        assert any(n["causal"] for n in nodes) or all(ql == 1 for _, ql in batch)
+
+
 # ---------------------------------------------------------------------------------- GPU
 
 
