@@ -11,18 +11,25 @@ constexpr int kMergeThreads = 256;
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
-// D / 8 lanes per (sequence, query head) row; each lane owns 8 adjacent channels (16 bytes
-// of a half-precision partial row).  A partial row is its stored halves times the row's
-// scale; {lse, scale} sit side by side.
-template <int D>
+// D / 8 lanes per (sequence, query head) row and share; each lane owns 8 adjacent channels
+// (16 bytes of a half-precision partial row).  A partial row is its stored halves times the
+// row's scale; {lse, scale} sit side by side.  With SPLIT > 1 (plans with many partials per
+// row: long contexts cut into many chunks) SPLIT such lane groups take every SPLIT-th
+// partial of the row each and combine their running results at the end, which puts SPLIT
+// times the loads in flight.
+template <int D, int SPLIT>
 __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p) {
   constexpr int V = 8;
-  constexpr int kLanesPerRow = D / V;
+  constexpr int kLanesPerShare = D / V;
+  constexpr int kLanesPerRow = kLanesPerShare * SPLIT;
+  static_assert(kLanesPerRow <= 64, "the shares of a row combine inside one wave");
   const int row = blockIdx.x * (kMergeThreads / kLanesPerRow) + threadIdx.x / kLanesPerRow;
-  const int sub = threadIdx.x % kLanesPerRow;
-  if (row >= p.num_seqs * p.num_q_heads) return;
-  const int s = row / p.num_q_heads, hq = row - s * p.num_q_heads;
-  const int np = p.seq_npart[s];
+  const int sub = threadIdx.x % kLanesPerShare;
+  const int share = (threadIdx.x / kLanesPerShare) % SPLIT;
+  // (rows past the end keep running with no partials: the shares of a row exchange registers below)
+  const bool live_row = row < p.num_seqs * p.num_q_heads;
+  const int s = live_row ? row / p.num_q_heads : 0, hq = live_row ? row - s * p.num_q_heads : 0;
+  const int np = live_row ? p.seq_npart[s] : 0;
   const int64_t base = (int64_t)s * p.max_partials;
   const _Float16* rows = static_cast<const _Float16*>(p.partial_out);
   const float2* lse_scale = reinterpret_cast<const float2*>(p.partial_lse);
@@ -34,7 +41,7 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
 #pragma unroll
   for (int e = 0; e < V; ++e) acc[e] = 0.f;
 #pragma unroll 4
-  for (int i = 0; i < np; ++i) {
+  for (int i = share; i < np; i += SPLIT) {
     const int64_t pr = (base + i) * p.num_q_heads + hq;
     const float2 ls = lse_scale[pr];
     const f16x8 o = *reinterpret_cast<const f16x8*>(rows + pr * D + sub * V);
@@ -49,6 +56,19 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
     for (int e = 0; e < V; ++e) acc[e] = acc[e] * keep + ws * (float)o[e];
     m = m_new;
   }
+  // combine the shares: the same update with a whole running result in place of one partial
+#pragma unroll
+  for (int off = kLanesPerShare; off < kLanesPerRow; off <<= 1) {
+    const float m_o = __shfl_xor(m, off), wsum_o = __shfl_xor(wsum, off);
+    const float m_new = fmaxf(m, m_o);
+    const float keep = m > -INFINITY ? __expf(m - m_new) : 0.f;
+    const float take = m_o > -INFINITY ? __expf(m_o - m_new) : 0.f;
+    wsum = wsum * keep + wsum_o * take;
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = acc[e] * keep + __shfl_xor(acc[e], off) * take;
+    m = m_new;
+  }
+  if (!live_row || share != 0) return;
   const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
   const int64_t o = (int64_t)s * p.out_seq_stride + (int64_t)hq * p.out_head_stride + sub * V;
   if (p.out_dtype == FCA_F32) {
@@ -92,13 +112,18 @@ hipError_t launch_copy(const void* src, void* dst, size_t bytes, hipStream_t str
 
 hipError_t launch_merge(const MergeParams& p, hipStream_t stream) {
   const int rows = p.num_seqs * p.num_q_heads;
-  const int per_block = kMergeThreads / (p.head_dim / 8);
+  if (rows == 0) return hipSuccess;
+  // rows that can have many partials are merged by four lane groups each
+  const int split = p.max_partials >= 16 ? 4 : 1;
+  const int per_block = kMergeThreads / (p.head_dim / 8 * split);
   const int grid = (rows + per_block - 1) / per_block;
-  if (grid == 0) return hipSuccess;
-  if (p.head_dim == 128)
-    hipLaunchKernelGGL(fca_merge_kernel<128>, dim3(grid), dim3(kMergeThreads), 0, stream, p);
-  else
-    hipLaunchKernelGGL(fca_merge_kernel<64>, dim3(grid), dim3(kMergeThreads), 0, stream, p);
+#define FCA_MERGE(D_, S_) hipLaunchKernelGGL((fca_merge_kernel<D_, S_>), dim3(grid), dim3(kMergeThreads), 0, stream, p)
+  if (p.head_dim == 128) {
+    if (split == 4) FCA_MERGE(128, 4); else FCA_MERGE(128, 1);
+  } else {
+    if (split == 4) FCA_MERGE(64, 4); else FCA_MERGE(64, 1);
+  }
+#undef FCA_MERGE
   return hipGetLastError();
 }
 
