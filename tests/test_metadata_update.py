@@ -155,3 +155,43 @@ def test_decode_loop_with_updates(gpu, index):
         assert md.header()["updates"] == step + 1
         ref_out, ref_lse = oracle_for(w)
         assert_matches_oracle(out, lse, ref_out, ref_lse, what=f"decode step {step}")
+
+
+def test_update_with_a_row_table_and_none_with_declared_groups(gpu):
+    """Query rows over a row table keep their forest across an update like plain rows (the
+    fingerprints follow the row table).  The kept forest may share less than a fresh build
+    would (two rows of one sequence gain a common block when they cross a block boundary),
+    so the check is the attention result.  A build with declared groups leaves nothing to
+    keep, so an update on it is a full build with the same result."""
+    import dataclasses
+
+    from arctic_platform_amd.forest import build_forest_metadata
+    from arctic_platform_amd.ops import forest_cascade_decode
+
+    w = make_config(2, device=gpu, shrink=8)
+    kw = dict(num_q_heads=w.num_q_heads, num_kv_heads=w.num_kv_heads, head_dim=w.head_dim, chunk_tokens=64, rows_per_item=64)
+    S = w.num_seqs
+    # two query rows per sequence: the sequence without its last token, and all of it
+    row_table = torch.arange(S, device=gpu).repeat_interleave(2).to(torch.int32)
+    lens = torch.stack([w.seq_lens - 1, w.seq_lens], 1).reshape(-1).contiguous()
+    lens = (lens - 2).clamp_(min=1).contiguous()  # start two tokens back, then step forward
+    q = torch.randn(2 * S, w.num_q_heads, w.head_dim, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(gpu)
+    md = build_forest_metadata(w.block_table, lens, row_table=row_table, **kw)
+    for n in range(2):
+        lens = (lens + 1).contiguous()  # the next step: both rows one token further
+        md = build_forest_metadata(w.block_table.clone(), lens, out=md, update=True, row_table=row_table, **kw)  # (the table may move; ids stay)
+        out, lse = forest_cascade_decode(q, w.kv_cache, md, w.scale)
+        torch.cuda.synchronize()
+        md.check()
+        assert md.header()["updates"] == n + 1, "the update fell back to a full build"
+        rows = dataclasses.replace(w, q=q, block_table=w.block_table[row_table.long()], seq_lens=lens)
+        ref_out, ref_lse = oracle_for(rows)
+        assert_matches_oracle(out, lse, ref_out, ref_lse, what=f"row-table update {n}")
+    groups = (row_table * w.block_table.shape[1] + (lens - 1) // 16).to(torch.int32)
+    md2 = build_forest_metadata(w.block_table, lens, row_table=row_table, row_group=groups, **kw)
+    again = build_forest_metadata(w.block_table, lens, out=md2, update=True, row_table=row_table, row_group=groups, **kw)
+    fresh = build_forest_metadata(w.block_table, lens, row_table=row_table, row_group=groups, **kw)
+    torch.cuda.synchronize()
+    again.check()
+    assert again.header()["updates"] == 0 and _semantics(again) == _semantics(fresh)
+    assert any(n["causal"] for n in again.nodes())
