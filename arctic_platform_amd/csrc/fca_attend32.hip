@@ -160,6 +160,21 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
   load_lane_meta(a0, a1, a_blk, a_seq);
   bf16x8 qreg[KS], nq[KS];
   load_q(qreg, seq, r1.x, kvh);
+  // fp8 scales of an item's KV head: fetched one item ahead like the query rows (read at
+  // the start of an item they would be waited for on the spot, with every tile in flight).
+  // The loads are unconditional; without a scale array they read the query tensor and the
+  // value is dropped.
+  auto load_scales = [&](int head, float& ks, float& vs) {
+    if constexpr (FP8) {
+      const float* kp = p.k_scale ? p.k_scale + head : reinterpret_cast<const float*>(p.q);
+      const float* vp = p.v_scale ? p.v_scale + head : reinterpret_cast<const float*>(p.q);
+      const float k = kp[opaque_zero], v = vp[opaque_zero];
+      ks = p.k_scale ? k : 1.f;
+      vs = p.v_scale ? v : 1.f;
+    }
+  };
+  float k_scale = 1.f, v_scale = 1.f, next_k_scale = 1.f, next_v_scale = 1.f;
+  load_scales(kvh, k_scale, v_scale);
   KT kb0, kb1;
   VT vb0, vb1;
   {
@@ -198,7 +213,7 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
     float sc = p.scale * kLog2e;
-    if (FP8 && p.k_scale) sc *= p.k_scale[kvh];
+    if (FP8) sc *= k_scale;
 
     // One 32-token tile.  RAGGED is the variant for the single tile that may run past the
     // end of the chunk: it masks scores and zeroes V there; full tiles carry no mask code.
@@ -323,6 +338,7 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
     load_record(tc, c0, c1, ckvh);
     issue_ticket(round + 4);
     load_q(nq, a_seq, a1.x, akvh);
+    load_scales(akvh, next_k_scale, next_v_scale);
 
     // ---- the last pair: refills come from the next item (of a ticket past the end: from
     // the last record of the list, loads nobody uses)
@@ -345,8 +361,7 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
     // goes out in sixteen pieces, and back-to-back partial writes to one cache line cost a
     // wave several microseconds per item.
     {
-      float vs = 1.f;
-      if (FP8 && p.v_scale) vs = p.v_scale[kvh];
+      const float vs = FP8 ? v_scale : 1.f;
       const float l = lrow + __shfl_xor(lrow, 32);
       stage_partial_row<D>(strip, m, h, acc, vs / l, prow, (mrow + fast_log2(l)) * kLn2, p.partial_lse);
       __builtin_amdgcn_wave_barrier();
@@ -359,6 +374,7 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
     if (ta >= ntickets) break;
 #pragma unroll
     for (int i = 0; i < KS; ++i) qreg[i] = nq[i];
+    k_scale = next_k_scale, v_scale = next_v_scale;
     r0 = a0, r1 = a1, kvh = akvh, my_blk = a_blk, seq = a_seq;
     a0 = b0, a1 = b1, akvh = bkvh, a_blk = b_blk, a_seq = b_seq;
     b0 = c0, b1 = c1, bkvh = ckvh;
