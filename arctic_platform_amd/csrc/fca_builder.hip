@@ -236,7 +236,8 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   int* slot = meta + L.s_slot;
   int* tmp0 = meta + L.s_tmp0;
   int* tmp1 = meta + L.s_tmp1;
-  int* cbad = meta + L.s_nitems;  // per leader: some member breaks the pattern of a query-run tile
+  int* cbad = meta + L.s_nitems;  // per leader, raised by members: in discovery, the group is more than one query run;
+                                  // in the pass for declared groups, the group is no tile of a query run
   int* cmax = cbad + S;           // per leader: largest member row minus the leader's row
   unsigned long long* hkeys = reinterpret_cast<unsigned long long*>(meta + L.hash_keys);
   int* hmin = meta + L.hash_min;
