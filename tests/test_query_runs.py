@@ -267,6 +267,74 @@ def test_query_runs_match_oracle(gpu, case):
 
 
 @pytest.mark.gpu
+def test_random_batches_of_query_rows(gpu):
+    """Random shapes (head size, GQA group incl. 7, tile height, fp8, chunk, level cap),
+    random prefix sharing between sequences, random runs, tiles declared per block, no
+    declarations, arbitrary declarations across sequences, rows in shuffled order: the node
+    lists equal the oracle's and every row equals flat attention."""
+    from arctic_platform_amd.forest import build_forest_metadata
+    from arctic_platform_amd.kv_layout import kv_cache_shape
+    from arctic_platform_amd.ops import forest_cascade_decode
+    from oracle.attention import flat_decode_attention
+    from tests.helpers import assert_matches_oracle
+
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=gpu)
+    for seed in range(60):
+        rng = random.Random(seed)
+        gen = torch.Generator().manual_seed(seed)
+        d, hkv, g = rng.choice([64, 128]), rng.choice([1, 2, 4]), rng.choice([1, 2, 4, 7, 8, 16])
+        hq, rows_per_item, fp8 = hkv * g, rng.choice([32, 64]), rng.random() < 0.3
+        chunk, levels = rng.choice([32, 64, 128, 1024]), rng.choice([0, 1, 2, 4, 8])
+        nseq, max_blocks = rng.randint(1, 10), rng.randint(2, 14)
+        nblocks = nseq * max_blocks + 2
+        table = torch.randperm(nblocks, generator=gen).to(torch.int32)[: nseq * max_blocks].view(nseq, max_blocks).clone()
+        for s in range(1, nseq):  # a sequence may start with the blocks of an earlier one
+            if rng.random() < 0.6:
+                t, k = rng.randrange(s), rng.randint(1, max_blocks)
+                table[s, :k] = table[t, :k]
+        batch = []
+        for s in range(nseq):
+            ql = min(rng.choice([1, 1, 1, 2, 3, 5, 16, 17, 33]), max_blocks * BLOCK)
+            batch.append((rng.randint(0, max_blocks * BLOCK - ql), ql))
+        mode = rng.choice(["tiles", "tiles", "none", "odd"])
+        row_table, row_lens, row_group = run_rows(batch, max_blocks)
+        if mode == "odd":  # arbitrary declarations, across sequences too
+            row_group = [rng.randrange(3) for _ in row_group]
+        if rng.random() < 0.3:  # rows in any order: declared tiles then are not runs of adjacent rows
+            perm = list(range(len(row_table)))
+            rng.shuffle(perm)
+            row_table, row_lens, row_group = ([v[i] for i in perm] for v in (row_table, row_lens, row_group))
+        groups = None if mode == "none" else row_group
+        cache = torch.randn(kv_cache_shape(nblocks, BLOCK, hkv, d), generator=gen)
+        k_scale = v_scale = None
+        if fp8:
+            k_scale = (torch.rand(hkv, generator=gen) * 0.09 + 0.01).to(gpu)
+            v_scale = (torch.rand(hkv, generator=gen) * 0.09 + 0.01).to(gpu)
+            cache = (cache * 20).clamp(-448, 448).to(torch.float8_e4m3fn).to(gpu)
+        else:
+            cache = cache.to(torch.bfloat16).to(gpu)
+        q = torch.randn(len(row_table), hq, d, generator=gen).to(torch.bfloat16).to(gpu)
+        what = f"seed {seed}: D {d}, Hq {hq} / Hkv {hkv}, rows {rows_per_item}, fp8 {fp8}, chunk {chunk}, levels {levels}, {mode}"
+        md = build_forest_metadata(
+            table.to(gpu), i32(row_lens), num_q_heads=hq, num_kv_heads=hkv, head_dim=d, chunk_tokens=chunk, rows_per_item=rows_per_item,
+            max_levels=levels, row_table=i32(row_table), row_group=None if groups is None else i32(groups),
+        )
+        out, lse = forest_cascade_decode(q, cache, md, d**-0.5, k_scale, v_scale)
+        torch.cuda.synchronize()
+        md.check()
+        nodes, leaves = discover_forest(table.tolist(), row_lens, max_levels=levels, row_table=row_table, row_group=groups)
+        assert canonical_nodes(md.nodes()) == canonical_nodes(nodes), what
+        key = lambda ns: sorted((tuple(sorted(n["members"])), n["tokens"], n["causal"]) for n in ns)
+        assert key(md.nodes()) == key(nodes), what
+        assert [l["tokens"] for l in md.leaves()] == [l["tokens"] for l in leaves], what
+        ref_out, ref_lse = flat_decode_attention(
+            q.cpu(), cache.cpu(), table[torch.tensor(row_table)], torch.tensor(row_lens), d**-0.5,
+            None if k_scale is None else k_scale.cpu(), None if v_scale is None else v_scale.cpu(),
+        )
+        assert_matches_oracle(out, lse, ref_out, ref_lse, what=what)
+
+
+@pytest.mark.gpu
 def test_declared_groups_that_are_no_tiles(gpu):
     """Groups the caller declares across table rows (an explicit tree spec) and groups whose
     lengths do not form a run: shared node before the members' own blocks, private leaves."""
