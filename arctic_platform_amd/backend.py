@@ -51,10 +51,6 @@ class CommonAttentionMetadata:
     num_actual_tokens: int | None = None
 
 
-# Query runs up to this length count as decode for the choice of the row-tile height.
-MAX_DECODE_QUERY_LEN = 16
-
-
 @dataclasses.dataclass
 class ForestCascadeMetadata:
     forest: ForestMetadata
@@ -168,8 +164,12 @@ class ForestCascadeMetadataBuilder:
             update=update and row_group is None,
             row_table=row_table,
             row_group=row_group,
-            # short runs read a block about once per launch, like plain decode
-            kv_reread=m.max_query_len > MAX_DECODE_QUERY_LEN,
+            # With three or more query tokens per sequence the rows of a shared prompt usually
+            # fill more than one row tile, and every tile reads the prompt again: loads that
+            # stay in the caches then win (q = 4: 578 -> 516 us per layer at the 512-sequence
+            # shape, q = 8: 948 -> 742 us); one or two tokens read a block about once, like
+            # plain decode, and stream.
+            kv_reread=m.max_query_len > 2,
         )
         self._workspaces[key] = forest
         return ForestCascadeMetadata(forest=forest, slot_mapping=m.slot_mapping[:num_tokens], num_decode_tokens=num_tokens)
