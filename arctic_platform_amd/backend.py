@@ -60,11 +60,14 @@ class ForestCascadeMetadata:
 
 def parse_forest_cascade_configs(value) -> dict:
     """``forest_cascade_attn_configs`` arrives as a JSON string (``"{}"`` in the recipes)
-    or a dict.  Known keys: chunk_tokens, rows_per_item, max_levels, enable, rebuild_every."""
+    or a dict.  Known keys: chunk_tokens, rows_per_item, max_levels, enable, rebuild_every,
+    kv_reread (true: keep KV loads cacheable, for batches whose shared prompts carry more
+    query rows than one row tile holds, e.g. more than rows_per_item / (Hq / Hkv) samples per
+    prompt; false: stream; absent: decided per step from the query lengths)."""
     if value is None or value == "":
         return {}
     cfg = json.loads(value) if isinstance(value, str) else dict(value)
-    unknown = set(cfg) - {"chunk_tokens", "rows_per_item", "max_levels", "enable", "rebuild_every"}
+    unknown = set(cfg) - {"chunk_tokens", "rows_per_item", "max_levels", "enable", "rebuild_every", "kv_reread"}
     if unknown:
         raise ValueError(f"unknown forest_cascade_attn_configs keys: {sorted(unknown)}")
     return cfg
@@ -117,6 +120,7 @@ class ForestCascadeMetadataBuilder:
         self.chunk_tokens = int(cfg.get("chunk_tokens", 1024))
         self.max_levels = int(cfg.get("max_levels", 4))
         self.rebuild_every = max(1, int(cfg.get("rebuild_every", 32)))
+        self.kv_reread = None if cfg.get("kv_reread") is None else bool(cfg["kv_reread"])
         group = num_q_heads // num_kv_heads
         self.rows_per_item = int(cfg.get("rows_per_item", 64 if group > 32 else 32))
         # several query tokens per sequence multiply the rows of every shared node: unless the
@@ -169,7 +173,7 @@ class ForestCascadeMetadataBuilder:
             # stay in the caches then win (q = 4: 578 -> 516 us per layer at the 512-sequence
             # shape, q = 8: 948 -> 742 us); one or two tokens read a block about once, like
             # plain decode, and stream.
-            kv_reread=m.max_query_len > 2,
+            kv_reread=m.max_query_len > 2 if self.kv_reread is None else self.kv_reread,
         )
         self._workspaces[key] = forest
         return ForestCascadeMetadata(forest=forest, slot_mapping=m.slot_mapping[:num_tokens], num_decode_tokens=num_tokens)

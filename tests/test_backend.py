@@ -26,6 +26,9 @@ def test_backend_surface():
 def test_config_string_and_rejections():
     assert parse_forest_cascade_configs("{}") == {} and parse_forest_cascade_configs(None) == {}
     assert parse_forest_cascade_configs('{"chunk_tokens": 512}') == {"chunk_tokens": 512}
+    assert parse_forest_cascade_configs('{"kv_reread": true}') == {"kv_reread": True}
+    assert ForestCascadeMetadataBuilder(32, 8, 128, device="cpu", forest_cascade_attn_configs={"kv_reread": False}).kv_reread is False
+    assert ForestCascadeMetadataBuilder(32, 8, 128, device="cpu").kv_reread is None
     with pytest.raises(ValueError):
         parse_forest_cascade_configs({"bogus": 1})
     with pytest.raises(NotImplementedError):
