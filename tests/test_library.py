@@ -80,6 +80,19 @@ def test_block_size_and_null_pointers(lib):
     assert lib.fca_decode_step(ctypes.byref(plan), ctypes.byref(t), None, None, None, None, 0, 0, 0, None, None) == -1
 
 
+def test_row_entry_points_check_their_arguments(lib):
+    plan = make_plan(4, 8, 32, 8, 128)
+    one = ctypes.c_void_p(16)  # never dereferenced: the checks come first
+    # a row table needs the number of table rows
+    assert lib.fca_build_metadata_rows(ctypes.byref(plan), one, 8, 0, one, None, one, one, 0, None) == -1
+    assert "table_rows" in lib.fca_last_error().decode()
+    assert lib.fca_build_metadata_rows(ctypes.byref(plan), None, 8, 2, one, None, one, one, 0, None) == -1
+    assert lib.fca_rows_from_query_runs(one, one, 0, 4, 8, one, one, one, None) == -1
+    assert lib.fca_rows_from_query_runs(one, one, 1 << 20, 4, 1 << 12, one, one, one, None) == -2  # group ids need 32 bits
+    assert lib.fca_rows_from_query_runs(None, None, 2, 0, 8, None, None, None, None) == 0  # nothing to do
+    assert lib.fca_rows_from_query_runs(None, one, 2, 4, 8, one, one, one, None) == -1
+
+
 def test_operators_refuse_cpu_tensors():
     import torch
 
