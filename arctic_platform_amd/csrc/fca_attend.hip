@@ -183,21 +183,6 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 64)) void fca_a
     load_record(my_wave, r0, r1, kvh);
     load_lane_meta(r0, r1, my_blk, seq);
     load_q(seq, r1.x, kvh);
-    // fp8 scales of an item's KV head, fetched together with the item's query rows (read
-    // where they are used they would be waited for on the spot, with the next loads in
-    // flight).  The loads are unconditional; without a scale array they read the query
-    // tensor and the value is dropped.
-    auto load_scales = [&](int head, float& ks, float& vs) {
-      if constexpr (FP8) {
-        const float* kp = p.k_scale ? p.k_scale + head : reinterpret_cast<const float*>(p.q);
-        const float* vp = p.v_scale ? p.v_scale + head : reinterpret_cast<const float*>(p.q);
-        const float k = kp[opaque_zero], v = vp[opaque_zero];
-        ks = p.k_scale ? k : 1.f;
-        vs = p.v_scale ? v : 1.f;
-      }
-    };
-    float k_scale = 1.f, v_scale = 1.f;
-    load_scales(kvh, k_scale, v_scale);
     // The tile buffer, refilled in halves.
     KT kb;
     VT vb;
@@ -257,7 +242,7 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 64)) void fca_a
           for (int r = 0; r < 16; ++r) acc[rt][db][r] = 0.f;
       }
       float sc = p.scale * kLog2e;
-      if (FP8) sc *= k_scale;
+      if (FP8 && p.k_scale) sc *= p.k_scale[kvh];
 
       // One 32-token tile.  RAGGED is the variant for the single tile that may run past the
       // end of the chunk: it masks scores and zeroes V there; full tiles carry no mask code.
@@ -403,12 +388,10 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 64)) void fca_a
       if (trips < 2) load_record(t_next, n0, n1, nkvh);
       if (trips < 3) load_lane_meta(n0, n1, nmy_blk, nseq);
       const bool more = t_next < ntickets;
-      float next_k_scale = 1.f, next_v_scale = 1.f;
       if (more) {
         // q registers and the tile buffer are dead now: request the next item's query rows
         // and first tile before writing this item's partial
         load_q(nseq, n1.x, nkvh);
-        load_scales(nkvh, next_k_scale, next_v_scale);
         request_first_tiles(nmy_blk, __builtin_amdgcn_readfirstlane(n0.z), nkvh);
       }
 
@@ -416,7 +399,10 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 64)) void fca_a
       // query row, so normalisation is per lane.  The rows then pass through a wave-private
       // strip of LDS so that they leave as whole rows: stored straight from the accumulator
       // layout a row goes out in sixteen pieces, and partial writes of a cache line are slow.
-      const float vs = FP8 ? v_scale : 1.f;  // (this item's: the next item's are on their way)
+      // (The fp8 scales are read where they are used: this kernel has no register to carry
+      // them an item ahead, and its item boundaries wait for the loads in flight anyway.)
+      float vs = 1.f;
+      if (FP8 && p.v_scale) vs = p.v_scale[kvh];
 #pragma unroll
       for (int rt = 0; rt < NRT; ++rt) {
         if (rt > 0 && !two_tiles) continue;
@@ -428,7 +414,6 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 64)) void fca_a
       store_partial_rows<D, STREAM>(strip, rows, lane, p.partial_out);
       __builtin_amdgcn_wave_barrier();
       if (!more) break;
-      k_scale = next_k_scale, v_scale = next_v_scale;
       r0 = n0;
       r1 = n1;
       kvh = nkvh;

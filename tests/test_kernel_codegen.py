@@ -1,0 +1,72 @@
+"""Properties of the compiled attention kernels that the measured speed rests on, checked
+on the generated gfx950 assembly (no GPU needed): the kernels use no scratch memory, and
+inside the tile loop of the 32-row kernel no wait covers the tile that was requested last.
+
+gfx9 counts outstanding vector memory operations in order and the compiler sizes every
+wait for the shortest path to it, so a load that is issued on some paths only, or a value
+that has to be parked behind a load, silently turns a counted wait into a wait for
+everything in flight.  Nothing fails when that happens; the kernel just streams slower.
+"""
+
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "arctic_platform_amd", "csrc")
+FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "--cuda-device-only"]
+
+
+@pytest.fixture(scope="module")
+def hipcc():
+    exe = shutil.which("hipcc") or ("/opt/rocm/bin/hipcc" if os.path.exists("/opt/rocm/bin/hipcc") else None)
+    if exe is None:
+        pytest.skip("no hipcc")
+    return exe
+
+
+def _functions(asm):
+    """name -> body of every kernel in an assembly listing."""
+    out = {}
+    for m in re.finditer(r"^(_ZN3fca\w+):[^\n]*\n(.*?)^\.Lfunc_end", asm, flags=re.M | re.S):
+        out[m.group(1)] = m.group(2)
+    return out
+
+
+def test_attention_kernels_use_no_scratch(hipcc, tmp_path):
+    for src in ("fca_attend32.hip", "fca_attend.hip"):
+        res = subprocess.run(
+            [hipcc, *FLAGS, "-c", "-Rpass-analysis=kernel-resource-usage", os.path.join(CSRC, src), "-o", str(tmp_path / "o.o")],
+            capture_output=True, text=True, cwd=CSRC,
+        )
+        assert res.returncode == 0, res.stderr[-2000:]
+        sizes = re.findall(r"ScratchSize \[bytes/lane\]: (\d+)", res.stderr)
+        assert len(sizes) == 8 and set(sizes) == {"0"}, (src, sizes)
+
+
+def test_tile_loop_of_the_32_row_kernel_keeps_a_tile_in_flight(hipcc, tmp_path):
+    out = tmp_path / "a32.s"
+    res = subprocess.run([hipcc, *FLAGS, "-S", os.path.join(CSRC, "fca_attend32.hip"), "-o", str(out)], capture_output=True, text=True, cwd=CSRC)
+    assert res.returncode == 0, res.stderr[-2000:]
+    kernels = _functions(out.read_text())
+    # <head size 128, bf16, streaming>: the kernel of the headline configuration
+    name = "_ZN3fca19fca_attend32_kernelILi128ELb0ELb1EEEvNS_12AttendParamsE"
+    assert name in kernels, sorted(kernels)
+    loads_per_tile = 16  # 8 K + 2 x 4 V loads of 16 bytes per lane
+    seen = 0
+    for block in re.split(r"^\.LBB", kernels[name], flags=re.M):
+        header = block.split("\n", 1)[0]
+        if "Depth=2" not in header:  # the tile loop is the only loop nested inside the item loop that holds MFMAs
+            continue
+        if "v_mfma" not in block:
+            continue
+        waits = [int(n) for n in re.findall(r"s_waitcnt vmcnt\((\d+)\)", block)]
+        assert waits, header
+        # every wait inside the loop leaves at least the loads of one whole tile outstanding
+        assert min(waits) >= loads_per_tile, (header, waits)
+        assert len(re.findall(r"global_load_dwordx4", block)) == loads_per_tile, header
+        seen += 1
+    assert seen >= 1
