@@ -26,6 +26,7 @@ the trainer is the in-tree counterpart
 
 from __future__ import annotations
 
+import collections
 import dataclasses
 import json
 
@@ -103,11 +104,14 @@ class ForestCascadeAttentionBackend:
 
 class ForestCascadeMetadataBuilder:
     """Makes the forest metadata once per scheduler step.  Workspaces are kept per batch
-    shape (num_reqs, max_blocks), so a steady decode loop allocates nothing.  A step on a
+    shape (num_reqs, max_blocks), so a steady decode loop allocates nothing; the least
+    recently used ones are dropped beyond ``MAX_KEPT_WORKSPACES`` shapes.  A step on a
     shape seen before asks for an update: the device keeps the forest of the last build when
     the rows still carry it (sequences only grew) and builds anew otherwise.  Every
     ``rebuild_every``-th step is a full build regardless, so sharing that appeared since
     (a new request with a cached prompt) is picked up."""
+
+    MAX_KEPT_WORKSPACES = 16
 
     def __init__(self, num_q_heads, num_kv_heads, head_dim, device="cuda", forest_cascade_attn_configs=None):
         cfg = parse_forest_cascade_configs(forest_cascade_attn_configs)
@@ -128,8 +132,16 @@ class ForestCascadeMetadataBuilder:
         self.rows_multi_token = int(cfg.get("rows_per_item", 64))
         if group > self.rows_per_item:
             raise ValueError(f"{group} query heads per KV head do not fit rows_per_item={self.rows_per_item}")
-        self._workspaces: dict = {}
+        self._workspaces: collections.OrderedDict = collections.OrderedDict()
         self._steps_since_build: dict = {}
+
+    def _keep(self, key, value):
+        """Remember a workspace; forget the least recently used ones beyond the cap."""
+        self._workspaces[key] = value
+        self._workspaces.move_to_end(key)
+        while len(self._workspaces) > self.MAX_KEPT_WORKSPACES:
+            old, _ = self._workspaces.popitem(last=False)
+            self._steps_since_build.pop(old, None)
 
     def build(self, common_prefix_len: int, common_attn_metadata: CommonAttentionMetadata) -> ForestCascadeMetadata:
         m = common_attn_metadata
@@ -145,7 +157,8 @@ class ForestCascadeMetadataBuilder:
             num_tokens = m.num_actual_tokens if m.num_actual_tokens is not None else int(starts[-1])
             rows_key = (num_tokens, "rows")
             if rows_key not in self._workspaces:
-                self._workspaces[rows_key] = tuple(torch.empty(num_tokens, dtype=torch.int32, device=bt.device) for _ in range(3))
+                self._keep(rows_key, tuple(torch.empty(num_tokens, dtype=torch.int32, device=bt.device) for _ in range(3)))
+            self._workspaces.move_to_end(rows_key)
             row_table, sl, row_group = rows_from_query_runs(
                 starts.to(torch.int32).contiguous(), sl.contiguous(), num_tokens, bt.shape[1], out=self._workspaces[rows_key]
             )
@@ -175,7 +188,7 @@ class ForestCascadeMetadataBuilder:
             # plain decode, and stream.
             kv_reread=m.max_query_len > 2 if self.kv_reread is None else self.kv_reread,
         )
-        self._workspaces[key] = forest
+        self._keep(key, forest)
         return ForestCascadeMetadata(forest=forest, slot_mapping=m.slot_mapping[:num_tokens], num_decode_tokens=num_tokens)
 
 

@@ -43,6 +43,15 @@ def test_config_string_and_rejections():
         builder.build(0, meta)
 
 
+def test_workspace_cache_is_bounded():
+    b = ForestCascadeMetadataBuilder(32, 8, 128, device="cpu")
+    for shape in range(3 * b.MAX_KEPT_WORKSPACES):
+        b._steps_since_build[shape] = 0
+        b._keep(shape, object())
+    assert len(b._workspaces) == b.MAX_KEPT_WORKSPACES and len(b._steps_since_build) == b.MAX_KEPT_WORKSPACES
+    assert list(b._workspaces)[0] == 2 * b.MAX_KEPT_WORKSPACES  # the oldest went first
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("index", [2, 5])
 def test_decode_loop_through_backend(gpu, index):
