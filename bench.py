@@ -86,9 +86,11 @@ def time_steps(torch, ops, build, w, caches, md, out, lse, steps, warmup, layers
     return wall, kernel_us
 
 
-def cpu_baseline(torch, w, nseq):
+def cpu_baseline(torch, w, nseq, gpu_out=None):
     """The oracle's flat attention (fp32, every sequence gathers its own pages, no
-    sharing exploited) on the first ``nseq`` sequences, scaled to the whole batch."""
+    sharing exploited) on the first ``nseq`` sequences, scaled to the whole batch.  With
+    ``gpu_out`` (the timed path's output rows of those sequences) the oracle's result also
+    checks it, to the parity tolerance of the tests."""
     from oracle.attention import flat_decode_attention
 
     cores = os.cpu_count() or 1
@@ -107,7 +109,7 @@ def cpu_baseline(torch, w, nseq):
     times = []
     for it in range(3):
         t0 = time.perf_counter()
-        flat_decode_attention(q, cache, table, lens, w.scale, ks, vs, dtype=torch.float32)
+        ref_out, _ = flat_decode_attention(q, cache, table, lens, w.scale, ks, vs, dtype=torch.float32)
         times.append(time.perf_counter() - t0)
     sample_s = median(times[1:]) if len(times) > 1 else times[0]
     scale_up = float(w.seq_lens.sum()) / float(lens.sum())
@@ -118,6 +120,11 @@ def cpu_baseline(torch, w, nseq):
     t0 = time.perf_counter()
     cascade_decode_attention(q, cache, table, lens, w.scale, ks, vs, dtype=torch.float32)
     cascade_s = time.perf_counter() - t0
+    err = None
+    if gpu_out is not None:
+        diff = (gpu_out.cpu().float() - ref_out.float()).abs()
+        err = float(diff.max())
+        assert bool((diff <= 2e-2 + 2e-2 * ref_out.float().abs()).all()), f"timed output differs from the oracle: max |err| {err}"
     return {
         "value": sample_s * scale_up * 1e6,
         "unit": "us/step",
@@ -126,6 +133,7 @@ def cpu_baseline(torch, w, nseq):
         "sample": f"first {nseq} of {w.num_seqs} sequences ({int(lens.sum())} of {int(w.seq_lens.sum())} gathered tokens), "
         f"flat fp32 attention on torch-CPU, {sample_s:.2f} s measured, scaled by tokens x{scale_up:.2f}",
         "cascade_restatement_us": cascade_s * scale_up * 1e6,
+        "max_abs_err_of_timed_output": err,
     }
 
 
@@ -200,7 +208,9 @@ def main_query_runs(args):
     t0 = time.perf_counter()
     ref_out, _ = flat_decode_attention(q[idx.to(dev)].cpu(), caches[0].cpu(), table.cpu()[row_table.cpu()[idx].long()], lens.cpu()[idx], scale, dtype=torch.float32)
     cpu_s = time.perf_counter() - t0
-    err = float((out[idx.to(dev)].cpu().float() - ref_out).abs().max())
+    diff = (out[idx.to(dev)].cpu().float() - ref_out).abs()
+    err = float(diff.max())
+    assert bool((diff <= 2e-2 + 2e-2 * ref_out.abs()).all()), f"timed output differs from the oracle: max |err| {err}"
     scale_up = float(lens.double().sum()) / float(lens.cpu()[idx].double().sum())
     hdr = md.header()
     print(json.dumps({
@@ -260,6 +270,7 @@ def main():
 
     wall, kern_us = time_steps(torch, ops, refresh, w, caches, md, out, None, args.steps, args.warmup, args.layers)
     step_us = wall / args.steps * 1e6
+    checked_rows = out[: max(0, min(args.cpu_seqs, w.num_seqs))].clone()  # compared with the oracle below
     kern = sum(kern_us) / len(kern_us)
 
     # builder and merge on their own, for the breakdown
@@ -395,7 +406,7 @@ def main():
         del nc
 
     if args.cpu_seqs > 0:
-        result["cpu_baseline"] = cpu_baseline(torch, w, args.cpu_seqs)
+        result["cpu_baseline"] = cpu_baseline(torch, w, args.cpu_seqs, checked_rows)
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result))
