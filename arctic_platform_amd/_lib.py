@@ -33,7 +33,21 @@ EXPORTS = (
     "fca_decode_step",
     "fca_append_kv",
     "fca_calibration_copy",
+    "fca_split_layout_ints",
+    "fca_split_layout_build",
+    "fca_split_workspace_bytes",
+    "fca_split_attention_forward",
+    "fca_split_attention_backward",
 )
+
+
+class FcaSplitPlan(ctypes.Structure):
+    _fields_ = [
+        ("num_tokens", ctypes.c_int32),
+        ("num_q_heads", ctypes.c_int32),
+        ("num_kv_heads", ctypes.c_int32),
+        ("head_dim", ctypes.c_int32),
+    ]
 
 
 class FcaPlan(ctypes.Structure):
@@ -144,6 +158,14 @@ def load_library() -> ctypes.CDLL:
     lib.fca_decode_step.argtypes = [P(FcaPlan), P(FcaTensors), VP, VP, VP, VP, I64, I64, I32, VP, VP]
     lib.fca_append_kv.argtypes = [VP, VP, I64, I64, I32, I32, I32, VP, VP, VP, I64, I64, I32, VP, VP, VP]
     lib.fca_calibration_copy.argtypes = [VP, VP, ctypes.c_size_t, VP]
+    F32 = ctypes.c_float
+    lib.fca_split_layout_ints.argtypes = [I32, P(I64)]
+    lib.fca_split_layout_build.argtypes = [I32, VP, VP, VP, I32, VP]
+    lib.fca_split_workspace_bytes.argtypes = [P(FcaSplitPlan), SZ, SZ]
+    lib.fca_split_attention_forward.argtypes = [P(FcaSplitPlan), VP, I64, VP, I64, VP, I64, VP, F32, VP, VP, I64, VP, VP]
+    lib.fca_split_attention_backward.argtypes = (
+        [P(FcaSplitPlan)] + [VP, I64] * 5 + [VP, VP, F32, VP] + [VP, I64] * 3 + [VP]
+    )
     for name in EXPORTS:
         if name not in ("fca_version", "fca_last_error"):
             getattr(lib, name).restype = ctypes.c_int

@@ -319,3 +319,143 @@ int fca_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void*
 }
 
 }  // extern "C"
+
+namespace {
+int check_split(const fca_split_plan* p) {
+  if (!p) return fail(FCA_ERR_INVALID_ARG, "plan is NULL");
+  if (p->num_tokens < 0 || p->num_tokens > (1 << 30)) return fail(FCA_ERR_INVALID_ARG, "num_tokens %d is out of range", p->num_tokens);
+  if (p->head_dim != 64 && p->head_dim != 128)
+    return fail(FCA_ERR_UNSUPPORTED, "head_dim %d is not supported (64 or 128)", p->head_dim);
+  if (p->num_kv_heads < 1 || p->num_q_heads < p->num_kv_heads || p->num_q_heads % p->num_kv_heads)
+    return fail(FCA_ERR_INVALID_ARG, "num_q_heads %d must be a positive multiple of num_kv_heads %d", p->num_q_heads,
+                p->num_kv_heads);
+  return FCA_OK;
+}
+int check_rows(const char* name, const void* ptr, int64_t stride, int heads, int head_dim) {
+  if (!ptr) return fail(FCA_ERR_INVALID_ARG, "%s is NULL", name);
+  if ((reinterpret_cast<uintptr_t>(ptr) & 15) || stride % 8 || stride < (int64_t)heads * head_dim)
+    return fail(FCA_ERR_INVALID_ARG, "%s must be 16-byte aligned with a row stride that is a multiple of 8 and at least heads * head_dim", name);
+  return FCA_OK;
+}
+struct SplitScratch {
+  size_t kv_tiles, q_tiles, delta;  // bytes
+};
+SplitScratch split_scratch(const fca_split_plan* p) {
+  const size_t padded = 32 * (size_t)((p->num_tokens + 31) / 32);
+  return {padded * p->num_kv_heads * p->head_dim * 2, padded * p->num_q_heads * p->head_dim * 2, padded * p->num_q_heads * 4};
+}
+}  // namespace
+
+extern "C" {
+
+int fca_split_layout_ints(int32_t num_tokens, int64_t* num_ints) {
+  if (num_tokens < 0 || !num_ints) return fail(FCA_ERR_INVALID_ARG, "num_tokens must be >= 0 and num_ints non-NULL");
+  *num_ints = fca::make_split_layout((num_tokens + 31) / 32).total;
+  return FCA_OK;
+}
+
+int fca_split_layout_build(int32_t num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,
+                           const int32_t* response_tokens, int32_t num_tokens, int32_t* layout_host) {
+  if (num_groups < 0 || num_tokens < 0) return fail(FCA_ERR_INVALID_ARG, "num_groups and num_tokens must be >= 0");
+  if (num_groups > 0 && (!prompt_tokens || !group_sizes)) return fail(FCA_ERR_INVALID_ARG, "prompt_tokens and group_sizes must be non-NULL");
+  int64_t total = 0, samples = 0;
+  for (int g = 0; g < num_groups; ++g) {
+    if (prompt_tokens[g] < 0 || group_sizes[g] < 0) return fail(FCA_ERR_INVALID_ARG, "group %d has a negative count", g);
+    total += prompt_tokens[g];
+    for (int s = 0; s < group_sizes[g]; ++s) {
+      if (!response_tokens || response_tokens[samples + s] < 0)
+        return fail(FCA_ERR_INVALID_ARG, "response_tokens is NULL or negative for sample %lld", (long long)(samples + s));
+      total += response_tokens[samples + s];
+    }
+    samples += group_sizes[g];
+  }
+  if (total != num_tokens)
+    return fail(FCA_ERR_INVALID_ARG, "the layout holds %lld tokens, num_tokens says %d", (long long)total, num_tokens);
+  if (num_tokens == 0) return FCA_OK;
+  if (!layout_host) return fail(FCA_ERR_INVALID_ARG, "layout_host is NULL");
+  fca::build_split_layout(num_groups, prompt_tokens, group_sizes, response_tokens, (num_tokens + 31) / 32, layout_host);
+  return FCA_OK;
+}
+
+int fca_split_workspace_bytes(const fca_split_plan* plan, size_t* forward_bytes, size_t* backward_bytes) {
+  if (int rc = check_split(plan)) return rc;
+  const SplitScratch s = split_scratch(plan);
+  if (forward_bytes) *forward_bytes = s.kv_tiles;
+  if (backward_bytes) *backward_bytes = s.kv_tiles + 2 * s.q_tiles + s.delta;
+  return FCA_OK;
+}
+
+int fca_split_attention_forward(const fca_split_plan* plan, const void* q_dev, int64_t q_stride, const void* k_dev,
+                                int64_t k_stride, const void* v_dev, int64_t v_stride, const int32_t* layout_dev,
+                                float scale, void* workspace_dev, void* out_dev, int64_t out_stride, float* lse_dev,
+                                void* stream) {
+  if (int rc = check_split(plan)) return rc;
+  if (plan->num_tokens == 0) return FCA_OK;
+  if (!(scale > 0.f)) return fail(FCA_ERR_INVALID_ARG, "scale must be positive");
+  if (int rc = check_rows("q", q_dev, q_stride, plan->num_q_heads, plan->head_dim)) return rc;
+  if (int rc = check_rows("k", k_dev, k_stride, plan->num_kv_heads, plan->head_dim)) return rc;
+  if (int rc = check_rows("v", v_dev, v_stride, plan->num_kv_heads, plan->head_dim)) return rc;
+  if (int rc = check_rows("out", out_dev, out_stride, plan->num_q_heads, plan->head_dim)) return rc;
+  if (!layout_dev || !workspace_dev || !lse_dev || (reinterpret_cast<uintptr_t>(layout_dev) & 15) ||
+      (reinterpret_cast<uintptr_t>(workspace_dev) & 15) || (reinterpret_cast<uintptr_t>(lse_dev) & 15))
+    return fail(FCA_ERR_INVALID_ARG, "layout, workspace and lse must be non-NULL and 16-byte aligned");
+  fca::SplitParams p{};
+  p.q = q_dev, p.k = k_dev, p.v = v_dev;
+  p.q_stride = q_stride, p.k_stride = k_stride, p.v_stride = v_stride, p.o_stride = out_stride;
+  p.vt = workspace_dev;
+  p.out = out_dev;
+  p.lse = lse_dev;
+  p.layout = layout_dev;
+  p.num_tokens = plan->num_tokens;
+  p.num_tiles = (plan->num_tokens + 31) / 32;
+  p.num_q_heads = plan->num_q_heads;
+  p.num_kv_heads = plan->num_kv_heads;
+  p.scale = scale;
+  hipError_t e = fca::launch_split_forward(p, plan->head_dim, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? FCA_OK : hip_fail(e, "split attention forward launch");
+}
+
+int fca_split_attention_backward(const fca_split_plan* plan, const void* q_dev, int64_t q_stride, const void* k_dev,
+                                 int64_t k_stride, const void* v_dev, int64_t v_stride, const void* out_dev,
+                                 int64_t out_stride, const void* dout_dev, int64_t dout_stride, const float* lse_dev,
+                                 const int32_t* layout_dev, float scale, void* workspace_dev, void* dq_dev,
+                                 int64_t dq_stride, void* dk_dev, int64_t dk_stride, void* dv_dev, int64_t dv_stride,
+                                 void* stream) {
+  if (int rc = check_split(plan)) return rc;
+  if (plan->num_tokens == 0) return FCA_OK;
+  if (!(scale > 0.f)) return fail(FCA_ERR_INVALID_ARG, "scale must be positive");
+  const int hq = plan->num_q_heads, hkv = plan->num_kv_heads, d = plan->head_dim;
+  if (int rc = check_rows("q", q_dev, q_stride, hq, d)) return rc;
+  if (int rc = check_rows("k", k_dev, k_stride, hkv, d)) return rc;
+  if (int rc = check_rows("v", v_dev, v_stride, hkv, d)) return rc;
+  if (int rc = check_rows("out", out_dev, out_stride, hq, d)) return rc;
+  if (int rc = check_rows("dout", dout_dev, dout_stride, hq, d)) return rc;
+  if (int rc = check_rows("dq", dq_dev, dq_stride, hq, d)) return rc;
+  if (int rc = check_rows("dk", dk_dev, dk_stride, hkv, d)) return rc;
+  if (int rc = check_rows("dv", dv_dev, dv_stride, hkv, d)) return rc;
+  if (!layout_dev || !workspace_dev || !lse_dev || (reinterpret_cast<uintptr_t>(layout_dev) & 15) ||
+      (reinterpret_cast<uintptr_t>(workspace_dev) & 15) || (reinterpret_cast<uintptr_t>(lse_dev) & 15))
+    return fail(FCA_ERR_INVALID_ARG, "layout, workspace and lse must be non-NULL and 16-byte aligned");
+  const SplitScratch s = split_scratch(plan);
+  char* ws = static_cast<char*>(workspace_dev);
+  fca::SplitParams p{};
+  p.q = q_dev, p.k = k_dev, p.v = v_dev, p.out_in = out_dev, p.dout = dout_dev;
+  p.q_stride = q_stride, p.k_stride = k_stride, p.v_stride = v_stride, p.o_stride = out_stride, p.do_stride = dout_stride;
+  p.kt = ws;
+  p.qt = ws + s.kv_tiles;
+  p.dot = ws + s.kv_tiles + s.q_tiles;
+  p.delta = reinterpret_cast<float*>(ws + s.kv_tiles + 2 * s.q_tiles);
+  p.lse = const_cast<float*>(lse_dev);
+  p.dq = dq_dev, p.dk = dk_dev, p.dv = dv_dev;
+  p.dq_stride = dq_stride, p.dk_stride = dk_stride, p.dv_stride = dv_stride;
+  p.layout = layout_dev;
+  p.num_tokens = plan->num_tokens;
+  p.num_tiles = (plan->num_tokens + 31) / 32;
+  p.num_q_heads = hq;
+  p.num_kv_heads = hkv;
+  p.scale = scale;
+  hipError_t e = fca::launch_split_backward(p, d, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? FCA_OK : hip_fail(e, "split attention backward launch");
+}
+
+}  // extern "C"

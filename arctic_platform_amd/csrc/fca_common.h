@@ -181,6 +181,42 @@ struct AppendParams {
   int32_t num_tokens, num_kv_heads, head_dim;
 };
 
+// Split attention over packed training tensors (fca_split.hip).  Tensors are [T, H, D]
+// bf16 with a token stride; `t` tensors are transposed tile copies [H][tiles][D][32].
+struct SplitParams {
+  const void *q, *k, *v, *out_in, *dout;
+  int64_t q_stride, k_stride, v_stride, o_stride, do_stride;  // token strides, elements
+  const void *kt, *vt, *qt, *dot;
+  void* out;
+  float* lse;    // [Hq][tiles * 32] natural log
+  float* delta;  // [Hq][tiles * 32] rowsum(dout * out)
+  void *dq, *dk, *dv;
+  int64_t dq_stride, dk_stride, dv_stride;
+  const int32_t* layout;
+  int32_t num_tokens, num_tiles, num_q_heads, num_kv_heads;
+  float scale;
+};
+// Offsets into the int32 layout array of a batch of `tiles` 32-token tiles.
+struct SplitLayout {
+  int64_t kv_lim, q_tiles, kv_qend, q_order, kv_order, total;
+};
+__host__ __device__ inline SplitLayout make_split_layout(int64_t tiles) {
+  SplitLayout L;
+  L.kv_lim = 0;
+  L.q_tiles = 32 * tiles;
+  L.kv_qend = L.q_tiles + 4 * tiles;
+  L.q_order = L.kv_qend + tiles;
+  L.kv_order = L.q_order + tiles;
+  L.total = L.kv_order + tiles;
+  return L;
+}
+void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,
+                        const int32_t* response_tokens, int64_t tiles, int32_t* out);
+hipError_t launch_split_transpose(const void* x, int64_t stride, int heads, int head_dim, int num_tokens, int tiles,
+                                  void* xt, hipStream_t stream);
+hipError_t launch_split_forward(const SplitParams& p, int head_dim, hipStream_t stream);
+hipError_t launch_split_backward(const SplitParams& p, int head_dim, hipStream_t stream);
+
 hipError_t launch_build(const BuildParams& p, hipStream_t stream);
 hipError_t launch_rows(const int32_t* query_start_loc, const int32_t* seq_lens, int num_reqs, int num_rows, int max_blocks,
                        int32_t* row_table, int32_t* row_lens, int32_t* row_group, hipStream_t stream);

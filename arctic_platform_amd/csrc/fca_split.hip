@@ -1,0 +1,470 @@
+// Split attention of the trainer over a deduplicated, unpadded batch, forward and backward,
+// for gfx950.  Token order: for every prompt group the prompt once, then the response of
+// every sample of the group (arctic_platform/rl/zorro_train/zorro_train.py:311-356).  A
+// prompt row attends causally to its prompt; a response row attends to the whole prompt of
+// its group and causally to its own response
+// (arctic_platform/rl/zorro_train/qwen_attention_patcher.py:1198-1228, where the second
+// call gets one copy of the prompt's K and V per sample).  Here nothing is copied per
+// sample: since a group's responses follow its prompt, "row r attends to key t" is
+//     t <= r < lim(t),   lim(t) = end of the group for a prompt token,
+//                                 end of its own response for a response token,
+// one int per key.  Work is cut into tiles of 32 consecutive tokens of the packed order; a
+// tile may straddle segments, the per-element test above sorts that out.
+//
+// Kernels, one wave per (tile, head), no workgroup barrier, operands straight from global
+// memory into MFMA operand registers (mfma_f32_32x32x16_bf16):
+//   forward    per query tile, over the key tiles it can see (two ranges: the prompt's
+//              tiles, then from the tile its own segment starts in up to its own):
+//              St[tok x row] = K . Qt, online softmax per lane, Ot[d x row] += Vt . Pt
+//   dq         per query tile, the same walk: Pt from the saved log-sum-exp,
+//              dPt = V . dOt, dSt = Pt (dPt - delta), dQt[d x row] += Kt . dSt
+//   dk, dv     per key tile, over the query tiles that can see it (one range) and the query
+//              heads of its KV head: S[row x tok] = Q . Kt', P, dP = dO . Vt',
+//              dVt[d x tok] += dOt . P, dKt[d x tok] += Qt . dS; a prompt's dK and dV
+//              collect every sample of the group in registers and are written once
+// The second product of each chain contracts over tokens (or rows), which a [T, H, D]
+// tensor does not hold contiguously: a transposing pass first writes the tiles
+// [H][tile][D][32] of V (forward), of K, Q and dO (backward), zero past the last token.
+// The first product feeds its rows in the order that makes its output registers the B
+// operand of the second, so probabilities never leave registers.
+#include <algorithm>
+#include <numeric>
+#include <type_traits>
+#include <vector>
+
+#include "fca_attend_common.h"
+
+namespace fca {
+
+// ---- host: the layout array ------------------------------------------------------------
+void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,
+                        const int32_t* response_tokens, int64_t tiles, int32_t* out) {
+  const SplitLayout L = make_split_layout(tiles);
+  const int64_t padded = 32 * tiles;
+  std::vector<int32_t> own(padded, 0), pstart(padded, 0), pend(padded, 0);
+  int32_t* lim = out + L.kv_lim;
+  int64_t t = 0;
+  int64_t ri = 0;
+  auto fill = [&](int64_t from, int64_t to, int64_t limit, int64_t p0, int64_t p1) {
+    for (int64_t x = from; x < to; ++x) {
+      lim[x] = (int32_t)limit;
+      own[x] = (int32_t)from;
+      pstart[x] = (int32_t)p0;
+      pend[x] = (int32_t)p1;
+    }
+  };
+  for (int g = 0; g < num_groups; ++g) {
+    const int64_t p0 = t, p1 = t + prompt_tokens[g];
+    int64_t gend = p1;
+    for (int s = 0; s < group_sizes[g]; ++s) gend += response_tokens[ri + s];
+    fill(p0, p1, gend, p0, p1);
+    t = p1;
+    for (int s = 0; s < group_sizes[g]; ++s) {
+      const int64_t s1 = t + response_tokens[ri + s];
+      fill(t, s1, s1, p0, p1);
+      t = s1;
+    }
+    ri += group_sizes[g];
+  }
+  for (int64_t x = t; x < padded; ++x) lim[x] = 0;
+  std::vector<int64_t> qcost(tiles), kcost(tiles);
+  for (int64_t i = 0; i < tiles; ++i) {
+    // The needs of a tile's first row cover those of the rows behind it: they belong to
+    // later segments, whose own tokens and (if the group changes inside the tile) prompt
+    // lie between the first row and themselves.
+    const int64_t r0 = 32 * i;
+    const int32_t b0 = own[r0] / 32;
+    const int32_t a0 = pstart[r0] / 32;
+    int32_t a1 = pend[r0] > pstart[r0] ? (pend[r0] + 31) / 32 : a0;
+    a1 = std::max(a0, std::min(a1, b0));
+    int32_t* rec = out + L.q_tiles + 4 * i;
+    rec[0] = a0, rec[1] = a1, rec[2] = b0, rec[3] = 0;
+    qcost[i] = (a1 - a0) + (i - b0 + 1);
+    int32_t mx = 0;
+    for (int x = 0; x < 32; ++x) mx = std::max(mx, lim[r0 + x]);
+    out[L.kv_qend + i] = (mx + 31) / 32;
+    kcost[i] = out[L.kv_qend + i] - i;
+  }
+  auto order = [&](const std::vector<int64_t>& cost, int32_t* dst) {
+    std::iota(dst, dst + tiles, 0);
+    std::stable_sort(dst, dst + tiles, [&](int32_t a, int32_t b) { return cost[a] > cost[b]; });
+  };
+  order(qcost, out + L.q_order);
+  order(kcost, out + L.kv_order);
+}
+
+namespace {
+
+// Row fed to lane m of the first product: bits 2 and 3 of m swapped.  Output register r of
+// lane half h then belongs to row 16 * (r / 8) + 8 * h + r % 8, and registers 8 * blk ..
+// 8 * blk + 7 are the B operand of the second product for the contiguous rows
+// 16 * blk + 8 * h .. + 7.
+__device__ inline int fed_row(int m) { return (m & ~12) | ((m & 4) << 1) | ((m & 8) >> 1); }
+
+__device__ inline i32x4 ld16(const void* base, int64_t elem) {
+  return *reinterpret_cast<const i32x4*>(static_cast<const __bf16*>(base) + elem);
+}
+__device__ inline bf16x8 as_bf16(i32x4 w) { return __builtin_bit_cast(bf16x8, w); }
+
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+
+// acc[db][4 * q4 + e] of lane (n, h) is channel 32 * db + 8 * q4 + 4 * h + e of row/token n.
+template <int D>
+__device__ inline void store_rows(void* dst, int64_t row_elem, int h, const f32x16 (&acc)[D / 32], float mul) {
+  __bf16* o = static_cast<__bf16*>(dst) + row_elem + 4 * h;
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+      bf16x4 w;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) w[e] = (__bf16)(acc[db][4 * q4 + e] * mul);
+      *reinterpret_cast<bf16x4*>(o + 32 * db + 8 * q4) = w;
+    }
+}
+
+// ---- transposed tiles ---------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(kThreads) void split_transpose_kernel(const __bf16* x, int64_t stride, int T, int nt,
+                                                                  __bf16* xt) {
+  __shared__ __attribute__((aligned(16))) __bf16 tile[D][40];
+  const int j = blockIdx.x, hh = blockIdx.y;
+  for (int p = threadIdx.x; p < 32 * D / 8; p += kThreads) {
+    const int tk = p / (D / 8), c = (p % (D / 8)) * 8;
+    const int64_t t = 32 * (int64_t)j + tk;
+    i32x4 w = {0, 0, 0, 0};
+    if (t < T) w = ld16(x, t * stride + hh * D + c);
+    const bf16x8 e = as_bf16(w);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) tile[c + i][tk] = e[i];
+  }
+  __syncthreads();
+  __bf16* dst = xt + ((int64_t)hh * nt + j) * D * 32;
+  for (int p = threadIdx.x; p < D * 4; p += kThreads) {
+    const int d = p / 4, part = p % 4;
+    *reinterpret_cast<i32x4*>(dst + d * 32 + part * 8) = *reinterpret_cast<const i32x4*>(&tile[d][part * 8]);
+  }
+}
+
+// delta[h][t] = sum_d dout[t, h, d] * out[t, h, d]; zero past the last token.
+template <int D>
+__global__ __launch_bounds__(kThreads) void split_delta_kernel(SplitParams p) {
+  constexpr int LPR = D / 8;
+  const int64_t padded = 32 * (int64_t)p.num_tiles;
+  const int64_t idx = (int64_t)blockIdx.x * (kThreads / LPR) + threadIdx.x / LPR;
+  if (idx >= padded * p.num_q_heads) return;  // whole lane groups leave together
+  const int64_t t = idx % padded;
+  const int hh = (int)(idx / padded);
+  const int c = (threadIdx.x % LPR) * 8;
+  float sum = 0.f;
+  if (t < p.num_tokens) {
+    const bf16x8 a = as_bf16(ld16(p.dout, t * p.do_stride + hh * D + c));
+    const bf16x8 b = as_bf16(ld16(p.out_in, t * p.o_stride + hh * D + c));
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sum += (float)a[i] * (float)b[i];
+  }
+#pragma unroll
+  for (int w = 1; w < LPR; w *= 2) sum += __shfl_xor(sum, w);
+  if (threadIdx.x % LPR == 0) p.delta[hh * padded + t] = sum;
+}
+
+// ---- forward and dq: one wave per (query tile, query head) -----------------------------------
+template <int D, bool BWD>
+struct KeyTile {
+  i32x4 k[D / 16];                   // K rows, first product
+  i32x4 vn[BWD ? D / 16 : 1];        // V rows (dq: dP)
+  i32x4 tr[2][D / 32];               // transposed tile: V (forward), K (dq)
+  i32x4 lim[2][2];
+  int j;
+};
+
+template <int D, bool BWD>
+__global__ __launch_bounds__(kThreads, 1) void split_query_kernel(SplitParams p) {
+  constexpr int KS = D / 16, NDB = D / 32;
+  using Tile = KeyTile<D, BWD>;
+  const SplitLayout L = make_split_layout(p.num_tiles);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = lane & 31, h = lane >> 5;
+  const int hq = blockIdx.y * kWaves + wave;
+  if (hq >= p.num_q_heads) return;
+  const int hkv = hq / (p.num_q_heads / p.num_kv_heads);
+  const int T = p.num_tokens, nt = p.num_tiles;
+  const int64_t padded = 32 * (int64_t)nt;
+  const int i = __builtin_amdgcn_readfirstlane(p.layout[L.q_order + blockIdx.x]);
+  const int a0 = __builtin_amdgcn_readfirstlane(p.layout[L.q_tiles + 4 * i]);
+  const int a1 = __builtin_amdgcn_readfirstlane(p.layout[L.q_tiles + 4 * i + 1]);
+  const int b0 = __builtin_amdgcn_readfirstlane(p.layout[L.q_tiles + 4 * i + 2]);
+  const int na = a1 - a0, ntile = na + i - b0 + 1;
+  const int r = 32 * i + n;
+  const int64_t rc = min(r, T - 1);
+
+  bf16x8 qreg[KS], doreg[BWD ? KS : 1];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) qreg[s] = as_bf16(ld16(p.q, rc * p.q_stride + hq * D + 16 * s + 8 * h));
+  float lse2 = 0.f, delta = 0.f;
+  if constexpr (BWD) {
+#pragma unroll
+    for (int s = 0; s < KS; ++s) doreg[s] = as_bf16(ld16(p.dout, rc * p.do_stride + hq * D + 16 * s + 8 * h));
+    lse2 = p.lse[hq * padded + r] * kLog2e;
+    delta = p.delta[hq * padded + r];
+  }
+  const void* trsrc = BWD ? p.kt : p.vt;
+  const float sc = p.scale * kLog2e;
+
+  f32x16 acc[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+#pragma unroll
+    for (int x = 0; x < 16; ++x) acc[db][x] = 0.f;
+  float mrow = -1e30f, lrow = 0.f;
+
+  auto load = [&](Tile& t, int idx) {
+    idx = min(idx, ntile - 1);
+    const int j = idx < na ? a0 + idx : b0 + idx - na;
+    t.j = j;
+    const int64_t tok = min(32 * j + fed_row(n), T - 1);
+#pragma unroll
+    for (int s = 0; s < KS; ++s) t.k[s] = ld16(p.k, tok * p.k_stride + hkv * D + 16 * s + 8 * h);
+    if constexpr (BWD) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) t.vn[s] = ld16(p.v, tok * p.v_stride + hkv * D + 16 * s + 8 * h);
+    }
+    const int64_t base = (((int64_t)hkv * nt + j) * D + n) * 32 + 8 * h;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) t.tr[blk][db] = ld16(trsrc, base + (int64_t)db * 32 * 32 + 16 * blk);
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+        t.lim[blk][half] = *reinterpret_cast<const i32x4*>(p.layout + L.kv_lim + 32 * j + 16 * blk + 8 * h + 4 * half);
+  };
+
+  auto compute = [&](const Tile& t) {
+    f32x16 sr;
+#pragma unroll
+    for (int x = 0; x < 16; ++x) sr[x] = 0.f;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) sr = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(t.k[s]), qreg[s], sr, 0, 0, 0);
+    const int tok0 = 32 * t.j + 8 * h;
+    bool ok[16];
+#pragma unroll
+    for (int x = 0; x < 16; ++x) {
+      const int tok = tok0 + 16 * (x >> 3) + (x & 7);
+      ok[x] = tok <= r && t.lim[x >> 3][(x >> 2) & 1][x & 3] > r;
+    }
+    bf16x8 pb[2];
+    if constexpr (!BWD) {
+#pragma unroll
+      for (int x = 0; x < 16; ++x)
+        if (!ok[x]) sr[x] = -INFINITY;
+      float mx = sr[0];
+#pragma unroll
+      for (int x = 1; x < 16; ++x) mx = fmaxf(mx, sr[x]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      // the reference point of the exponentials moves only when a row's maximum rises by
+      // more than kRescaleSlack above it; the log-sum-exp does not depend on it
+      const float mtile = mx * sc;
+      if (__builtin_amdgcn_readfirstlane(__any(mtile > mrow + kRescaleSlack))) {
+        const float mnew = fmaxf(mrow, mtile);
+        const float alpha = fast_exp2(mrow - mnew);
+        lrow *= alpha;
+        mrow = mnew;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+          for (int x = 0; x < 16; ++x) acc[db][x] *= alpha;
+      }
+      float sum = 0.f;
+#pragma unroll
+      for (int x = 0; x < 16; ++x) {
+        const float e = fast_exp2(__builtin_fmaf(sr[x], sc, -mrow));
+        sum += e;
+        pb[x >> 3][x & 7] = (__bf16)e;
+      }
+      lrow += sum;
+    } else {
+      f32x16 dp;
+#pragma unroll
+      for (int x = 0; x < 16; ++x) dp[x] = 0.f;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(t.vn[s]), doreg[s], dp, 0, 0, 0);
+#pragma unroll
+      for (int x = 0; x < 16; ++x) {
+        const float e = ok[x] ? fast_exp2(__builtin_fmaf(sr[x], sc, -lse2)) : 0.f;
+        pb[x >> 3][x & 7] = (__bf16)(e * (dp[x] - delta));
+      }
+    }
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(t.tr[blk][db]), pb[blk], acc[db], 0, 0, 0);
+  };
+
+  // two tile buffers: the next tile is requested before the current one is used; requests
+  // past the end repeat the last tile, so every path issues the same loads
+  Tile ta, tb;
+  load(ta, 0);
+  for (int idx = 0; idx < ntile; idx += 2) {
+    load(tb, idx + 1);
+    compute(ta);
+    load(ta, idx + 2);
+    if (idx + 1 < ntile) compute(tb);
+  }
+
+  if constexpr (!BWD) {
+    const float l = lrow + __shfl_xor(lrow, 32);
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    if (r < T) store_rows<D>(p.out, (int64_t)r * p.o_stride + hq * D, h, acc, inv);
+    if (h == 0) p.lse[hq * padded + r] = l > 0.f ? (mrow + fast_log2(l)) * kLn2 : 0.f;
+  } else {
+    if (r < T) store_rows<D>(p.dq, (int64_t)r * p.dq_stride + hq * D, h, acc, p.scale);
+  }
+}
+
+// ---- dk, dv: one wave per (key tile, KV head) --------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(kThreads, 1) void split_key_kernel(SplitParams p) {
+  constexpr int KS = D / 16, NDB = D / 32;
+  const SplitLayout L = make_split_layout(p.num_tiles);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = lane & 31, h = lane >> 5;
+  const int hkv = blockIdx.y * kWaves + wave;
+  if (hkv >= p.num_kv_heads) return;
+  const int group = p.num_q_heads / p.num_kv_heads;
+  const int T = p.num_tokens, nt = p.num_tiles;
+  const int64_t padded = 32 * (int64_t)nt;
+  const int j = __builtin_amdgcn_readfirstlane(p.layout[L.kv_order + blockIdx.x]);
+  const int qend = __builtin_amdgcn_readfirstlane(p.layout[L.kv_qend + j]);
+  const int t = 32 * j + n;
+  const int64_t tc = min(t, T - 1);
+  const int lim_t = p.layout[L.kv_lim + t];
+  const float sc = p.scale * kLog2e;
+
+  bf16x8 kreg[KS], vreg[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    kreg[s] = as_bf16(ld16(p.k, tc * p.k_stride + hkv * D + 16 * s + 8 * h));
+    vreg[s] = as_bf16(ld16(p.v, tc * p.v_stride + hkv * D + 16 * s + 8 * h));
+  }
+  f32x16 acck[NDB], accv[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+#pragma unroll
+    for (int x = 0; x < 16; ++x) acck[db][x] = 0.f, accv[db][x] = 0.f;
+
+  for (int i = j; i < qend; ++i) {
+    const int64_t row = min(32 * i + fed_row(n), T - 1);
+    for (int g = 0; g < group; ++g) {
+      const int hq = hkv * group + g;
+      i32x4 qn[KS], don[KS], qtr[2][NDB], dotr[2][NDB];
+      f32x4 ls[2][2], dl[2][2];
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        qn[s] = ld16(p.q, row * p.q_stride + hq * D + 16 * s + 8 * h);
+        don[s] = ld16(p.dout, row * p.do_stride + hq * D + 16 * s + 8 * h);
+      }
+      const int64_t base = (((int64_t)hq * nt + i) * D + n) * 32 + 8 * h;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+          qtr[blk][db] = ld16(p.qt, base + (int64_t)db * 32 * 32 + 16 * blk);
+          dotr[blk][db] = ld16(p.dot, base + (int64_t)db * 32 * 32 + 16 * blk);
+        }
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int64_t at = hq * padded + 32 * i + 16 * blk + 8 * h + 4 * half;
+          ls[blk][half] = *reinterpret_cast<const f32x4*>(p.lse + at);
+          dl[blk][half] = *reinterpret_cast<const f32x4*>(p.delta + at);
+        }
+      f32x16 sr, dp;
+#pragma unroll
+      for (int x = 0; x < 16; ++x) sr[x] = 0.f, dp[x] = 0.f;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        sr = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(qn[s]), kreg[s], sr, 0, 0, 0);
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(don[s]), vreg[s], dp, 0, 0, 0);
+      }
+      bf16x8 pb[2], dsb[2];
+      const int row0 = 32 * i + 8 * h;
+#pragma unroll
+      for (int x = 0; x < 16; ++x) {
+        const int qrow = row0 + 16 * (x >> 3) + (x & 7);
+        const bool ok = t <= qrow && qrow < lim_t;
+        const float e = ok ? fast_exp2(__builtin_fmaf(sr[x], sc, -ls[x >> 3][(x >> 2) & 1][x & 3] * kLog2e)) : 0.f;
+        pb[x >> 3][x & 7] = (__bf16)e;
+        dsb[x >> 3][x & 7] = (__bf16)(e * (dp[x] - dl[x >> 3][(x >> 2) & 1][x & 3]));
+      }
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+          accv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(dotr[blk][db]), pb[blk], accv[db], 0, 0, 0);
+          acck[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(qtr[blk][db]), dsb[blk], acck[db], 0, 0, 0);
+        }
+    }
+  }
+  if (t < T) {
+    store_rows<D>(p.dk, (int64_t)t * p.dk_stride + hkv * D, h, acck, p.scale);
+    store_rows<D>(p.dv, (int64_t)t * p.dv_stride + hkv * D, h, accv, 1.f);
+  }
+}
+
+template <typename F>
+hipError_t by_head_dim(int head_dim, F&& f) {
+  if (head_dim == 128) return f(std::integral_constant<int, 128>{});
+  if (head_dim == 64) return f(std::integral_constant<int, 64>{});
+  return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+hipError_t launch_split_transpose(const void* x, int64_t stride, int heads, int head_dim, int num_tokens, int tiles,
+                                  void* xt, hipStream_t stream) {
+  return by_head_dim(head_dim, [&](auto d) {
+    constexpr int D = decltype(d)::value;
+    split_transpose_kernel<D><<<dim3(tiles, heads), kThreads, 0, stream>>>(static_cast<const __bf16*>(x), stride, num_tokens,
+                                                                          tiles, static_cast<__bf16*>(xt));
+    return hipGetLastError();
+  });
+}
+
+hipError_t launch_split_forward(const SplitParams& p, int head_dim, hipStream_t stream) {
+  if (hipError_t e = launch_split_transpose(p.v, p.v_stride, p.num_kv_heads, head_dim, p.num_tokens, p.num_tiles,
+                                            const_cast<void*>(p.vt), stream))
+    return e;
+  return by_head_dim(head_dim, [&](auto d) {
+    constexpr int D = decltype(d)::value;
+    const dim3 grid(p.num_tiles, (p.num_q_heads + kWaves - 1) / kWaves);
+    split_query_kernel<D, false><<<grid, kThreads, 0, stream>>>(p);
+    return hipGetLastError();
+  });
+}
+
+hipError_t launch_split_backward(const SplitParams& p, int head_dim, hipStream_t stream) {
+  const int T = p.num_tokens, nt = p.num_tiles;
+  if (hipError_t e = launch_split_transpose(p.k, p.k_stride, p.num_kv_heads, head_dim, T, nt, const_cast<void*>(p.kt), stream))
+    return e;
+  if (hipError_t e = launch_split_transpose(p.q, p.q_stride, p.num_q_heads, head_dim, T, nt, const_cast<void*>(p.qt), stream))
+    return e;
+  if (hipError_t e = launch_split_transpose(p.dout, p.do_stride, p.num_q_heads, head_dim, T, nt, const_cast<void*>(p.dot), stream))
+    return e;
+  return by_head_dim(head_dim, [&](auto d) {
+    constexpr int D = decltype(d)::value;
+    const int64_t rows = 32 * (int64_t)nt * p.num_q_heads;
+    const int per_block = kThreads / (D / 8);
+    split_delta_kernel<D><<<(unsigned)((rows + per_block - 1) / per_block), kThreads, 0, stream>>>(p);
+    if (hipError_t e = hipGetLastError()) return e;
+    split_query_kernel<D, true><<<dim3(nt, (p.num_q_heads + kWaves - 1) / kWaves), kThreads, 0, stream>>>(p);
+    if (hipError_t e = hipGetLastError()) return e;
+    split_key_kernel<D><<<dim3(nt, (p.num_kv_heads + kWaves - 1) / kWaves), kThreads, 0, stream>>>(p);
+    return hipGetLastError();
+  });
+}
+
+}  // namespace fca

@@ -1,0 +1,163 @@
+"""Split attention of the trainer over a deduplicated, unpadded batch, forward and backward.
+
+Host-side face of ``fca_split_attention_forward`` / ``fca_split_attention_backward``.  It
+stands where the trainer's patched attention forward makes its two ``attention_interface``
+calls and regroups their outputs (``patched_forward_split_unpadded``,
+arctic_platform/rl/zorro_train/qwen_attention_patcher.py:1186-1231): prompt rows attend
+causally to their prompt, response rows to the whole prompt of their group and causally to
+their own response.  The tensors stay in deduplicated order (for every prompt group the
+prompt once, then the response of every sample, zorro_train.py:311-356); nothing is copied
+per sample, and in the backward a prompt's dK and dV collect all samples of its group.
+
+``SplitLayout.from_group_token_layout`` takes what ``ZoRRoTrain.get_group_token_layout``
+returns (zorro_train.py:2413-2436): a list of dicts with ``prompt_tokens`` and
+``response_tokens``.  A layout is made once per batch and serves every layer.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _lib
+
+
+def _stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+class SplitLayout:
+    """Token layout of one deduplicated batch: ``[(prompt_tokens, [response_tokens, ...]), ...]``."""
+
+    def __init__(self, groups, device="cuda"):
+        self.groups = [(int(p), [int(n) for n in rs]) for p, rs in groups]
+        prompt = np.asarray([p for p, _ in self.groups], dtype=np.int32)
+        sizes = np.asarray([len(rs) for _, rs in self.groups], dtype=np.int32)
+        resp = np.asarray([n for _, rs in self.groups for n in rs], dtype=np.int32)
+        self.num_tokens = int(prompt.sum()) + int(resp.sum())
+        self.num_tiles = (self.num_tokens + 31) // 32
+        lib = _lib.load_library()
+        n = ctypes.c_int64()
+        _lib.check(lib.fca_split_layout_ints(self.num_tokens, ctypes.byref(n)))
+        self.host = np.zeros(max(int(n.value), 1), dtype=np.int32)
+        _lib.check(
+            lib.fca_split_layout_build(
+                len(self.groups), prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, self.num_tokens, self.host.ctypes.data
+            )
+        )
+        self.device = torch.device(device)
+        self.dev = torch.from_numpy(self.host).to(self.device) if self.device.type == "cuda" else None
+        self._scratch = {}
+
+    @classmethod
+    def from_group_token_layout(cls, layout, device="cuda"):
+        return cls([(g["prompt_tokens"], g["response_tokens"]) for g in layout], device=device)
+
+    # views of the layout array (tests, inspection)
+    def kv_lim(self):
+        return self.host[: 32 * self.num_tiles]
+
+    def q_tiles(self):
+        o = 32 * self.num_tiles
+        return self.host[o : o + 4 * self.num_tiles].reshape(-1, 4)
+
+    def kv_qend(self):
+        o = 36 * self.num_tiles
+        return self.host[o : o + self.num_tiles]
+
+    def orders(self):
+        o = 37 * self.num_tiles
+        return self.host[o : o + self.num_tiles], self.host[o + self.num_tiles : o + 2 * self.num_tiles]
+
+    def scratch(self, plan, backward: bool) -> torch.Tensor:
+        """Scratch of a call, kept with the layout: layers run one after the other on a stream."""
+        fwd, bwd = ctypes.c_size_t(), ctypes.c_size_t()
+        _lib.check(_lib.load_library().fca_split_workspace_bytes(ctypes.byref(plan), ctypes.byref(fwd), ctypes.byref(bwd)))
+        need = bwd.value if backward else fwd.value
+        key = "bwd" if backward else "fwd"
+        buf = self._scratch.get(key)
+        if buf is None or buf.numel() < need:
+            buf = self._scratch[key] = torch.empty(max(need, 16), dtype=torch.uint8, device=self.device)
+        return buf
+
+
+def _check_rows(name, x, tokens):
+    if x.dtype != torch.bfloat16 or x.dim() != 3 or x.shape[0] != tokens:
+        raise ValueError(f"{name} must be bfloat16 [T, H, D] with T = {tokens}, got {tuple(x.shape)} {x.dtype}")
+    if not x.is_cuda:
+        raise RuntimeError(f"split attention runs on the GPU; {name} must be a device tensor")
+    if x.stride(2) != 1 or x.stride(1) != x.shape[2]:
+        raise ValueError(f"the heads of a token of {name} must be contiguous")
+
+
+def _plan(q, k):
+    return _lib.FcaSplitPlan(q.shape[0], q.shape[1], k.shape[1], q.shape[2])
+
+
+def split_attention_forward(q, k, v, layout: SplitLayout, scale: float):
+    """q ``[T, Hq, D]``, k, v ``[T, Hkv, D]`` bf16 in deduplicated order.  Returns
+    ``(out [T, Hq, D] bf16, lse fp32 [Hq, 32 * ceil(T / 32)])``; ``lse[:, :T]`` is the
+    natural-log log-sum-exp of every row's scores."""
+    t = layout.num_tokens
+    for name, x in (("q", q), ("k", k), ("v", v)):
+        _check_rows(name, x, t)
+    plan = _plan(q, k)
+    out = torch.empty((t, q.shape[1], q.shape[2]), dtype=torch.bfloat16, device=q.device)
+    lse = torch.empty((q.shape[1], 32 * layout.num_tiles), dtype=torch.float32, device=q.device)
+    if t == 0:
+        return out, lse
+    _lib.check(
+        _lib.load_library().fca_split_attention_forward(
+            ctypes.byref(plan), q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
+            layout.dev.data_ptr(), float(scale), layout.scratch(plan, False).data_ptr(), out.data_ptr(), out.stride(0),
+            lse.data_ptr(), _stream_ptr(q.device),
+        )
+    )
+    return out, lse
+
+
+def split_attention_backward(dout, q, k, v, out, lse, layout: SplitLayout, scale: float):
+    """Gradients ``(dq, dk, dv)`` of ``split_attention_forward``'s ``out`` with respect to
+    its inputs, for the upstream gradient ``dout``."""
+    t = layout.num_tokens
+    for name, x in (("q", q), ("k", k), ("v", v), ("out", out), ("dout", dout)):
+        _check_rows(name, x, t)
+    plan = _plan(q, k)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    for name, x in (("dq", dq), ("dk", dk), ("dv", dv)):
+        _check_rows(name, x, t)
+    if t == 0:
+        return dq, dk, dv
+    _lib.check(
+        _lib.load_library().fca_split_attention_backward(
+            ctypes.byref(plan), q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
+            out.data_ptr(), out.stride(0), dout.data_ptr(), dout.stride(0), lse.data_ptr(), layout.dev.data_ptr(),
+            float(scale), layout.scratch(plan, True).data_ptr(), dq.data_ptr(), dq.stride(0), dk.data_ptr(), dk.stride(0),
+            dv.data_ptr(), dv.stride(0), _stream_ptr(q.device),
+        )
+    )
+    return dq, dk, dv
+
+
+class _SplitAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, layout, scale):
+        out, lse = split_attention_forward(q, k, v, layout, scale)
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.layout, ctx.scale = layout, scale
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse = ctx.saved_tensors
+        if dout.stride(2) != 1 or dout.stride(1) != dout.shape[2]:
+            dout = dout.contiguous()
+        dq, dk, dv = split_attention_backward(dout, q, k, v, out, lse, ctx.layout, ctx.scale)
+        return dq, dk, dv, None, None
+
+
+def split_attention(q, k, v, layout: SplitLayout, scale: float):
+    """Differentiable split attention: ``out [T, Hq, D]`` in deduplicated order."""
+    return _SplitAttention.apply(q, k, v, layout, scale)

@@ -228,6 +228,48 @@ int fca_append_kv(const void* key_dev, const void* value_dev, int64_t token_stri
                   void* k_cache_dev, void* v_cache_dev, int64_t kv_block_stride, int64_t kv_head_stride, int32_t kv_dtype,
                   const float* k_scale_dev, const float* v_scale_dev, void* stream);
 
+/* ---- split attention of the trainer (forward and backward) ---------------------------
+ * Attention over a deduplicated, unpadded training batch: q [T, Hq, D], k and v
+ * [T, Hkv, D], bf16, tokens in deduplicated order (for every prompt group the prompt once,
+ * then the response of every sample: ZoRRoTrain._dedup_input_ids,
+ * arctic_platform/rl/zorro_train/zorro_train.py:311-356).  Replaces the two
+ * attention_interface calls of patched_forward_split_unpadded and the regrouping around
+ * them (arctic_platform/rl/zorro_train/qwen_attention_patcher.py:1186-1231): prompt rows
+ * attend causally to their prompt, response rows to their group's whole prompt and causally
+ * to their own response.  Row strides are in elements; the heads of a token are contiguous
+ * ([H, D]); every pointer 16-byte aligned, strides multiples of 8. */
+typedef struct fca_split_plan {
+  int32_t num_tokens; /* T: tokens of the deduplicated batch */
+  int32_t num_q_heads;
+  int32_t num_kv_heads;
+  int32_t head_dim; /* 64 or 128 */
+} fca_split_plan;
+
+/* int32 entries of the layout array of a batch of num_tokens tokens. */
+int fca_split_layout_ints(int32_t num_tokens, int64_t* num_ints);
+/* Host function: fills the layout array (host memory, fca_split_layout_ints entries) from
+ * the token layout of ZoRRoTrain.get_group_token_layout (zorro_train.py:2413-2436):
+ * prompt_tokens[g], group_sizes[g] samples per group, response_tokens one per sample in
+ * group order.  The counts must add up to num_tokens.  The caller copies the array to the
+ * device once per batch; every layer's forward and backward reads it. */
+int fca_split_layout_build(int32_t num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,
+                           const int32_t* response_tokens, int32_t num_tokens, int32_t* layout_host);
+/* Bytes of device scratch a forward / a backward call needs (transposed operand tiles). */
+int fca_split_workspace_bytes(const fca_split_plan* plan, size_t* forward_bytes, size_t* backward_bytes);
+/* out [T, Hq, D] bf16; lse fp32 [Hq][32 * ceil(T / 32)], natural log (kept for backward). */
+int fca_split_attention_forward(const fca_split_plan* plan, const void* q_dev, int64_t q_stride, const void* k_dev,
+                                int64_t k_stride, const void* v_dev, int64_t v_stride, const int32_t* layout_dev,
+                                float scale, void* workspace_dev, void* out_dev, int64_t out_stride, float* lse_dev,
+                                void* stream);
+/* Gradients dq [T, Hq, D], dk, dv [T, Hkv, D] (bf16, fp32 accumulation; a prompt's dk and
+ * dv sum over the samples of its group) from dout, the forward's inputs, out and lse. */
+int fca_split_attention_backward(const fca_split_plan* plan, const void* q_dev, int64_t q_stride, const void* k_dev,
+                                 int64_t k_stride, const void* v_dev, int64_t v_stride, const void* out_dev,
+                                 int64_t out_stride, const void* dout_dev, int64_t dout_stride, const float* lse_dev,
+                                 const int32_t* layout_dev, float scale, void* workspace_dev, void* dq_dev,
+                                 int64_t dq_stride, void* dk_dev, int64_t dk_stride, void* dv_dev, int64_t dv_stride,
+                                 void* stream);
+
 /* Plain device-to-device copy with 16-byte loads and stores.  No counterpart in the
  * reference: it is the known-size yardstick for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE
  * readings of the kernels above. */

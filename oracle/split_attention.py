@@ -1,0 +1,125 @@
+"""Test infrastructure only: CPU restatement of the trainer's split attention over a
+deduplicated, unpadded batch.  Nothing in the product imports it.
+
+Deduplicated order of the tokens (``ZoRRoTrain._dedup_input_ids``,
+arctic_platform/rl/zorro_train/zorro_train.py:311-356; read back by
+``get_group_token_layout``, :2413-2436): for every prompt group the prompt once, then the
+response of every sample of the group.  A layout here is that function's result reduced
+to what attention needs: a list of ``(prompt_tokens, [response_tokens, ...])``.
+
+The patched attention forward makes two attention calls per layer
+(``patched_forward_split_unpadded``, arctic_platform/rl/zorro_train/
+qwen_attention_patcher.py:1117-1259): causal attention of every unique prompt over itself
+(:1198-1208), and attention of every response over its prompt followed by itself, causal
+with the mask aligned bottom-right (:1211-1228: K and V are the prompt's rows followed by
+the response's, one copy per sample), and puts the outputs back in deduplicated order
+(:1229-1231).  ``split_attention`` below follows those two calls with plain tensor
+algebra in the given dtype; autograd through it is the backward the kernels are checked
+against.  ``full_attention_of_samples`` is the computation the split replaces, every
+sample's whole sequence attended causally on its own, which is what the reference's own
+test compares the patched model with (tests/zorro_train/test_once_patcher.py:189-206).
+
+Pins (tests/test_split_attention.py): split == full on the rows both produce, for outputs
+and for gradients (prompt rows of a group receive the sum over its samples), a closed form
+(constant V), and the row sums of the probabilities implied by the log-sum-exp.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+
+def segments(layout):
+    """[(group, kind, start, length)] in deduplicated order; kind 'p' or 'r'."""
+    out, t = [], 0
+    for g, (prompt, responses) in enumerate(layout):
+        out.append((g, "p", t, int(prompt)))
+        t += int(prompt)
+        for n in responses:
+            out.append((g, "r", t, int(n)))
+            t += int(n)
+    return out
+
+
+def total_tokens(layout) -> int:
+    return sum(int(p) + sum(int(n) for n in rs) for p, rs in layout)
+
+
+def _attend(q, k, v, scale, first_key_offset):
+    """q [Lq, Hq, D], k/v [Lk, Hkv, D]; query i sees keys 0 .. first_key_offset + i
+    (bottom-right aligned causal mask when first_key_offset = Lk - Lq).  Returns out and
+    the natural-log log-sum-exp [Lq, Hq]."""
+    lq, hq, _ = q.shape
+    lk, hkv, _ = k.shape
+    rep = hq // hkv
+    kk = k.repeat_interleave(rep, dim=1)
+    vv = v.repeat_interleave(rep, dim=1)
+    s = torch.einsum("qhd,khd->hqk", q, kk) * scale
+    keys = torch.arange(lk)[None, :]
+    rows = torch.arange(lq)[:, None]
+    s = s.masked_fill(keys > rows + first_key_offset, -math.inf)
+    lse = torch.logsumexp(s, dim=-1)
+    p = torch.exp(s - lse[..., None])
+    return torch.einsum("hqk,khd->qhd", p, vv), lse.transpose(0, 1)
+
+
+def split_attention(q, k, v, layout, scale, dtype=torch.float64):
+    """q [T, Hq, D], k/v [T, Hkv, D] in deduplicated order.  Returns (out [T, Hq, D],
+    lse [T, Hq]) in ``dtype``.  Differentiable."""
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    outs, lses = [], []
+    prompt_of = {}
+    for g, kind, start, n in segments(layout):
+        if kind == "p":
+            prompt_of[g] = (start, n)
+            o, l = _attend(q[start : start + n], k[start : start + n], v[start : start + n], scale, 0)
+        else:
+            ps, pn = prompt_of[g]
+            kk = torch.cat([k[ps : ps + pn], k[start : start + n]])
+            vv = torch.cat([v[ps : ps + pn], v[start : start + n]])
+            o, l = _attend(q[start : start + n], kk, vv, scale, pn)
+        outs.append(o)
+        lses.append(l)
+    return torch.cat(outs), torch.cat(lses)
+
+
+def reconstruct(x, layout):
+    """Deduplicated rows -> one tensor per sample: the prompt's rows followed by the
+    response's (the packed reconstruction, zorro_train.py:1071-1159)."""
+    samples = []
+    prompt = None
+    for g, kind, start, n in segments(layout):
+        if kind == "p":
+            prompt = x[start : start + n]
+        else:
+            samples.append(torch.cat([prompt, x[start : start + n]]))
+    return samples
+
+
+def full_attention_of_samples(q, k, v, layout, scale, dtype=torch.float64):
+    """Every sample's whole sequence attended causally on its own, from the deduplicated
+    tensors; returns per sample (out, lse) of prompt + response rows."""
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    return [
+        _attend(qs, ks, vs, scale, 0)
+        for qs, ks, vs in zip(reconstruct(q, layout), reconstruct(k, layout), reconstruct(v, layout))
+    ]
+
+
+def visible(layout):
+    """Brute force: boolean [T, T], entry (r, t) true when query row r attends to key t."""
+    n = total_tokens(layout)
+    vis = torch.zeros(n, n, dtype=torch.bool)
+    prompt_of = {}
+    for g, kind, start, length in segments(layout):
+        if kind == "p":
+            prompt_of[g] = (start, length)
+        for i in range(length):
+            r = start + i
+            vis[r, start : r + 1] = True
+            if kind == "r":
+                ps, pn = prompt_of[g]
+                vis[r, ps : ps + pn] = True
+    return vis

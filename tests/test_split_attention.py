@@ -1,0 +1,259 @@
+"""Split attention of the trainer over a deduplicated batch: the oracle's pins, the layout
+array (host code of the library, no GPU needed) and, on the GPU, forward and backward of
+the HIP kernels against the oracle."""
+
+import ctypes
+import math
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from arctic_platform_amd import _lib
+from arctic_platform_amd.split_attention import (
+    SplitLayout,
+    split_attention,
+    split_attention_backward,
+    split_attention_forward,
+)
+from oracle.split_attention import (
+    full_attention_of_samples,
+    reconstruct,
+    segments,
+    split_attention as oracle_split,
+    total_tokens,
+    visible,
+)
+
+LAYOUTS = [
+    [(40, [20, 33]), (7, [5])],
+    [(100, [64, 1, 70]), (0, [40]), (33, [0, 31])],
+    [(5, [3]), (1, [1, 1, 1, 1, 1, 1, 1, 1])],
+    [(64, [32, 32]), (32, [64])],
+]
+
+
+def _random_layout(rng):
+    return [
+        (rng.choice([0, 1, 5, 31, 32, 33, 70, 130]), [rng.choice([0, 1, 3, 17, 32, 40, 64, 90]) for _ in range(rng.randint(1, 4))])
+        for _ in range(rng.randint(1, 4))
+    ]
+
+
+def _inputs(layout, hq, hkv, d, seed, dtype=torch.float64):
+    g = torch.Generator().manual_seed(seed)
+    t = total_tokens(layout)
+    return (
+        torch.randn(t, hq, d, generator=g).to(dtype),
+        torch.randn(t, hkv, d, generator=g).to(dtype),
+        torch.randn(t, hkv, d, generator=g).to(dtype),
+    )
+
+
+# ---- the oracle's pins (CPU) ----------------------------------------------------------------
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_oracle_equals_full_attention_of_every_sample(layout):
+    """What the reference's own test asserts of the patched model
+    (tests/zorro_train/test_once_patcher.py:189-206): the deduplicated forward gives every
+    sample the rows that plain causal attention over its whole sequence gives, and the
+    prompt rows once.  Gradients: a prompt's K and V collect all samples of the group."""
+    q, k, v = _inputs(layout, 4, 2, 16, 3)
+    q.requires_grad_(), k.requires_grad_(), v.requires_grad_()
+    out, lse = oracle_split(q, k, v, layout, 0.25)
+    full = full_attention_of_samples(q, k, v, layout, 0.25)
+    # rows of the split result, sample by sample
+    outs, lses = reconstruct(out, layout), reconstruct(lse, layout)
+    for (fo, fl), so, sl in zip(full, outs, lses):
+        torch.testing.assert_close(so, fo, rtol=1e-12, atol=1e-12)
+        torch.testing.assert_close(sl, fl, rtol=1e-12, atol=1e-12)
+    # a loss that weighs every deduplicated row once; the same loss on the full
+    # computation takes a prompt row from the group's first sample only
+    w = torch.randn(out.shape, generator=torch.Generator().manual_seed(5), dtype=torch.float64)
+    gs = torch.autograd.grad((out * w).sum(), (q, k, v))
+    loss = 0.0
+    sample = 0
+    seen = set()
+    for g, kind, start, n in segments(layout):
+        if kind == "p":
+            prompt = (start, n)
+            continue
+        fo = full[sample][0]
+        ps, pn = prompt
+        if g not in seen:
+            loss = loss + (fo[:pn] * w[ps : ps + pn]).sum()
+            seen.add(g)
+        loss = loss + (fo[pn:] * w[start : start + n]).sum()
+        sample += 1
+    # prompts of groups whose samples are all empty still count
+    gf = torch.autograd.grad(loss, (q, k, v))
+    for a, b in zip(gs, gf):
+        torch.testing.assert_close(a, b, rtol=1e-10, atol=1e-10)
+
+
+def test_oracle_against_the_brute_force_mask_and_closed_forms():
+    layout = LAYOUTS[1]
+    q, k, v = _inputs(layout, 4, 2, 8, 11)
+    out, lse = oracle_split(q, k, v, layout, 0.3)
+    vis = visible(layout)
+    s = torch.einsum("qhd,khd->hqk", q, k.repeat_interleave(2, 1)) * 0.3
+    s = s.masked_fill(~vis[None], -math.inf)
+    torch.testing.assert_close(lse, torch.logsumexp(s, -1).T, rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(out, torch.einsum("hqk,khd->qhd", torch.softmax(s, -1), v.repeat_interleave(2, 1)), rtol=1e-12, atol=1e-12)
+    # constant values: every output row is that constant; zero queries: lse = log(keys seen)
+    vc = torch.ones_like(v) * 0.75
+    oc, lz = oracle_split(torch.zeros_like(q), k, vc, layout, 0.3)
+    assert torch.allclose(oc, torch.full_like(oc, 0.75), atol=1e-14)
+    torch.testing.assert_close(lz, vis.sum(1).double().log()[:, None].expand(-1, 4), rtol=1e-12, atol=1e-12)
+
+
+# ---- the layout array (host code of the library) -------------------------------------------------
+def test_layout_array_against_brute_force():
+    rng = random.Random(7)
+    layouts = LAYOUTS + [_random_layout(rng) for _ in range(120)]
+    for layout in layouts:
+        if total_tokens(layout) == 0:
+            continue
+        L = SplitLayout(layout, device="cpu")
+        t, nt = L.num_tokens, L.num_tiles
+        vis = visible(layout).numpy()
+        lim = L.kv_lim()
+        r, c = np.arange(t)[:, None], np.arange(t)[None, :]
+        assert (((c <= r) & (r < lim[:t][None, :])) == vis).all(), layout
+        assert (lim[t:] == 0).all()
+        padded = np.zeros((32 * nt, 32 * nt), bool)
+        padded[:t, :t] = vis
+        tiles = padded.reshape(nt, 32, nt, 32).any(axis=(1, 3))  # [query tile, key tile]
+        for i, (a0, a1, b0, _) in enumerate(L.q_tiles()):
+            assert a0 <= a1 <= b0 <= i
+            covered = set(range(a0, a1)) | set(range(b0, i + 1))
+            assert set(np.nonzero(tiles[i])[0].tolist()) <= covered, (layout, i)
+        for j, qend in enumerate(L.kv_qend()):
+            need = np.nonzero(tiles[:, j])[0]
+            assert need.min() >= j and need.max() < qend, (layout, j)
+        for order in L.orders():
+            assert sorted(order.tolist()) == list(range(nt))
+
+
+def test_layout_walks_only_what_is_needed():
+    """Eight long responses over one prompt: a query tile of the last response walks the
+    prompt's tiles and its own, not the seven responses in between."""
+    L = SplitLayout([(1024, [512] * 8)], device="cpu")
+    a0, a1, b0, _ = L.q_tiles()[L.num_tiles - 1]
+    assert (a0, a1) == (0, 32) and b0 == (1024 + 7 * 512) // 32
+    assert L.kv_qend()[0] == L.num_tiles and L.kv_qend()[40] == (1024 + 512) // 32
+    # heaviest work first
+    qo, ko = L.orders()
+    cost = [(a1 - a0) + (i - b0 + 1) for i, (a0, a1, b0, _) in enumerate(L.q_tiles())]
+    assert [cost[i] for i in qo] == sorted(cost, reverse=True)
+    assert ko[0] == 0
+
+
+def test_layout_arguments_are_checked():
+    lib = _lib.load_library()
+    prompt = np.asarray([4], dtype=np.int32)
+    sizes = np.asarray([2], dtype=np.int32)
+    resp = np.asarray([3, 2], dtype=np.int32)
+    out = np.zeros(64, dtype=np.int32)
+    assert lib.fca_split_layout_build(1, prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, 9, out.ctypes.data) == 0
+    assert lib.fca_split_layout_build(1, prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, 10, out.ctypes.data) < 0
+    assert b"holds 9 tokens" in lib.fca_last_error()
+    resp[1] = -1
+    assert lib.fca_split_layout_build(1, prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, 6, out.ctypes.data) < 0
+    plan = _lib.FcaSplitPlan(100, 6, 4, 128)
+    assert lib.fca_split_workspace_bytes(ctypes.byref(plan), None, None) < 0
+    plan = _lib.FcaSplitPlan(100, 8, 2, 128)
+    fwd, bwd = ctypes.c_size_t(), ctypes.c_size_t()
+    assert lib.fca_split_workspace_bytes(ctypes.byref(plan), ctypes.byref(fwd), ctypes.byref(bwd)) == 0
+    assert fwd.value == 128 * 2 * 128 * 2 and bwd.value == fwd.value + 2 * 128 * 8 * 128 * 2 + 128 * 8 * 4
+    with pytest.raises(RuntimeError, match="GPU"):
+        L = SplitLayout([(4, [3, 2])], device="cpu")
+        x = torch.zeros(9, 4, 64, dtype=torch.bfloat16)
+        split_attention_forward(x, x, x, L, 0.125)
+
+
+# ---- the kernels (GPU) ----------------------------------------------------------------------
+def _close(name, got, ref, scale_tol):
+    """bf16 results of fp32 accumulations over bf16 probabilities: 2e-2 relative plus
+    ``scale_tol`` of the tensor's largest magnitude."""
+    got, ref = got.detach().cpu().double(), ref.detach().double()
+    bound = scale_tol * ref.abs().max() + 2e-2 * ref.abs()
+    err = (got - ref).abs()
+    assert bool((err <= bound).all()), f"{name}: max |err| {err.max():.4g}, largest reference {ref.abs().max():.4g}"
+
+
+def _run_case(layout, hq, hkv, d, seed, strided=False):
+    q, k, v = _inputs(layout, hq, hkv, d, seed, torch.bfloat16)
+    t = q.shape[0]
+    scale = d**-0.5
+    L = SplitLayout(layout)
+    if strided:
+        # slices of one projection output [T, (Hq + 2 Hkv) * D], the way a fused QKV arrives
+        fused = torch.cat([q.reshape(t, -1), k.reshape(t, -1), v.reshape(t, -1)], dim=1).cuda()
+        qd = fused[:, : hq * d].view(t, hq, d)
+        kd = fused[:, hq * d : (hq + hkv) * d].view(t, hkv, d)
+        vd = fused[:, (hq + hkv) * d :].view(t, hkv, d)
+        assert qd.stride(0) == (hq + 2 * hkv) * d
+    else:
+        qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    out, lse = split_attention_forward(qd, kd, vd, L, scale)
+    q64, k64, v64 = (x.double().requires_grad_() for x in (q, k, v))
+    ro, rl = oracle_split(q64, k64, v64, layout, scale)
+    _close("out", out, ro, 2e-2 / max(1.0, float(ro.detach().abs().max())))
+    torch.testing.assert_close(lse[:, :t].T.cpu().double(), rl.detach(), rtol=1e-3, atol=1e-3)
+    dout = torch.randn(t, hq, d, generator=torch.Generator().manual_seed(seed + 1)).bfloat16()
+    ro.backward(dout.double())
+    dq, dk, dv = split_attention_backward(dout.cuda(), qd, kd, vd, out, lse, L, scale)
+    _close("dq", dq, q64.grad, 1e-2)
+    _close("dk", dk, k64.grad, 1e-2)
+    _close("dv", dv, v64.grad, 1e-2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("layout", LAYOUTS)
+@pytest.mark.parametrize("heads", [(4, 2, 128), (8, 1, 64), (2, 2, 128)])
+def test_forward_and_backward_match_the_oracle(layout, heads):
+    _run_case(layout, *heads, seed=21)
+
+
+@pytest.mark.gpu
+def test_random_layouts_match_the_oracle():
+    rng = random.Random(99)
+    done = 0
+    while done < 12:
+        layout = _random_layout(rng)
+        if total_tokens(layout) == 0:
+            continue
+        print("layout", layout, flush=True)
+        _run_case(layout, 4, 2, rng.choice([64, 128]), seed=done)
+        done += 1
+
+
+@pytest.mark.gpu
+def test_strided_inputs_of_a_fused_projection():
+    _run_case([(70, [40, 33, 12])], 8, 2, 128, seed=4, strided=True)
+
+
+@pytest.mark.gpu
+def test_training_shape_through_autograd():
+    """One group of a GRPO batch at real head counts: 8 responses over a prompt, Hq 32 /
+    Hkv 8 / D 128, through torch.autograd (what the trainer's layer would call)."""
+    layout = [(600, [300, 420, 150, 512, 64, 333, 200, 97])]
+    q, k, v = _inputs(layout, 32, 8, 128, 2, torch.bfloat16)
+    scale = 128**-0.5
+    L = SplitLayout.from_group_token_layout([{"prompt_tokens": 600, "response_tokens": layout[0][1]}])
+    qd, kd, vd = (x.cuda().requires_grad_() for x in (q, k, v))
+    out = split_attention(qd, kd, vd, L, scale)
+    w = torch.randn(out.shape, generator=torch.Generator().manual_seed(8)).bfloat16()
+    (out.float() * w.cuda().float()).sum().backward()
+    q64, k64, v64 = (x.double().requires_grad_() for x in (q, k, v))
+    ro, _ = oracle_split(q64, k64, v64, layout, scale)
+    (ro * w.double()).sum().backward()
+    _close("out", out, ro, 2e-2 / max(1.0, float(ro.detach().abs().max())))
+    _close("dq", qd.grad, q64.grad, 1e-2)
+    _close("dk", kd.grad, k64.grad, 1e-2)
+    _close("dv", vd.grad, v64.grad, 1e-2)
+    # the layout serves a second layer without new scratch
+    before = {k_: b.data_ptr() for k_, b in L._scratch.items()}
+    split_attention(qd, kd, vd, L, scale).sum().backward()
+    assert before == {k_: b.data_ptr() for k_, b in L._scratch.items()}
