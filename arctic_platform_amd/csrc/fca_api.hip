@@ -380,8 +380,8 @@ int fca_split_layout_build(int32_t num_groups, const int32_t* prompt_tokens, con
 int fca_split_workspace_bytes(const fca_split_plan* plan, size_t* forward_bytes, size_t* backward_bytes) {
   if (int rc = check_split(plan)) return rc;
   const SplitScratch s = split_scratch(plan);
-  if (forward_bytes) *forward_bytes = s.kv_tiles;
-  if (backward_bytes) *backward_bytes = s.kv_tiles + 2 * s.q_tiles + s.delta;
+  if (forward_bytes) *forward_bytes = 2 * s.kv_tiles;
+  if (backward_bytes) *backward_bytes = 3 * s.kv_tiles + 4 * s.q_tiles + s.delta;
   return FCA_OK;
 }
 
@@ -402,7 +402,8 @@ int fca_split_attention_forward(const fca_split_plan* plan, const void* q_dev, i
   fca::SplitParams p{};
   p.q = q_dev, p.k = k_dev, p.v = v_dev;
   p.q_stride = q_stride, p.k_stride = k_stride, p.v_stride = v_stride, p.o_stride = out_stride;
-  p.vt = workspace_dev;
+  p.kn = workspace_dev;
+  p.vr = static_cast<char*>(workspace_dev) + split_scratch(plan).kv_tiles;
   p.out = out_dev;
   p.lse = lse_dev;
   p.layout = layout_dev;
@@ -441,10 +442,14 @@ int fca_split_attention_backward(const fca_split_plan* plan, const void* q_dev, 
   fca::SplitParams p{};
   p.q = q_dev, p.k = k_dev, p.v = v_dev, p.out_in = out_dev, p.dout = dout_dev;
   p.q_stride = q_stride, p.k_stride = k_stride, p.v_stride = v_stride, p.o_stride = out_stride, p.do_stride = dout_stride;
-  p.kt = ws;
-  p.qt = ws + s.kv_tiles;
-  p.dot = ws + s.kv_tiles + s.q_tiles;
-  p.delta = reinterpret_cast<float*>(ws + s.kv_tiles + 2 * s.q_tiles);
+  p.kn = ws;
+  p.kr = ws + s.kv_tiles;
+  p.vn = ws + 2 * s.kv_tiles;
+  p.qn = ws + 3 * s.kv_tiles;
+  p.qr = ws + 3 * s.kv_tiles + s.q_tiles;
+  p.don = ws + 3 * s.kv_tiles + 2 * s.q_tiles;
+  p.dor = ws + 3 * s.kv_tiles + 3 * s.q_tiles;
+  p.delta = reinterpret_cast<float*>(ws + 3 * s.kv_tiles + 4 * s.q_tiles);
   p.lse = const_cast<float*>(lse_dev);
   p.dq = dq_dev, p.dk = dk_dev, p.dv = dv_dev;
   p.dq_stride = dq_stride, p.dk_stride = dk_stride, p.dv_stride = dv_stride;

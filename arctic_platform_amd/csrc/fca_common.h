@@ -186,7 +186,9 @@ struct AppendParams {
 struct SplitParams {
   const void *q, *k, *v, *out_in, *dout;
   int64_t q_stride, k_stride, v_stride, o_stride, do_stride;  // token strides, elements
-  const void *kt, *vt, *qt, *dot;
+  // operand images of 32-token tiles, [H][tiles][slot][64 lanes][8]: `n` = rows as the first
+  // product of a chain takes them, `r` = transposed as the second product takes them
+  const void *kn, *kr, *vn, *vr, *qn, *qr, *don, *dor;
   void* out;
   float* lse;    // [Hq][tiles * 32] natural log
   float* delta;  // [Hq][tiles * 32] rowsum(dout * out)
@@ -212,8 +214,8 @@ __host__ __device__ inline SplitLayout make_split_layout(int64_t tiles) {
 }
 void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,
                         const int32_t* response_tokens, int64_t tiles, int32_t* out);
-hipError_t launch_split_transpose(const void* x, int64_t stride, int heads, int head_dim, int num_tokens, int tiles,
-                                  void* xt, hipStream_t stream);
+hipError_t launch_split_images(const void* x, int64_t stride, int heads, int head_dim, int num_tokens, int tiles,
+                               void* rows_image, void* transposed_image, hipStream_t stream);
 hipError_t launch_split_forward(const SplitParams& p, int head_dim, hipStream_t stream);
 hipError_t launch_split_backward(const SplitParams& p, int head_dim, hipStream_t stream);
 

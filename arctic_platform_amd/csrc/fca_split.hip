@@ -41,12 +41,14 @@ void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int3
                         const int32_t* response_tokens, int64_t tiles, int32_t* out) {
   const SplitLayout L = make_split_layout(tiles);
   const int64_t padded = 32 * tiles;
-  std::vector<int32_t> own(padded, 0), pstart(padded, 0), pend(padded, 0);
+  std::vector<int32_t> own(padded, 0), pstart(padded, 0), pend(padded, 0), group_of(padded, 0);
   int32_t* lim = out + L.kv_lim;
   int64_t t = 0;
   int64_t ri = 0;
+  int group = 0;
   auto fill = [&](int64_t from, int64_t to, int64_t limit, int64_t p0, int64_t p1) {
     for (int64_t x = from; x < to; ++x) {
+      group_of[x] = group;
       lim[x] = (int32_t)limit;
       own[x] = (int32_t)from;
       pstart[x] = (int32_t)p0;
@@ -54,6 +56,7 @@ void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int3
     }
   };
   for (int g = 0; g < num_groups; ++g) {
+    group = g;
     const int64_t p0 = t, p1 = t + prompt_tokens[g];
     int64_t gend = p1;
     for (int s = 0; s < group_sizes[g]; ++s) gend += response_tokens[ri + s];
@@ -67,7 +70,7 @@ void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int3
     ri += group_sizes[g];
   }
   for (int64_t x = t; x < padded; ++x) lim[x] = 0;
-  std::vector<int64_t> qcost(tiles), kcost(tiles);
+  std::vector<int64_t> qcost(tiles);
   for (int64_t i = 0; i < tiles; ++i) {
     // The needs of a tile's first row cover those of the rows behind it: they belong to
     // later segments, whose own tokens and (if the group changes inside the tile) prompt
@@ -83,14 +86,17 @@ void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int3
     int32_t mx = 0;
     for (int x = 0; x < 32; ++x) mx = std::max(mx, lim[r0 + x]);
     out[L.kv_qend + i] = (mx + 31) / 32;
-    kcost[i] = out[L.kv_qend + i] - i;
   }
-  auto order = [&](const std::vector<int64_t>& cost, int32_t* dst) {
-    std::iota(dst, dst + tiles, 0);
-    std::stable_sort(dst, dst + tiles, [&](int32_t a, int32_t b) { return cost[a] > cost[b]; });
-  };
-  order(qcost, out + L.q_order);
-  order(kcost, out + L.kv_order);
+  // Query tiles: group by group, so that the workgroups in flight read the same prompt, and
+  // the longest walks of a group first.  Key tiles are taken in packed order, four adjacent
+  // ones per workgroup: within a group that is the prompt's tiles, the heaviest, first.
+  int32_t* qo = out + L.q_order;
+  std::iota(qo, qo + tiles, 0);
+  std::stable_sort(qo, qo + tiles, [&](int32_t a, int32_t b) {
+    const int ga = group_of[32 * (int64_t)a], gb = group_of[32 * (int64_t)b];
+    return ga != gb ? ga < gb : qcost[a] > qcost[b];
+  });
+  std::iota(out + L.kv_order, out + L.kv_order + tiles, 0);
 }
 
 namespace {
@@ -123,26 +129,38 @@ __device__ inline void store_rows(void* dst, int64_t row_elem, int h, const f32x
     }
 }
 
-// ---- transposed tiles ---------------------------------------------------------------------
+// ---- operand images --------------------------------------------------------------------------
+// One workgroup per (tile, head): the tile's 32 rows go through LDS and leave in MFMA operand
+// order, 16 bytes per lane and slot, so that every operand load of the attention kernels is
+// one contiguous kilobyte per wave.
+//   rows image        slot s, lane (m, h):        x[fed_row(m)][16 s + 8 h .. + 7]
+//   transposed image  slot (blk, db), lane (m, h): x[16 blk + 8 h + i][32 db + m], i = 0 .. 7
+// Rows past the last token are zero.
 template <int D>
-__global__ __launch_bounds__(kThreads) void split_transpose_kernel(const __bf16* x, int64_t stride, int T, int nt,
-                                                                  __bf16* xt) {
-  __shared__ __attribute__((aligned(16))) __bf16 tile[D][40];
+__global__ __launch_bounds__(kThreads) void split_images_kernel(const __bf16* x, int64_t stride, int T, int nt,
+                                                               __bf16* rows_image, __bf16* transposed_image) {
+  __shared__ __attribute__((aligned(16))) __bf16 tile[32][D + 8];
   const int j = blockIdx.x, hh = blockIdx.y;
   for (int p = threadIdx.x; p < 32 * D / 8; p += kThreads) {
     const int tk = p / (D / 8), c = (p % (D / 8)) * 8;
     const int64_t t = 32 * (int64_t)j + tk;
     i32x4 w = {0, 0, 0, 0};
     if (t < T) w = ld16(x, t * stride + hh * D + c);
-    const bf16x8 e = as_bf16(w);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) tile[c + i][tk] = e[i];
+    *reinterpret_cast<i32x4*>(&tile[tk][c]) = w;
   }
   __syncthreads();
-  __bf16* dst = xt + ((int64_t)hh * nt + j) * D * 32;
-  for (int p = threadIdx.x; p < D * 4; p += kThreads) {
-    const int d = p / 4, part = p % 4;
-    *reinterpret_cast<i32x4*>(dst + d * 32 + part * 8) = *reinterpret_cast<const i32x4*>(&tile[d][part * 8]);
+  const int64_t base = ((int64_t)hh * nt + j) * (D / 16) * 512;
+  for (int p = threadIdx.x; p < (D / 16) * 64; p += kThreads) {
+    const int slot = p / 64, l = p % 64, m = l & 31, h = l >> 5;
+    if (rows_image)
+      *reinterpret_cast<i32x4*>(rows_image + base + p * 8) = *reinterpret_cast<const i32x4*>(&tile[fed_row(m)][16 * slot + 8 * h]);
+    if (transposed_image) {
+      const int blk = slot / (D / 32), db = slot % (D / 32);
+      bf16x8 e;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) e[i] = tile[16 * blk + 8 * h + i][32 * db + m];
+      *reinterpret_cast<bf16x8*>(transposed_image + base + p * 8) = e;
+    }
   }
 }
 
@@ -185,12 +203,16 @@ __global__ __launch_bounds__(kThreads, 1) void split_query_kernel(SplitParams p)
   const SplitLayout L = make_split_layout(p.num_tiles);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 31, h = lane >> 5;
-  const int hq = blockIdx.y * kWaves + wave;
+  // consecutive workgroups go to different XCDs: with the head quad running fastest an XCD
+  // keeps to the same KV heads (when their number divides 8 or is a multiple of it) and its
+  // L2 holds their K and V of the group in flight
+  const int quads = (p.num_q_heads + kWaves - 1) / kWaves;
+  const int hq = (blockIdx.x % quads) * kWaves + wave;
   if (hq >= p.num_q_heads) return;
   const int hkv = hq / (p.num_q_heads / p.num_kv_heads);
   const int T = p.num_tokens, nt = p.num_tiles;
   const int64_t padded = 32 * (int64_t)nt;
-  const int i = __builtin_amdgcn_readfirstlane(p.layout[L.q_order + blockIdx.x]);
+  const int i = __builtin_amdgcn_readfirstlane(p.layout[L.q_order + blockIdx.x / quads]);
   const int a0 = __builtin_amdgcn_readfirstlane(p.layout[L.q_tiles + 4 * i]);
   const int a1 = __builtin_amdgcn_readfirstlane(p.layout[L.q_tiles + 4 * i + 1]);
   const int b0 = __builtin_amdgcn_readfirstlane(p.layout[L.q_tiles + 4 * i + 2]);
@@ -208,7 +230,7 @@ __global__ __launch_bounds__(kThreads, 1) void split_query_kernel(SplitParams p)
     lse2 = p.lse[hq * padded + r] * kLog2e;
     delta = p.delta[hq * padded + r];
   }
-  const void* trsrc = BWD ? p.kt : p.vt;
+  const void* trsrc = BWD ? p.kr : p.vr;
   const float sc = p.scale * kLog2e;
 
   f32x16 acc[NDB];
@@ -222,18 +244,17 @@ __global__ __launch_bounds__(kThreads, 1) void split_query_kernel(SplitParams p)
     idx = min(idx, ntile - 1);
     const int j = idx < na ? a0 + idx : b0 + idx - na;
     t.j = j;
-    const int64_t tok = min(32 * j + fed_row(n), T - 1);
+    const int64_t base = ((int64_t)hkv * nt + j) * KS * 512 + lane * 8;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) t.k[s] = ld16(p.k, tok * p.k_stride + hkv * D + 16 * s + 8 * h);
+    for (int s = 0; s < KS; ++s) t.k[s] = ld16(p.kn, base + s * 512);
     if constexpr (BWD) {
 #pragma unroll
-      for (int s = 0; s < KS; ++s) t.vn[s] = ld16(p.v, tok * p.v_stride + hkv * D + 16 * s + 8 * h);
+      for (int s = 0; s < KS; ++s) t.vn[s] = ld16(p.vn, base + s * 512);
     }
-    const int64_t base = (((int64_t)hkv * nt + j) * D + n) * 32 + 8 * h;
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-      for (int db = 0; db < NDB; ++db) t.tr[blk][db] = ld16(trsrc, base + (int64_t)db * 32 * 32 + 16 * blk);
+      for (int db = 0; db < NDB; ++db) t.tr[blk][db] = ld16(trsrc, base + (blk * NDB + db) * 512);
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
@@ -331,12 +352,14 @@ __global__ __launch_bounds__(kThreads, 1) void split_key_kernel(SplitParams p) {
   const SplitLayout L = make_split_layout(p.num_tiles);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 31, h = lane >> 5;
-  const int hkv = blockIdx.y * kWaves + wave;
-  if (hkv >= p.num_kv_heads) return;
+  // a workgroup = four adjacent key tiles of one KV head: its waves walk nearly the same
+  // query tiles at the same time
+  const int hkv = blockIdx.x % p.num_kv_heads;
   const int group = p.num_q_heads / p.num_kv_heads;
   const int T = p.num_tokens, nt = p.num_tiles;
   const int64_t padded = 32 * (int64_t)nt;
-  const int j = __builtin_amdgcn_readfirstlane(p.layout[L.kv_order + blockIdx.x]);
+  const int j = (blockIdx.x / p.num_kv_heads) * kWaves + wave;
+  if (j >= nt) return;
   const int qend = __builtin_amdgcn_readfirstlane(p.layout[L.kv_qend + j]);
   const int t = 32 * j + n;
   const int64_t tc = min(t, T - 1);
@@ -356,23 +379,22 @@ __global__ __launch_bounds__(kThreads, 1) void split_key_kernel(SplitParams p) {
     for (int x = 0; x < 16; ++x) acck[db][x] = 0.f, accv[db][x] = 0.f;
 
   for (int i = j; i < qend; ++i) {
-    const int64_t row = min(32 * i + fed_row(n), T - 1);
     for (int g = 0; g < group; ++g) {
       const int hq = hkv * group + g;
       i32x4 qn[KS], don[KS], qtr[2][NDB], dotr[2][NDB];
       f32x4 ls[2][2], dl[2][2];
+      const int64_t base = ((int64_t)hq * nt + i) * KS * 512 + lane * 8;
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
-        qn[s] = ld16(p.q, row * p.q_stride + hq * D + 16 * s + 8 * h);
-        don[s] = ld16(p.dout, row * p.do_stride + hq * D + 16 * s + 8 * h);
+        qn[s] = ld16(p.qn, base + s * 512);
+        don[s] = ld16(p.don, base + s * 512);
       }
-      const int64_t base = (((int64_t)hq * nt + i) * D + n) * 32 + 8 * h;
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
         for (int db = 0; db < NDB; ++db) {
-          qtr[blk][db] = ld16(p.qt, base + (int64_t)db * 32 * 32 + 16 * blk);
-          dotr[blk][db] = ld16(p.dot, base + (int64_t)db * 32 * 32 + 16 * blk);
+          qtr[blk][db] = ld16(p.qr, base + (blk * NDB + db) * 512);
+          dotr[blk][db] = ld16(p.dor, base + (blk * NDB + db) * 512);
         }
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk)
@@ -424,23 +446,26 @@ hipError_t by_head_dim(int head_dim, F&& f) {
 
 }  // namespace
 
-hipError_t launch_split_transpose(const void* x, int64_t stride, int heads, int head_dim, int num_tokens, int tiles,
-                                  void* xt, hipStream_t stream) {
+hipError_t launch_split_images(const void* x, int64_t stride, int heads, int head_dim, int num_tokens, int tiles,
+                               void* rows_image, void* transposed_image, hipStream_t stream) {
   return by_head_dim(head_dim, [&](auto d) {
     constexpr int D = decltype(d)::value;
-    split_transpose_kernel<D><<<dim3(tiles, heads), kThreads, 0, stream>>>(static_cast<const __bf16*>(x), stride, num_tokens,
-                                                                          tiles, static_cast<__bf16*>(xt));
+    split_images_kernel<D><<<dim3(tiles, heads), kThreads, 0, stream>>>(static_cast<const __bf16*>(x), stride, num_tokens, tiles,
+                                                                       static_cast<__bf16*>(rows_image),
+                                                                       static_cast<__bf16*>(transposed_image));
     return hipGetLastError();
   });
 }
 
 hipError_t launch_split_forward(const SplitParams& p, int head_dim, hipStream_t stream) {
-  if (hipError_t e = launch_split_transpose(p.v, p.v_stride, p.num_kv_heads, head_dim, p.num_tokens, p.num_tiles,
-                                            const_cast<void*>(p.vt), stream))
+  const int T = p.num_tokens, nt = p.num_tiles;
+  if (hipError_t e = launch_split_images(p.k, p.k_stride, p.num_kv_heads, head_dim, T, nt, const_cast<void*>(p.kn), nullptr, stream))
+    return e;
+  if (hipError_t e = launch_split_images(p.v, p.v_stride, p.num_kv_heads, head_dim, T, nt, nullptr, const_cast<void*>(p.vr), stream))
     return e;
   return by_head_dim(head_dim, [&](auto d) {
     constexpr int D = decltype(d)::value;
-    const dim3 grid(p.num_tiles, (p.num_q_heads + kWaves - 1) / kWaves);
+    const unsigned grid = (unsigned)p.num_tiles * ((p.num_q_heads + kWaves - 1) / kWaves);
     split_query_kernel<D, false><<<grid, kThreads, 0, stream>>>(p);
     return hipGetLastError();
   });
@@ -448,21 +473,20 @@ hipError_t launch_split_forward(const SplitParams& p, int head_dim, hipStream_t 
 
 hipError_t launch_split_backward(const SplitParams& p, int head_dim, hipStream_t stream) {
   const int T = p.num_tokens, nt = p.num_tiles;
-  if (hipError_t e = launch_split_transpose(p.k, p.k_stride, p.num_kv_heads, head_dim, T, nt, const_cast<void*>(p.kt), stream))
-    return e;
-  if (hipError_t e = launch_split_transpose(p.q, p.q_stride, p.num_q_heads, head_dim, T, nt, const_cast<void*>(p.qt), stream))
-    return e;
-  if (hipError_t e = launch_split_transpose(p.dout, p.do_stride, p.num_q_heads, head_dim, T, nt, const_cast<void*>(p.dot), stream))
-    return e;
+  auto V = [](const void* x) { return const_cast<void*>(x); };
+  if (hipError_t e = launch_split_images(p.k, p.k_stride, p.num_kv_heads, head_dim, T, nt, V(p.kn), V(p.kr), stream)) return e;
+  if (hipError_t e = launch_split_images(p.v, p.v_stride, p.num_kv_heads, head_dim, T, nt, V(p.vn), nullptr, stream)) return e;
+  if (hipError_t e = launch_split_images(p.q, p.q_stride, p.num_q_heads, head_dim, T, nt, V(p.qn), V(p.qr), stream)) return e;
+  if (hipError_t e = launch_split_images(p.dout, p.do_stride, p.num_q_heads, head_dim, T, nt, V(p.don), V(p.dor), stream)) return e;
   return by_head_dim(head_dim, [&](auto d) {
     constexpr int D = decltype(d)::value;
     const int64_t rows = 32 * (int64_t)nt * p.num_q_heads;
     const int per_block = kThreads / (D / 8);
     split_delta_kernel<D><<<(unsigned)((rows + per_block - 1) / per_block), kThreads, 0, stream>>>(p);
     if (hipError_t e = hipGetLastError()) return e;
-    split_query_kernel<D, true><<<dim3(nt, (p.num_q_heads + kWaves - 1) / kWaves), kThreads, 0, stream>>>(p);
+    split_query_kernel<D, true><<<(unsigned)nt * ((p.num_q_heads + kWaves - 1) / kWaves), kThreads, 0, stream>>>(p);
     if (hipError_t e = hipGetLastError()) return e;
-    split_key_kernel<D><<<dim3(nt, (p.num_kv_heads + kWaves - 1) / kWaves), kThreads, 0, stream>>>(p);
+    split_key_kernel<D><<<(unsigned)((nt + kWaves - 1) / kWaves) * p.num_kv_heads, kThreads, 0, stream>>>(p);
     return hipGetLastError();
   });
 }

@@ -165,7 +165,8 @@ def test_layout_arguments_are_checked():
     plan = _lib.FcaSplitPlan(100, 8, 2, 128)
     fwd, bwd = ctypes.c_size_t(), ctypes.c_size_t()
     assert lib.fca_split_workspace_bytes(ctypes.byref(plan), ctypes.byref(fwd), ctypes.byref(bwd)) == 0
-    assert fwd.value == 128 * 2 * 128 * 2 and bwd.value == fwd.value + 2 * 128 * 8 * 128 * 2 + 128 * 8 * 4
+    kv, qq = 128 * 2 * 128 * 2, 128 * 8 * 128 * 2
+    assert fwd.value == 2 * kv and bwd.value == 3 * kv + 4 * qq + 128 * 8 * 4
     with pytest.raises(RuntimeError, match="GPU"):
         L = SplitLayout([(4, [3, 2])], device="cpu")
         x = torch.zeros(9, 4, 64, dtype=torch.bfloat16)
