@@ -200,7 +200,7 @@ struct SplitParams {
 };
 // Offsets into the int32 layout array of a batch of `tiles` 32-token tiles.
 struct SplitLayout {
-  int64_t kv_lim, q_tiles, kv_qend, q_order, kv_order, total;
+  int64_t kv_lim, q_tiles, kv_qend, q_order, kv_limmin, total;
 };
 __host__ __device__ inline SplitLayout make_split_layout(int64_t tiles) {
   SplitLayout L;
@@ -208,8 +208,8 @@ __host__ __device__ inline SplitLayout make_split_layout(int64_t tiles) {
   L.q_tiles = 32 * tiles;
   L.kv_qend = L.q_tiles + 4 * tiles;
   L.q_order = L.kv_qend + tiles;
-  L.kv_order = L.q_order + tiles;
-  L.total = L.kv_order + tiles;
+  L.kv_limmin = L.q_order + tiles;
+  L.total = L.kv_limmin + tiles;
   return L;
 }
 void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,

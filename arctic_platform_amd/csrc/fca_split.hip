@@ -86,6 +86,9 @@ void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int3
     int32_t mx = 0;
     for (int x = 0; x < 32; ++x) mx = std::max(mx, lim[r0 + x]);
     out[L.kv_qend + i] = (mx + 31) / 32;
+    int32_t mn = lim[r0];
+    for (int x = 1; x < 32; ++x) mn = std::min(mn, lim[r0 + x]);
+    out[L.kv_limmin + i] = mn;
   }
   // Query tiles: group by group, so that the workgroups in flight read the same prompt, and
   // the longest walks of a group first.  Key tiles are taken in packed order, four adjacent
@@ -96,7 +99,7 @@ void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int3
     const int ga = group_of[32 * (int64_t)a], gb = group_of[32 * (int64_t)b];
     return ga != gb ? ga < gb : qcost[a] > qcost[b];
   });
-  std::iota(out + L.kv_order, out + L.kv_order + tiles, 0);
+
 }
 
 namespace {
@@ -187,28 +190,28 @@ __global__ __launch_bounds__(kThreads) void split_delta_kernel(SplitParams p) {
 }
 
 // ---- forward and dq: one wave per (query tile, query head) -----------------------------------
-template <int D, bool BWD>
-struct KeyTile {
-  i32x4 k[D / 16];                   // K rows, first product
-  i32x4 vn[BWD ? D / 16 : 1];        // V rows (dq: dP)
-  i32x4 tr[2][D / 32];               // transposed tile: V (forward), K (dq)
-  i32x4 lim[2][2];
-  int j;
-};
-
-template <int D, bool BWD>
-__global__ __launch_bounds__(kThreads, 1) void split_query_kernel(SplitParams p) {
-  constexpr int KS = D / 16, NDB = D / 32;
-  using Tile = KeyTile<D, BWD>;
+// Operand slots of one key tile, 1 KB each: K rows [0, KS), then (dq) V rows [KS, 2 KS), then
+// the transposed image, V's (forward) or K's (dq).
+// SHARED: the four waves of a workgroup are four query heads of one KV head on the same query
+// tile, so they walk the same key tiles: each wave fetches a quarter of a tile's slots one
+// tile ahead, the tile is passed around through LDS (two buffers, one barrier per tile) and
+// the L1 sees a quarter of the operand traffic.  Without it (query heads per KV head not a
+// multiple of four) every wave fetches its own tiles into two register buffers.
+template <int D, bool BWD, bool SHARED>
+__global__ __launch_bounds__(kThreads, SHARED ? 2 : 1) void split_query_kernel(SplitParams p) {
+  constexpr int KS = D / 16, NDB = D / 32, SLOTS = (BWD ? 3 : 2) * KS, PER = SLOTS / kWaves;
+  __shared__ i32x4 lds[SHARED ? 2 : 1][SHARED ? SLOTS : 1][64];
   const SplitLayout L = make_split_layout(p.num_tiles);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
   // consecutive workgroups go to different XCDs: with the head quad running fastest an XCD
   // keeps to the same KV heads (when their number divides 8 or is a multiple of it) and its
   // L2 holds their K and V of the group in flight
   const int quads = (p.num_q_heads + kWaves - 1) / kWaves;
   const int hq = (blockIdx.x % quads) * kWaves + wave;
-  if (hq >= p.num_q_heads) return;
+  if constexpr (!SHARED) {
+    if (hq >= p.num_q_heads) return;
+  }
   const int hkv = hq / (p.num_q_heads / p.num_kv_heads);
   const int T = p.num_tokens, nt = p.num_tiles;
   const int64_t padded = 32 * (int64_t)nt;
@@ -230,7 +233,6 @@ __global__ __launch_bounds__(kThreads, 1) void split_query_kernel(SplitParams p)
     lse2 = p.lse[hq * padded + r] * kLog2e;
     delta = p.delta[hq * padded + r];
   }
-  const void* trsrc = BWD ? p.kr : p.vr;
   const float sc = p.scale * kLog2e;
 
   f32x16 acc[NDB];
@@ -240,46 +242,47 @@ __global__ __launch_bounds__(kThreads, 1) void split_query_kernel(SplitParams p)
     for (int x = 0; x < 16; ++x) acc[db][x] = 0.f;
   float mrow = -1e30f, lrow = 0.f;
 
-  auto load = [&](Tile& t, int idx) {
+  auto tile_of = [&](int idx) {
     idx = min(idx, ntile - 1);
-    const int j = idx < na ? a0 + idx : b0 + idx - na;
-    t.j = j;
-    const int64_t base = ((int64_t)hkv * nt + j) * KS * 512 + lane * 8;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) t.k[s] = ld16(p.kn, base + s * 512);
-    if constexpr (BWD) {
-#pragma unroll
-      for (int s = 0; s < KS; ++s) t.vn[s] = ld16(p.vn, base + s * 512);
-    }
-#pragma unroll
-    for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-      for (int db = 0; db < NDB; ++db) t.tr[blk][db] = ld16(trsrc, base + (blk * NDB + db) * 512);
-#pragma unroll
-    for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-      for (int half = 0; half < 2; ++half)
-        t.lim[blk][half] = *reinterpret_cast<const i32x4*>(p.layout + L.kv_lim + 32 * j + 16 * blk + 8 * h + 4 * half);
+    return idx < na ? a0 + idx : b0 + idx - na;
+  };
+  // slot of a tile -> its place in the images (every image holds KS slots per tile)
+  auto slot_ptr = [&](int j, int slot) {
+    const void* src = slot < KS ? p.kn : !BWD ? p.vr : slot < 2 * KS ? p.vn : p.kr;
+    return static_cast<const __bf16*>(src) + (((int64_t)hkv * nt + j) * KS + slot % KS) * 512 + lane * 8;
   };
 
-  auto compute = [&](const Tile& t) {
+  // one key tile: `get(slot)` hands out operand registers; `limmin` = smallest lim of the tile
+  auto compute = [&](int j, int limmin, auto&& get) {
     f32x16 sr;
 #pragma unroll
     for (int x = 0; x < 16; ++x) sr[x] = 0.f;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) sr = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(t.k[s]), qreg[s], sr, 0, 0, 0);
-    const int tok0 = 32 * t.j + 8 * h;
+    for (int s = 0; s < KS; ++s) sr = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(get(s)), qreg[s], sr, 0, 0, 0);
+    // every row of this query tile sees every token of an earlier tile whose limits all lie
+    // behind the query tile; anything else is tested element by element
     bool ok[16];
 #pragma unroll
-    for (int x = 0; x < 16; ++x) {
-      const int tok = tok0 + 16 * (x >> 3) + (x & 7);
-      ok[x] = tok <= r && t.lim[x >> 3][(x >> 2) & 1][x & 3] > r;
+    for (int x = 0; x < 16; ++x) ok[x] = true;
+    const bool masked = !(j < i && limmin >= 32 * i + 32);
+    if (masked) {
+      const int tok0 = 32 * j + 8 * h;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const i32x4 lim = *reinterpret_cast<const i32x4*>(p.layout + L.kv_lim + tok0 + 16 * blk + 4 * half);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) ok[8 * blk + 4 * half + e] = tok0 + 16 * blk + 4 * half + e <= r && lim[e] > r;
+        }
     }
     bf16x8 pb[2];
     if constexpr (!BWD) {
+      if (masked) {
 #pragma unroll
-      for (int x = 0; x < 16; ++x)
-        if (!ok[x]) sr[x] = -INFINITY;
+        for (int x = 0; x < 16; ++x)
+          if (!ok[x]) sr[x] = -INFINITY;
+      }
       float mx = sr[0];
 #pragma unroll
       for (int x = 1; x < 16; ++x) mx = fmaxf(mx, sr[x]);
@@ -310,7 +313,7 @@ __global__ __launch_bounds__(kThreads, 1) void split_query_kernel(SplitParams p)
 #pragma unroll
       for (int x = 0; x < 16; ++x) dp[x] = 0.f;
 #pragma unroll
-      for (int s = 0; s < KS; ++s) dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(t.vn[s]), doreg[s], dp, 0, 0, 0);
+      for (int s = 0; s < KS; ++s) dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(get(KS + s)), doreg[s], dp, 0, 0, 0);
 #pragma unroll
       for (int x = 0; x < 16; ++x) {
         const float e = ok[x] ? fast_exp2(__builtin_fmaf(sr[x], sc, -lse2)) : 0.f;
@@ -321,18 +324,54 @@ __global__ __launch_bounds__(kThreads, 1) void split_query_kernel(SplitParams p)
     for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
       for (int db = 0; db < NDB; ++db)
-        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(t.tr[blk][db]), pb[blk], acc[db], 0, 0, 0);
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(get(SLOTS - KS + blk * NDB + db)), pb[blk], acc[db], 0, 0, 0);
   };
 
-  // two tile buffers: the next tile is requested before the current one is used; requests
-  // past the end repeat the last tile, so every path issues the same loads
-  Tile ta, tb;
-  load(ta, 0);
-  for (int idx = 0; idx < ntile; idx += 2) {
-    load(tb, idx + 1);
-    compute(ta);
-    load(ta, idx + 2);
-    if (idx + 1 < ntile) compute(tb);
+  if constexpr (SHARED) {
+    // requests past the end repeat the last tile, so every path issues the same loads
+    i32x4 pf[PER];
+    int pf_limmin;
+    auto fetch = [&](int idx) {
+      const int j = tile_of(idx);
+#pragma unroll
+      for (int x = 0; x < PER; ++x) pf[x] = ld16(slot_ptr(j, wave * PER + x), 0);
+      pf_limmin = p.layout[L.kv_limmin + j];
+    };
+    auto publish = [&](int buf) {
+#pragma unroll
+      for (int x = 0; x < PER; ++x) lds[buf][wave * PER + x][lane] = pf[x];
+    };
+    fetch(0);
+    publish(0);
+    int limmin = __builtin_amdgcn_readfirstlane(pf_limmin);
+    __syncthreads();
+    for (int idx = 0; idx < ntile; ++idx) {
+      const int buf = idx & 1;
+      fetch(idx + 1);
+      compute(tile_of(idx), limmin, [&](int slot) { return lds[buf][slot][lane]; });
+      publish(buf ^ 1);
+      limmin = __builtin_amdgcn_readfirstlane(pf_limmin);
+      __syncthreads();
+    }
+  } else {
+    struct Tile {
+      i32x4 s[SLOTS];
+      int j, limmin;
+    };
+    auto load = [&](Tile& t, int idx) {
+      t.j = tile_of(idx);
+#pragma unroll
+      for (int x = 0; x < SLOTS; ++x) t.s[x] = ld16(slot_ptr(t.j, x), 0);
+      t.limmin = p.layout[L.kv_limmin + t.j];
+    };
+    Tile ta, tb;
+    load(ta, 0);
+    for (int idx = 0; idx < ntile; idx += 2) {
+      load(tb, idx + 1);
+      compute(ta.j, __builtin_amdgcn_readfirstlane(ta.limmin), [&](int slot) { return ta.s[slot]; });
+      load(ta, idx + 2);
+      if (idx + 1 < ntile) compute(tb.j, __builtin_amdgcn_readfirstlane(tb.limmin), [&](int slot) { return tb.s[slot]; });
+    }
   }
 
   if constexpr (!BWD) {
@@ -346,94 +385,133 @@ __global__ __launch_bounds__(kThreads, 1) void split_query_kernel(SplitParams p)
 }
 
 // ---- dk, dv: one wave per (key tile, KV head) --------------------------------------------------
-template <int D>
-__global__ __launch_bounds__(kThreads, 1) void split_key_kernel(SplitParams p) {
-  constexpr int KS = D / 16, NDB = D / 32;
+// A workgroup = four adjacent key tiles of one KV head.  Its waves need the same stream of
+// query-side operands, one step per (query tile, query head of the KV head): each wave
+// fetches a quarter of a step's slots one step ahead and the step is passed around through
+// LDS.  A wave computes only the steps inside its own tile's range of query tiles.  dV and dK
+// are two launches (DK = false / true): each keeps one set of accumulators, which leaves
+// room for two workgroups per CU, at the price of forming the probabilities twice.
+//   dV: slots Q rows [0, KS), dO transposed [KS, 2 KS):   P = exp(S - lse),  dVt += dOt . P
+//   dK: slots Q rows, dO rows, Q transposed:   dS = P (dO . V - delta),      dKt += Qt . dS
+template <int D, bool DK>
+__global__ __launch_bounds__(kThreads, 2) void split_key_kernel(SplitParams p) {
+  constexpr int KS = D / 16, NDB = D / 32, SLOTS = (DK ? 3 : 2) * KS, PER = SLOTS / kWaves;
+  __shared__ i32x4 lds[2][SLOTS][64];
+  __shared__ __attribute__((aligned(16))) float lds_ls[2][32], lds_dl[2][32];  // lse, delta of the step's rows
   const SplitLayout L = make_split_layout(p.num_tiles);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
-  // a workgroup = four adjacent key tiles of one KV head: its waves walk nearly the same
-  // query tiles at the same time
   const int hkv = blockIdx.x % p.num_kv_heads;
   const int group = p.num_q_heads / p.num_kv_heads;
   const int T = p.num_tokens, nt = p.num_tiles;
   const int64_t padded = 32 * (int64_t)nt;
-  const int j = (blockIdx.x / p.num_kv_heads) * kWaves + wave;
-  if (j >= nt) return;
-  const int qend = __builtin_amdgcn_readfirstlane(p.layout[L.kv_qend + j]);
+  const int j0 = (blockIdx.x / p.num_kv_heads) * kWaves;
+  const int j = min(j0 + wave, nt - 1);  // a wave past the last tile repeats it and stores nothing
+  const bool live = j0 + wave < nt;
+  const int qend = live ? __builtin_amdgcn_readfirstlane(p.layout[L.kv_qend + j]) : 0;
+  const int limmin = __builtin_amdgcn_readfirstlane(p.layout[L.kv_limmin + j]);
+  int qend_all = 0;
+  for (int w = 0; w < kWaves; ++w)
+    if (j0 + w < nt) qend_all = max(qend_all, __builtin_amdgcn_readfirstlane(p.layout[L.kv_qend + j0 + w]));
   const int t = 32 * j + n;
   const int64_t tc = min(t, T - 1);
   const int lim_t = p.layout[L.kv_lim + t];
   const float sc = p.scale * kLog2e;
 
-  bf16x8 kreg[KS], vreg[KS];
+  bf16x8 kreg[KS], vreg[DK ? KS : 1];
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
     kreg[s] = as_bf16(ld16(p.k, tc * p.k_stride + hkv * D + 16 * s + 8 * h));
-    vreg[s] = as_bf16(ld16(p.v, tc * p.v_stride + hkv * D + 16 * s + 8 * h));
+    if constexpr (DK) vreg[s] = as_bf16(ld16(p.v, tc * p.v_stride + hkv * D + 16 * s + 8 * h));
   }
-  f32x16 acck[NDB], accv[NDB];
+  f32x16 acc[NDB];
 #pragma unroll
   for (int db = 0; db < NDB; ++db)
 #pragma unroll
-    for (int x = 0; x < 16; ++x) acck[db][x] = 0.f, accv[db][x] = 0.f;
+    for (int x = 0; x < 16; ++x) acc[db][x] = 0.f;
 
-  for (int i = j; i < qend; ++i) {
-    for (int g = 0; g < group; ++g) {
-      const int hq = hkv * group + g;
-      i32x4 qn[KS], don[KS], qtr[2][NDB], dotr[2][NDB];
-      f32x4 ls[2][2], dl[2][2];
-      const int64_t base = ((int64_t)hq * nt + i) * KS * 512 + lane * 8;
+  // step = (query tile, query head of this KV head), head fastest
+  const int steps = (qend_all - j0) * group;
+  i32x4 pf[PER];
+  float pf_ls = 0.f, pf_dl = 0.f;  // wave 0 brings the rows' lse (lanes 0-31) and delta (lanes 32-63)
+  auto fetch = [&](int step) {
+    step = min(step, steps - 1);
+    const int i = j0 + step / group, hq = hkv * group + step % group;
+    const int64_t at = ((int64_t)hq * nt + i) * KS * 512 + lane * 8;
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        qn[s] = ld16(p.qn, base + s * 512);
-        don[s] = ld16(p.don, base + s * 512);
-      }
+    for (int x = 0; x < PER; ++x) {
+      const int slot = wave * PER + x;
+      const void* image = slot < KS ? p.qn : !DK ? p.dor : slot < 2 * KS ? p.don : p.qr;
+      pf[x] = ld16(image, at + (slot % KS) * 512);
+    }
+    if (wave == 0) {
+      const int64_t row = hq * padded + 32 * i + n;
+      pf_ls = p.lse[row] * kLog2e;
+      if constexpr (DK) pf_dl = p.delta[row];
+    }
+  };
+  auto publish = [&](int buf) {
 #pragma unroll
-      for (int blk = 0; blk < 2; ++blk)
+    for (int x = 0; x < PER; ++x) lds[buf][wave * PER + x][lane] = pf[x];
+    if (wave == 0) {
+      if (h == 0) lds_ls[buf][n] = pf_ls;
+      if (DK && h == 1) lds_dl[buf][n] = pf_dl;
+    }
+  };
+
+  if (steps > 0) {
+    fetch(0);
+    publish(0);
+    __syncthreads();
+    for (int step = 0; step < steps; ++step) {
+      const int buf = step & 1;
+      const int i = j0 + step / group;
+      fetch(step + 1);
+      if (live && i >= j && i < qend) {
+        f32x16 sr, dp;
 #pragma unroll
-        for (int db = 0; db < NDB; ++db) {
-          qtr[blk][db] = ld16(p.qr, base + (blk * NDB + db) * 512);
-          dotr[blk][db] = ld16(p.dor, base + (blk * NDB + db) * 512);
+        for (int x = 0; x < 16; ++x) sr[x] = 0.f, dp[x] = 0.f;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+          sr = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(lds[buf][s][lane]), kreg[s], sr, 0, 0, 0);
+          if constexpr (DK) dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(lds[buf][KS + s][lane]), vreg[s], dp, 0, 0, 0);
+        }
+        bf16x8 pb[2];
+        const int row0 = 32 * i + 8 * h;
+        const bool masked = !(i > j && limmin >= 32 * i + 32);
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          // registers 4 q4 .. 4 q4 + 3 belong to rows 16 (q4 / 2) + 8 h + 4 (q4 % 2) + 0 .. 3 of the tile
+          const int at = 16 * (q4 >> 1) + 8 * h + 4 * (q4 & 1);
+          const f32x4 ls = *reinterpret_cast<const f32x4*>(&lds_ls[buf][at]);
+          f32x4 dl = {0.f, 0.f, 0.f, 0.f};
+          if constexpr (DK) dl = *reinterpret_cast<const f32x4*>(&lds_dl[buf][at]);
+#pragma unroll
+          for (int e4 = 0; e4 < 4; ++e4) {
+            const int x = 4 * q4 + e4;
+            const int qrow = row0 + 16 * (x >> 3) + (x & 7);
+            const bool ok = !masked || (t <= qrow && qrow < lim_t);
+            float e = ok ? fast_exp2(__builtin_fmaf(sr[x], sc, -ls[e4])) : 0.f;
+            if constexpr (DK) e *= dp[x] - dl[e4];
+            pb[x >> 3][x & 7] = (__bf16)e;
+          }
         }
 #pragma unroll
-      for (int blk = 0; blk < 2; ++blk)
+        for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          const int64_t at = hq * padded + 32 * i + 16 * blk + 8 * h + 4 * half;
-          ls[blk][half] = *reinterpret_cast<const f32x4*>(p.lse + at);
-          dl[blk][half] = *reinterpret_cast<const f32x4*>(p.delta + at);
-        }
-      f32x16 sr, dp;
-#pragma unroll
-      for (int x = 0; x < 16; ++x) sr[x] = 0.f, dp[x] = 0.f;
-#pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        sr = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(qn[s]), kreg[s], sr, 0, 0, 0);
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(don[s]), vreg[s], dp, 0, 0, 0);
+          for (int db = 0; db < NDB; ++db)
+            acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(lds[buf][SLOTS - KS + blk * NDB + db][lane]), pb[blk],
+                                                              acc[db], 0, 0, 0);
       }
-      bf16x8 pb[2], dsb[2];
-      const int row0 = 32 * i + 8 * h;
-#pragma unroll
-      for (int x = 0; x < 16; ++x) {
-        const int qrow = row0 + 16 * (x >> 3) + (x & 7);
-        const bool ok = t <= qrow && qrow < lim_t;
-        const float e = ok ? fast_exp2(__builtin_fmaf(sr[x], sc, -ls[x >> 3][(x >> 2) & 1][x & 3] * kLog2e)) : 0.f;
-        pb[x >> 3][x & 7] = (__bf16)e;
-        dsb[x >> 3][x & 7] = (__bf16)(e * (dp[x] - dl[x >> 3][(x >> 2) & 1][x & 3]));
-      }
-#pragma unroll
-      for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-        for (int db = 0; db < NDB; ++db) {
-          accv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(dotr[blk][db]), pb[blk], accv[db], 0, 0, 0);
-          acck[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(qtr[blk][db]), dsb[blk], acck[db], 0, 0, 0);
-        }
+      publish(buf ^ 1);
+      __syncthreads();
     }
   }
-  if (t < T) {
-    store_rows<D>(p.dk, (int64_t)t * p.dk_stride + hkv * D, h, acck, p.scale);
-    store_rows<D>(p.dv, (int64_t)t * p.dv_stride + hkv * D, h, accv, 1.f);
+  if (live && t < T) {
+    if constexpr (DK)
+      store_rows<D>(p.dk, (int64_t)t * p.dk_stride + hkv * D, h, acc, p.scale);
+    else
+      store_rows<D>(p.dv, (int64_t)t * p.dv_stride + hkv * D, h, acc, 1.f);
   }
 }
 
@@ -466,7 +544,10 @@ hipError_t launch_split_forward(const SplitParams& p, int head_dim, hipStream_t 
   return by_head_dim(head_dim, [&](auto d) {
     constexpr int D = decltype(d)::value;
     const unsigned grid = (unsigned)p.num_tiles * ((p.num_q_heads + kWaves - 1) / kWaves);
-    split_query_kernel<D, false><<<grid, kThreads, 0, stream>>>(p);
+    if ((p.num_q_heads / p.num_kv_heads) % kWaves == 0)
+      split_query_kernel<D, false, true><<<grid, kThreads, 0, stream>>>(p);
+    else
+      split_query_kernel<D, false, false><<<grid, kThreads, 0, stream>>>(p);
     return hipGetLastError();
   });
 }
@@ -484,9 +565,16 @@ hipError_t launch_split_backward(const SplitParams& p, int head_dim, hipStream_t
     const int per_block = kThreads / (D / 8);
     split_delta_kernel<D><<<(unsigned)((rows + per_block - 1) / per_block), kThreads, 0, stream>>>(p);
     if (hipError_t e = hipGetLastError()) return e;
-    split_query_kernel<D, true><<<(unsigned)nt * ((p.num_q_heads + kWaves - 1) / kWaves), kThreads, 0, stream>>>(p);
+    const unsigned qgrid = (unsigned)nt * ((p.num_q_heads + kWaves - 1) / kWaves);
+    if ((p.num_q_heads / p.num_kv_heads) % kWaves == 0)
+      split_query_kernel<D, true, true><<<qgrid, kThreads, 0, stream>>>(p);
+    else
+      split_query_kernel<D, true, false><<<qgrid, kThreads, 0, stream>>>(p);
     if (hipError_t e = hipGetLastError()) return e;
-    split_key_kernel<D><<<(unsigned)((nt + kWaves - 1) / kWaves) * p.num_kv_heads, kThreads, 0, stream>>>(p);
+    const unsigned kgrid = (unsigned)((nt + kWaves - 1) / kWaves) * p.num_kv_heads;
+    split_key_kernel<D, false><<<kgrid, kThreads, 0, stream>>>(p);
+    if (hipError_t e = hipGetLastError()) return e;
+    split_key_kernel<D, true><<<kgrid, kThreads, 0, stream>>>(p);
     return hipGetLastError();
   });
 }

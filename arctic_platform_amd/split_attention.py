@@ -67,9 +67,13 @@ class SplitLayout:
         o = 36 * self.num_tiles
         return self.host[o : o + self.num_tiles]
 
-    def orders(self):
+    def q_order(self):
         o = 37 * self.num_tiles
-        return self.host[o : o + self.num_tiles], self.host[o + self.num_tiles : o + 2 * self.num_tiles]
+        return self.host[o : o + self.num_tiles]
+
+    def kv_limmin(self):
+        o = 38 * self.num_tiles
+        return self.host[o : o + self.num_tiles]
 
     def scratch(self, plan, backward: bool) -> torch.Tensor:
         """Scratch of a call, kept with the layout: layers run one after the other on a stream."""

@@ -131,8 +131,8 @@ def test_layout_array_against_brute_force():
         for j, qend in enumerate(L.kv_qend()):
             need = np.nonzero(tiles[:, j])[0]
             assert need.min() >= j and need.max() < qend, (layout, j)
-        for order in L.orders():
-            assert sorted(order.tolist()) == list(range(nt))
+        assert sorted(L.q_order().tolist()) == list(range(nt))
+        assert (L.kv_limmin() == lim.reshape(nt, 32).min(axis=1)).all()
 
 
 def test_layout_walks_only_what_is_needed():
@@ -142,11 +142,13 @@ def test_layout_walks_only_what_is_needed():
     a0, a1, b0, _ = L.q_tiles()[L.num_tiles - 1]
     assert (a0, a1) == (0, 32) and b0 == (1024 + 7 * 512) // 32
     assert L.kv_qend()[0] == L.num_tiles and L.kv_qend()[40] == (1024 + 512) // 32
-    # heaviest work first
-    qo, ko = L.orders()
+    # within a group the longest walks first; groups one after the other
     cost = [(a1 - a0) + (i - b0 + 1) for i, (a0, a1, b0, _) in enumerate(L.q_tiles())]
-    assert [cost[i] for i in qo] == sorted(cost, reverse=True)
-    assert ko[0] == 0
+    assert [cost[i] for i in L.q_order()] == sorted(cost, reverse=True)
+    two = SplitLayout([(64, [64]), (128, [32])], device="cpu")
+    assert sorted(two.q_order()[:4].tolist()) == [0, 1, 2, 3] and two.q_order()[4] == 8
+    # a tile inside a prompt needs no element-wise test against later query tiles of the group
+    assert L.kv_limmin()[0] == 1024 + 8 * 512 and L.kv_limmin()[L.num_tiles - 1] == 1024 + 8 * 512
 
 
 def test_layout_arguments_are_checked():
