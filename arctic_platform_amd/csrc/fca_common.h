@@ -200,7 +200,7 @@ struct SplitParams {
 };
 // Offsets into the int32 layout array of a batch of `tiles` 32-token tiles.
 struct SplitLayout {
-  int64_t kv_lim, q_tiles, kv_qend, q_order, kv_limmin, total;
+  int64_t kv_lim, q_tiles, kv_qend, q_order, kv_limmin, kv_order, total;
 };
 __host__ __device__ inline SplitLayout make_split_layout(int64_t tiles) {
   SplitLayout L;
@@ -209,7 +209,8 @@ __host__ __device__ inline SplitLayout make_split_layout(int64_t tiles) {
   L.kv_qend = L.q_tiles + 4 * tiles;
   L.q_order = L.kv_qend + tiles;
   L.kv_limmin = L.q_order + tiles;
-  L.total = L.kv_limmin + tiles;
+  L.kv_order = L.kv_limmin + tiles;  // ceil(tiles / 4) entries used
+  L.total = L.kv_order + tiles;
   return L;
 }
 void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,

@@ -91,14 +91,21 @@ void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int3
     out[L.kv_limmin + i] = mn;
   }
   // Query tiles: group by group, so that the workgroups in flight read the same prompt, and
-  // the longest walks of a group first.  Key tiles are taken in packed order, four adjacent
-  // ones per workgroup: within a group that is the prompt's tiles, the heaviest, first.
+  // the longest walks of a group first.  Key tiles go four adjacent ones per workgroup; these
+  // quads differ in length fifty-fold (a prompt's walk the whole group, a response's only
+  // itself), so the longest go first.
   int32_t* qo = out + L.q_order;
   std::iota(qo, qo + tiles, 0);
   std::stable_sort(qo, qo + tiles, [&](int32_t a, int32_t b) {
     const int ga = group_of[32 * (int64_t)a], gb = group_of[32 * (int64_t)b];
     return ga != gb ? ga < gb : qcost[a] > qcost[b];
   });
+  const int64_t quads = (tiles + 3) / 4;
+  std::vector<int64_t> kcost(quads, 0);
+  for (int64_t i = 0; i < tiles; ++i) kcost[i / 4] = std::max<int64_t>(kcost[i / 4], out[L.kv_qend + i] - 4 * (i / 4));
+  int32_t* ko = out + L.kv_order;
+  std::iota(ko, ko + tiles, 0);
+  std::stable_sort(ko, ko + quads, [&](int32_t a, int32_t b) { return kcost[a] > kcost[b]; });
 
 }
 
@@ -386,18 +393,50 @@ __global__ __launch_bounds__(kThreads, SHARED ? 2 : 1) void split_query_kernel(S
 
 // ---- dk, dv: one wave per (key tile, KV head) --------------------------------------------------
 // A workgroup = four adjacent key tiles of one KV head.  Its waves need the same stream of
-// query-side operands, one step per (query tile, query head of the KV head): each wave
-// fetches a quarter of a step's slots one step ahead and the step is passed around through
-// LDS.  A wave computes only the steps inside its own tile's range of query tiles.  dV and dK
-// are two launches (DK = false / true): each keeps one set of accumulators, which leaves
-// room for two workgroups per CU, at the price of forming the probabilities twice.
+// query-side operands, one step per (query tile, query head of the KV head), and the stream
+// is far larger than the L2, so a step's loads often take a trip to memory, several times
+// the step's arithmetic.  The stream therefore goes through a ring of kRing LDS stages filled
+// by direct-to-LDS loads (no landing registers): every wave requests a quarter of the slots
+// of the step kRing - 1 ahead, waits only for its own requests of the step about to be used
+// (loads complete in order, so "all but the newest kRing - 2 stages"), and one barrier per
+// step both publishes that stage and frees the one just used.  A wave computes only the
+// steps inside its own tile's range of query tiles.  dV and dK are two launches
+// (DK = false / true): each keeps one set of accumulators, which leaves room for two
+// workgroups per CU, at the price of forming the probabilities twice.
 //   dV: slots Q rows [0, KS), dO transposed [KS, 2 KS):   P = exp(S - lse),  dVt += dOt . P
 //   dK: slots Q rows, dO rows, Q transposed:   dS = P (dO . V - delta),      dKt += Qt . dS
+constexpr int kRing = 3;
+
+// Direct-to-LDS loads: every lane's 16 (4) bytes land at lds_slot + lane * 16 (4).  Written as
+// assembly so that the compiler's wait insertion does not know of them: it would otherwise
+// drain every outstanding request before each LDS read, and the ring below lives on requests
+// that stay in flight across steps.  Loads the compiler does not know of can only make its
+// own waits more conservative.  M0 (the LDS base of such a load) is restored.
+__device__ inline unsigned lds_address(const void* p) {
+  return __builtin_amdgcn_readfirstlane((unsigned)(size_t)((__attribute__((address_space(3))) void*)(p)));
+}
+__device__ inline void load_to_lds16(const void* src, const void* lds_slot) {
+  unsigned saved;
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+               : "=&s"(saved)
+               : "v"(src), "s"(lds_address(lds_slot))
+               : "memory");
+}
+__device__ inline void load_to_lds4(const void* src, const void* lds_slot) {
+  unsigned saved;
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\tglobal_load_lds_dword %1, off\n\ts_mov_b32 m0, %0"
+               : "=&s"(saved)
+               : "v"(src), "s"(lds_address(lds_slot))
+               : "memory");
+}
+// s_waitcnt that constrains only the vector-memory counter (gfx9 encoding)
+#define FCA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0f70 | ((n) & 15) | (((n) >> 4) << 14))
+
 template <int D, bool DK>
 __global__ __launch_bounds__(kThreads, 2) void split_key_kernel(SplitParams p) {
   constexpr int KS = D / 16, NDB = D / 32, SLOTS = (DK ? 3 : 2) * KS, PER = SLOTS / kWaves;
-  __shared__ i32x4 lds[2][SLOTS][64];
-  __shared__ __attribute__((aligned(16))) float lds_ls[2][32], lds_dl[2][32];  // lse, delta of the step's rows
+  __shared__ i32x4 lds[kRing][SLOTS][64];
+  __shared__ __attribute__((aligned(16))) float lds_stat[kRing][64];  // lse of the step's 32 rows, then their delta
   const SplitLayout L = make_split_layout(p.num_tiles);
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
@@ -405,7 +444,7 @@ __global__ __launch_bounds__(kThreads, 2) void split_key_kernel(SplitParams p) {
   const int group = p.num_q_heads / p.num_kv_heads;
   const int T = p.num_tokens, nt = p.num_tiles;
   const int64_t padded = 32 * (int64_t)nt;
-  const int j0 = (blockIdx.x / p.num_kv_heads) * kWaves;
+  const int j0 = __builtin_amdgcn_readfirstlane(p.layout[L.kv_order + blockIdx.x / p.num_kv_heads]) * kWaves;
   const int j = min(j0 + wave, nt - 1);  // a wave past the last tile repeats it and stores nothing
   const bool live = j0 + wave < nt;
   const int qend = live ? __builtin_amdgcn_readfirstlane(p.layout[L.kv_qend + j]) : 0;
@@ -430,43 +469,49 @@ __global__ __launch_bounds__(kThreads, 2) void split_key_kernel(SplitParams p) {
 #pragma unroll
     for (int x = 0; x < 16; ++x) acc[db][x] = 0.f;
 
-  // step = (query tile, query head of this KV head), head fastest
+  // step = (query tile, query head of this KV head), head fastest, query tiles from the last
+  // one down (the workgroups of a prompt's key tiles all end at the group's last query tile)
   const int steps = (qend_all - j0) * group;
-  i32x4 pf[PER];
-  float pf_ls = 0.f, pf_dl = 0.f;  // wave 0 brings the rows' lse (lanes 0-31) and delta (lanes 32-63)
-  auto fetch = [&](int step) {
-    step = min(step, steps - 1);
-    const int i = j0 + step / group, hq = hkv * group + step % group;
-    const int64_t at = ((int64_t)hq * nt + i) * KS * 512 + lane * 8;
+  // Requests of one step: PER slots per wave, and from wave 0 the rows' lse (lanes 0-31) and
+  // delta (lanes 32-63).  Steps past the end repeat the last one, so the count never changes.
+  // (No division by the group size inside the loop: both walks are kept as counters.)
+  int req_i = qend_all - 1, req_g = 0, req_buf = 0;  // the next request: query tile, head of the group, ring stage
+  auto request = [&]() {
+    const int hq = hkv * group + req_g;
+    const int64_t at = ((int64_t)hq * nt + req_i) * KS * 512 + lane * 8;
 #pragma unroll
     for (int x = 0; x < PER; ++x) {
       const int slot = wave * PER + x;
       const void* image = slot < KS ? p.qn : !DK ? p.dor : slot < 2 * KS ? p.don : p.qr;
-      pf[x] = ld16(image, at + (slot % KS) * 512);
+      load_to_lds16(static_cast<const __bf16*>(image) + at + (slot % KS) * 512, &lds[req_buf][slot][0]);
     }
     if (wave == 0) {
-      const int64_t row = hq * padded + 32 * i + n;
-      pf_ls = p.lse[row] * kLog2e;
-      if constexpr (DK) pf_dl = p.delta[row];
+      const float* src = (DK && h == 1 ? p.delta : p.lse) + hq * padded + 32 * req_i + n;
+      load_to_lds4(src, &lds_stat[req_buf][0]);
     }
-  };
-  auto publish = [&](int buf) {
-#pragma unroll
-    for (int x = 0; x < PER; ++x) lds[buf][wave * PER + x][lane] = pf[x];
-    if (wave == 0) {
-      if (h == 0) lds_ls[buf][n] = pf_ls;
-      if (DK && h == 1) lds_dl[buf][n] = pf_dl;
-    }
+    req_buf = req_buf + 1 == kRing ? 0 : req_buf + 1;
+    // past the last step the last one is requested again
+    if (req_g + 1 < group)
+      ++req_g;
+    else if (req_i > j0)
+      req_g = 0, --req_i;
   };
 
+  // The loads above must have landed before the first request: a wait for them placed inside
+  // the loop would also wait, every step, for the requests the compiler does not know of.
+  FCA_WAIT_VMCNT(0);
   if (steps > 0) {
-    fetch(0);
-    publish(0);
-    __syncthreads();
+    for (int s = 0; s < kRing - 1; ++s) request();
+    int i = qend_all - 1, g = 0, buf = 0;
     for (int step = 0; step < steps; ++step) {
-      const int buf = step & 1;
-      const int i = j0 + step / group;
-      fetch(step + 1);
+      // this wave's requests of `step` have landed; after the barrier so have everyone's, and
+      // everyone has finished with the stage of the step before, which the next request refills
+      if (wave == 0)
+        FCA_WAIT_VMCNT((kRing - 2) * (PER + 1));
+      else
+        FCA_WAIT_VMCNT((kRing - 2) * PER);
+      __builtin_amdgcn_s_barrier();
+      request();
       if (live && i >= j && i < qend) {
         f32x16 sr, dp;
 #pragma unroll
@@ -483,15 +528,15 @@ __global__ __launch_bounds__(kThreads, 2) void split_key_kernel(SplitParams p) {
         for (int q4 = 0; q4 < 4; ++q4) {
           // registers 4 q4 .. 4 q4 + 3 belong to rows 16 (q4 / 2) + 8 h + 4 (q4 % 2) + 0 .. 3 of the tile
           const int at = 16 * (q4 >> 1) + 8 * h + 4 * (q4 & 1);
-          const f32x4 ls = *reinterpret_cast<const f32x4*>(&lds_ls[buf][at]);
+          const f32x4 ls = *reinterpret_cast<const f32x4*>(&lds_stat[buf][at]);
           f32x4 dl = {0.f, 0.f, 0.f, 0.f};
-          if constexpr (DK) dl = *reinterpret_cast<const f32x4*>(&lds_dl[buf][at]);
+          if constexpr (DK) dl = *reinterpret_cast<const f32x4*>(&lds_stat[buf][32 + at]);
 #pragma unroll
           for (int e4 = 0; e4 < 4; ++e4) {
             const int x = 4 * q4 + e4;
             const int qrow = row0 + 16 * (x >> 3) + (x & 7);
             const bool ok = !masked || (t <= qrow && qrow < lim_t);
-            float e = ok ? fast_exp2(__builtin_fmaf(sr[x], sc, -ls[e4])) : 0.f;
+            float e = ok ? fast_exp2(__builtin_fmaf(sr[x], sc, -ls[e4] * kLog2e)) : 0.f;
             if constexpr (DK) e *= dp[x] - dl[e4];
             pb[x >> 3][x & 7] = (__bf16)e;
           }
@@ -503,9 +548,10 @@ __global__ __launch_bounds__(kThreads, 2) void split_key_kernel(SplitParams p) {
             acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(lds[buf][SLOTS - KS + blk * NDB + db][lane]), pb[blk],
                                                               acc[db], 0, 0, 0);
       }
-      publish(buf ^ 1);
-      __syncthreads();
+      buf = buf + 1 == kRing ? 0 : buf + 1;
+      if (++g == group) g = 0, --i;
     }
+    FCA_WAIT_VMCNT(0);  // the repeated requests past the last step
   }
   if (live && t < T) {
     if constexpr (DK)

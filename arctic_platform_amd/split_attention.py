@@ -75,6 +75,10 @@ class SplitLayout:
         o = 38 * self.num_tiles
         return self.host[o : o + self.num_tiles]
 
+    def kv_order(self):
+        o = 39 * self.num_tiles
+        return self.host[o : o + (self.num_tiles + 3) // 4]
+
     def scratch(self, plan, backward: bool) -> torch.Tensor:
         """Scratch of a call, kept with the layout: layers run one after the other on a stream."""
         fwd, bwd = ctypes.c_size_t(), ctypes.c_size_t()

@@ -46,6 +46,7 @@ def parse_args():
     ap.add_argument("--calibrate", action="store_true", help="also run the library's plain copy kernel over 1 GiB (counter yardstick)")
     ap.add_argument("--query-runs", default="", metavar="NxL", help="instead of a decode configuration: N sequences that each bring a run of L query tokens (a prefill chunk), e.g. 4x2048")
     ap.add_argument("--context", type=int, default=0, help="tokens already cached in front of every query run")
+    ap.add_argument("--split-train", default="", metavar="GxS", help="instead of a decode configuration: the trainer's split attention, forward + backward, over G prompt groups of S samples each, e.g. 8x8")
     return ap.parse_args()
 
 
@@ -231,12 +232,115 @@ def main_query_runs(args):
     }))
 
 
+def main_split_train(args):
+    """The trainer's split attention over a deduplicated batch: G prompt groups, S samples
+    each, prompts U[1024, 4096], responses U[1, 1024] tokens, Qwen3-4B heads.  A step is one
+    layer's forward and backward.  Flops are the algorithmic ones of the visible (row, key)
+    pairs: 4 D Hq per pair forward, 10 D Hq backward."""
+    import random
+
+    import torch
+
+    from arctic_platform_amd.split_attention import SplitLayout, split_attention_backward, split_attention_forward
+    from oracle.split_attention import split_attention as oracle_split
+
+    ngroups, nsamples = (int(v) for v in args.split_train.lower().split("x"))
+    hq, hkv, d = 32, 8, 128
+    scale = d**-0.5
+    rng = random.Random(1)
+    groups = [(rng.randint(1024, 4096), [rng.randint(1, 1024) for _ in range(nsamples)]) for _ in range(ngroups)]
+
+    def pairs_of(gs):
+        return sum(p * (p + 1) // 2 + sum(r * p + r * (r + 1) // 2 for r in rs) for p, rs in gs)
+
+    def tensors(gs, seed):
+        gen = torch.Generator().manual_seed(seed)
+        t = sum(p + sum(rs) for p, rs in gs)
+        mk = lambda h: torch.randn(t, h, d, generator=gen).to(torch.bfloat16)
+        return mk(hq), mk(hkv), mk(hkv), mk(hq)
+
+    dev = torch.device("cuda:0")
+    layout = SplitLayout(groups, device=dev)
+    q, k, v, dout = (x.to(dev) for x in tensors(groups, 77))
+    steps, warmup = min(args.steps, 20), min(args.warmup, 3)
+
+    def fwd():
+        return split_attention_forward(q, k, v, layout, scale)
+
+    out, lse = fwd()
+
+    def bwd():
+        return split_attention_backward(dout, q, k, v, out, lse, layout, scale)
+
+    def timed(fn, n):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e3 / n
+
+    for _ in range(warmup):
+        fwd(), bwd()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fwd(), bwd()
+    torch.cuda.synchronize()
+    step_us = (time.perf_counter() - t0) / steps * 1e6
+    fwd_us, bwd_us = timed(fwd, steps), timed(bwd, steps)
+    pairs = pairs_of(groups)
+    flops_f, flops_b = 4 * d * hq * pairs, 10 * d * hq * pairs
+
+    # CPU baseline and check: the smallest group with two of its samples, through the oracle (fp32, autograd)
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    torch.set_num_threads(cores)
+    sp, srs = min(groups, key=lambda g: g[0] + sum(g[1]))
+    sample = [(sp, srs[:2])]
+    sq, sk, sv, sdo = tensors(sample, 78)
+    sl = SplitLayout(sample, device=dev)
+    g_out, g_lse = split_attention_forward(sq.to(dev), sk.to(dev), sv.to(dev), sl, scale)
+    g_grads = split_attention_backward(sdo.to(dev), sq.to(dev), sk.to(dev), sv.to(dev), g_out, g_lse, sl, scale)
+    t0 = time.perf_counter()
+    rq, rk, rv = (x.float().requires_grad_() for x in (sq, sk, sv))
+    r_out, _ = oracle_split(rq, rk, rv, sample, scale, dtype=torch.float32)
+    r_out.backward(sdo.float())
+    cpu_s = time.perf_counter() - t0
+    errs = {}
+    for name, got, ref, rel in (("out", g_out, r_out.detach(), 0.0), ("dq", g_grads[0], rq.grad, 1e-2), ("dk", g_grads[1], rk.grad, 1e-2), ("dv", g_grads[2], rv.grad, 1e-2)):
+        diff = (got.cpu().float() - ref).abs()
+        bound = (2e-2 if rel == 0.0 else rel * float(ref.abs().max())) + 2e-2 * ref.abs()
+        assert bool((diff <= bound).all()), f"{name} differs from the oracle: max |err| {float(diff.max())}"
+        errs[name] = float(diff.max())
+    scale_up = pairs / pairs_of(sample)
+    tfl = lambda f, us: round(f / us / 1e6, 1)
+    print(json.dumps({
+        "metric": "split attention (ZoRRo Train) forward + backward µs/step, Qwen3-4B heads",
+        "value": round(step_us, 1), "unit": "us/step", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(step_us / 1e3, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 MFMA / f32 accumulate", "data": "synthetic",
+        "config": {"workload": f"{ngroups} prompt groups x {nsamples} samples, prompt U[1024,4096], response U[1,1024], Hq {hq} / Hkv {hkv} / D {d}, bf16, deduplicated order",
+                   "tokens": layout.num_tokens, "visible_pairs": pairs, "flops_forward": flops_f, "flops_backward": flops_b},
+        "roofline": {"kernel": "split_query_kernel + split_key_kernel (forward, dq, dv, dk)", "bound": "mfma",
+                     "achieved": tfl(flops_f + flops_b, fwd_us + bwd_us), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round((flops_f + flops_b) / (fwd_us + bwd_us) / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "forward_tflops": tfl(flops_f, fwd_us), "backward_tflops": tfl(flops_b, bwd_us)},
+        "breakdown_us": {"forward": round(fwd_us, 1), "backward": round(bwd_us, 1)},
+        "cpu_baseline": {"value": cpu_s * scale_up * 1e6, "unit": "us/step", "cores": cores, "kind": "port",
+                         "sample": f"one group (prompt {sp}, responses {srs[:2]}) through the fp32 oracle with autograd on torch-CPU, {cpu_s:.2f} s measured, scaled by visible pairs x{scale_up:.1f}"},
+        "max_abs_err_vs_oracle_sample": errs,
+    }))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path uses no collectives and the boxes have one GPU; run with --gpus 1")
     if args.query_runs:
         return main_query_runs(args)
+    if args.split_train:
+        return main_split_train(args)
     import torch
 
     from arctic_platform_amd import ops

@@ -133,6 +133,7 @@ def test_layout_array_against_brute_force():
             assert need.min() >= j and need.max() < qend, (layout, j)
         assert sorted(L.q_order().tolist()) == list(range(nt))
         assert (L.kv_limmin() == lim.reshape(nt, 32).min(axis=1)).all()
+        assert sorted(L.kv_order().tolist()) == list(range((nt + 3) // 4))
 
 
 def test_layout_walks_only_what_is_needed():
@@ -147,6 +148,8 @@ def test_layout_walks_only_what_is_needed():
     assert [cost[i] for i in L.q_order()] == sorted(cost, reverse=True)
     two = SplitLayout([(64, [64]), (128, [32])], device="cpu")
     assert sorted(two.q_order()[:4].tolist()) == [0, 1, 2, 3] and two.q_order()[4] == 8
+    # key tiles go four to a workgroup, the longest walks first: the prompt's, front to back
+    assert L.kv_order()[:8].tolist() == list(range(8))
     # a tile inside a prompt needs no element-wise test against later query tiles of the group
     assert L.kv_limmin()[0] == 1024 + 8 * 512 and L.kv_limmin()[L.num_tiles - 1] == 1024 + 8 * 512
 
