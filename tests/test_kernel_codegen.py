@@ -70,3 +70,29 @@ def test_tile_loop_of_the_32_row_kernel_keeps_a_tile_in_flight(hipcc, tmp_path):
         assert len(re.findall(r"global_load_dwordx4", block)) == loads_per_tile, header
         seen += 1
     assert seen >= 1
+
+
+def test_split_attention_kernels_use_no_scratch_and_keep_their_ring_in_flight(hipcc, tmp_path):
+    """The dK and dV kernels of the trainer's split attention stream their operands through
+    a ring of LDS stages filled by direct-to-LDS loads that stay in flight across steps.  The
+    only waits on the vector-memory counter the kernels may hold are the ones written in the
+    source: one for everything before the loop, the counted pair at the top of a step (wave 0
+    requests one load more per step than the others), one for everything after the loop.  A
+    wait the compiler adds inside the loop would drain the ring every step."""
+    out = tmp_path / "split.s"
+    res = subprocess.run(
+        [hipcc, *FLAGS, "-S", "-Rpass-analysis=kernel-resource-usage", os.path.join(CSRC, "fca_split.hip"), "-o", str(out)],
+        capture_output=True, text=True, cwd=CSRC,
+    )
+    assert res.returncode == 0, res.stderr[-2000:]
+    sizes = re.findall(r"ScratchSize \[bytes/lane\]: (\d+)", res.stderr)
+    assert len(sizes) >= 16 and set(sizes) == {"0"}, sizes
+    kernels = {k: v for k, v in _functions(out.read_text()).items() if "split_key_kernel" in k}
+    assert len(kernels) == 4, sorted(kernels)
+    for name, body in kernels.items():
+        head_dim = 128 if "ILi128E" in name else 64
+        slots = (3 if "Lb1E" in name else 2) * head_dim // 16
+        per_wave = slots // 4
+        waits = [int(n) for n in re.findall(r"s_waitcnt[^\n]*vmcnt\((\d+)\)", body)]
+        assert waits == [0, per_wave, per_wave + 1, 0], (name, waits)
+        assert body.count("global_load_lds_dwordx4") == 3 * per_wave, name  # two stages ahead of the loop, one inside
