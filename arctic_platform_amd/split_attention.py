@@ -55,6 +55,24 @@ class SplitLayout:
     def from_group_token_layout(cls, layout, device="cuda"):
         return cls([(g["prompt_tokens"], g["response_tokens"]) for g in layout], device=device)
 
+    @classmethod
+    def from_reconstruction_info(cls, reconstruction_info, device="cuda"):
+        """From the trainer's ``reconstruction_info`` itself: ``prompt_groups`` (lists of sample
+        indices) and ``segment_info`` (dicts with ``group_idx``, ``type`` "prompt" / "response",
+        ``original_idx`` and ``num_valid_tokens``, or ``start`` / ``end`` before unpadding), read the
+        way ``ZoRRoTrain.get_group_token_layout`` reads them (zorro_train.py:2409-2436): the
+        prompt's count from the group's first sample, one response count per sample in group order."""
+
+        def valid(seg):
+            return int(seg.get("num_valid_tokens", seg["end"] - seg["start"]))
+
+        segs = {(s["group_idx"], s["type"], s["original_idx"]): s for s in reconstruction_info["segment_info"]}
+        groups = []
+        for g, members in enumerate(reconstruction_info["prompt_groups"]):
+            prompt = valid(segs[(g, "prompt", members[0])])
+            groups.append((prompt, [valid(segs[(g, "response", m)]) for m in members]))
+        return cls(groups, device=device)
+
     # views of the layout array (tests, inspection)
     def kv_lim(self):
         return self.host[: 32 * self.num_tiles]

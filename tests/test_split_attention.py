@@ -154,6 +154,33 @@ def test_layout_walks_only_what_is_needed():
     assert L.kv_limmin()[0] == 1024 + 8 * 512 and L.kv_limmin()[L.num_tiles - 1] == 1024 + 8 * 512
 
 
+def test_layout_from_the_trainers_reconstruction_info():
+    """segment_info as ZoRRoTrain._dedup_input_ids leaves it (zorro_train.py:311-356: the prompt
+    segment recorded once per sample of the group, then one response segment per sample) and as
+    unpad_deduplicated_batch updates it (:646-672, num_valid_tokens).  Groups as in the
+    reference's own grouping test (tests/zorro_train/test_dedup.py:76-88): [[0, 2], [1, 3]]."""
+    groups = [[0, 2], [1, 3]]
+    prompt_len, response_len = 6, 4
+    valid = {("prompt", 0): 5, ("prompt", 2): 5, ("prompt", 1): 6, ("prompt", 3): 6,
+             ("response", 0): 4, ("response", 2): 1, ("response", 1): 0, ("response", 3): 3}
+    segment_info, pos = [], 0
+    for g, members in enumerate(groups):
+        for m in members:
+            segment_info.append(dict(start=pos, end=pos + prompt_len, original_idx=m, type="prompt", group_idx=g))
+        pos += prompt_len
+        for m in members:
+            segment_info.append(dict(start=pos, end=pos + response_len, original_idx=m, type="response", group_idx=g))
+            pos += response_len
+    info = dict(prompt_groups=groups, segment_info=segment_info)
+    padded = SplitLayout.from_reconstruction_info(info, device="cpu")
+    assert padded.groups == [(6, [4, 4]), (6, [4, 4])] and padded.num_tokens == 28
+    for seg in segment_info:
+        seg["num_valid_tokens"] = valid[(seg["type"], seg["original_idx"])]
+    unpadded = SplitLayout.from_reconstruction_info(info, device="cpu")
+    assert unpadded.groups == [(5, [4, 1]), (6, [0, 3])] and unpadded.num_tokens == 19
+    assert unpadded.kv_lim()[:19].tolist() == [10] * 5 + [9] * 4 + [10] + [19] * 6 + [19] * 3
+
+
 def test_layout_arguments_are_checked():
     lib = _lib.load_library()
     prompt = np.asarray([4], dtype=np.int32)
