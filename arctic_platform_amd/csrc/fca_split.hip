@@ -283,13 +283,13 @@ __global__ __launch_bounds__(kThreads, SHARED ? 2 : 1) void split_query_kernel(S
           for (int e = 0; e < 4; ++e) ok[8 * blk + 4 * half + e] = tok0 + 16 * blk + 4 * half + e <= r && lim[e] > r;
         }
     }
+    // a hidden score becomes -inf, whose exponential is 0 (no branch around the exponentials)
+    if (masked) {
+#pragma unroll
+      for (int x = 0; x < 16; ++x) sr[x] = ok[x] ? sr[x] : -INFINITY;
+    }
     bf16x8 pb[2];
     if constexpr (!BWD) {
-      if (masked) {
-#pragma unroll
-        for (int x = 0; x < 16; ++x)
-          if (!ok[x]) sr[x] = -INFINITY;
-      }
       float mx = sr[0];
 #pragma unroll
       for (int x = 1; x < 16; ++x) mx = fmaxf(mx, sr[x]);
@@ -323,7 +323,7 @@ __global__ __launch_bounds__(kThreads, SHARED ? 2 : 1) void split_query_kernel(S
       for (int s = 0; s < KS; ++s) dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16(get(KS + s)), doreg[s], dp, 0, 0, 0);
 #pragma unroll
       for (int x = 0; x < 16; ++x) {
-        const float e = ok[x] ? fast_exp2(__builtin_fmaf(sr[x], sc, -lse2)) : 0.f;
+        const float e = fast_exp2(__builtin_fmaf(sr[x], sc, -lse2));
         pb[x >> 3][x & 7] = (__bf16)(e * (dp[x] - delta));
       }
     }
@@ -523,7 +523,14 @@ __global__ __launch_bounds__(kThreads, 2) void split_key_kernel(SplitParams p) {
         }
         bf16x8 pb[2];
         const int row0 = 32 * i + 8 * h;
-        const bool masked = !(i > j && limmin >= 32 * i + 32);
+        // a hidden score becomes -inf, whose exponential is 0 (no branch around the exponentials)
+        if (!(i > j && limmin >= 32 * i + 32)) {
+#pragma unroll
+          for (int x = 0; x < 16; ++x) {
+            const int qrow = row0 + 16 * (x >> 3) + (x & 7);
+            sr[x] = (t <= qrow && qrow < lim_t) ? sr[x] : -INFINITY;
+          }
+        }
 #pragma unroll
         for (int q4 = 0; q4 < 4; ++q4) {
           // registers 4 q4 .. 4 q4 + 3 belong to rows 16 (q4 / 2) + 8 h + 4 (q4 % 2) + 0 .. 3 of the tile
@@ -534,9 +541,7 @@ __global__ __launch_bounds__(kThreads, 2) void split_key_kernel(SplitParams p) {
 #pragma unroll
           for (int e4 = 0; e4 < 4; ++e4) {
             const int x = 4 * q4 + e4;
-            const int qrow = row0 + 16 * (x >> 3) + (x & 7);
-            const bool ok = !masked || (t <= qrow && qrow < lim_t);
-            float e = ok ? fast_exp2(__builtin_fmaf(sr[x], sc, -ls[e4] * kLog2e)) : 0.f;
+            float e = fast_exp2(__builtin_fmaf(sr[x], sc, -ls[e4] * kLog2e));
             if constexpr (DK) e *= dp[x] - dl[e4];
             pb[x >> 3][x & 7] = (__bf16)e;
           }
