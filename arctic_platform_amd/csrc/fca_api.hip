@@ -381,7 +381,7 @@ int fca_split_workspace_bytes(const fca_split_plan* plan, size_t* forward_bytes,
   if (int rc = check_split(plan)) return rc;
   const SplitScratch s = split_scratch(plan);
   if (forward_bytes) *forward_bytes = 2 * s.kv_tiles;
-  if (backward_bytes) *backward_bytes = 3 * s.kv_tiles + 4 * s.q_tiles + s.delta;
+  if (backward_bytes) *backward_bytes = 3 * s.kv_tiles + 4 * s.q_tiles + 2 * s.delta;
   return FCA_OK;
 }
 
@@ -450,6 +450,7 @@ int fca_split_attention_backward(const fca_split_plan* plan, const void* q_dev, 
   p.don = ws + 3 * s.kv_tiles + 2 * s.q_tiles;
   p.dor = ws + 3 * s.kv_tiles + 3 * s.q_tiles;
   p.delta = reinterpret_cast<float*>(ws + 3 * s.kv_tiles + 4 * s.q_tiles);
+  p.lse2 = reinterpret_cast<float*>(ws + 3 * s.kv_tiles + 4 * s.q_tiles + s.delta);
   p.lse = const_cast<float*>(lse_dev);
   p.dq = dq_dev, p.dk = dk_dev, p.dv = dv_dev;
   p.dq_stride = dq_stride, p.dk_stride = dk_stride, p.dv_stride = dv_stride;

@@ -192,6 +192,7 @@ struct SplitParams {
   void* out;
   float* lse;    // [Hq][tiles * 32] natural log
   float* delta;  // [Hq][tiles * 32] rowsum(dout * out)
+  float* lse2;   // [Hq][tiles * 32] lse * log2(e), made by the backward's first pass
   void *dq, *dk, *dv;
   int64_t dq_stride, dk_stride, dv_stride;
   const int32_t* layout;

@@ -174,7 +174,8 @@ __global__ __launch_bounds__(kThreads) void split_images_kernel(const __bf16* x,
   }
 }
 
-// delta[h][t] = sum_d dout[t, h, d] * out[t, h, d]; zero past the last token.
+// delta[h][t] = sum_d dout[t, h, d] * out[t, h, d]; zero past the last token.  Also leaves the
+// log-sum-exp in log2 units.
 template <int D>
 __global__ __launch_bounds__(kThreads) void split_delta_kernel(SplitParams p) {
   constexpr int LPR = D / 8;
@@ -193,7 +194,10 @@ __global__ __launch_bounds__(kThreads) void split_delta_kernel(SplitParams p) {
   }
 #pragma unroll
   for (int w = 1; w < LPR; w *= 2) sum += __shfl_xor(sum, w);
-  if (threadIdx.x % LPR == 0) p.delta[hh * padded + t] = sum;
+  if (threadIdx.x % LPR == 0) {
+    p.delta[hh * padded + t] = sum;
+    p.lse2[hh * padded + t] = p.lse[hh * padded + t] * kLog2e;  // the form the dk and dv kernels subtract
+  }
 }
 
 // ---- forward and dq: one wave per (query tile, query head) -----------------------------------
@@ -415,18 +419,18 @@ constexpr int kRing = 3;
 __device__ inline unsigned lds_address(const void* p) {
   return __builtin_amdgcn_readfirstlane((unsigned)(size_t)((__attribute__((address_space(3))) void*)(p)));
 }
-__device__ inline void load_to_lds16(const void* src, const void* lds_slot) {
+__device__ inline void load_to_lds16(const void* src, unsigned lds_slot) {
   unsigned saved;
   asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
                : "=&s"(saved)
-               : "v"(src), "s"(lds_address(lds_slot))
+               : "v"(src), "s"(lds_slot)
                : "memory");
 }
-__device__ inline void load_to_lds4(const void* src, const void* lds_slot) {
+__device__ inline void load_to_lds4(const void* src, unsigned lds_slot) {
   unsigned saved;
   asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\tglobal_load_lds_dword %1, off\n\ts_mov_b32 m0, %0"
                : "=&s"(saved)
-               : "v"(src), "s"(lds_address(lds_slot))
+               : "v"(src), "s"(lds_slot)
                : "memory");
 }
 // s_waitcnt that constrains only the vector-memory counter (gfx9 encoding)
@@ -436,7 +440,7 @@ template <int D, bool DK>
 __global__ __launch_bounds__(kThreads, 2) void split_key_kernel(SplitParams p) {
   constexpr int KS = D / 16, NDB = D / 32, SLOTS = (DK ? 3 : 2) * KS, PER = SLOTS / kWaves;
   __shared__ i32x4 lds[kRing][SLOTS][64];
-  __shared__ __attribute__((aligned(16))) float lds_stat[kRing][64];  // lse of the step's 32 rows, then their delta
+  __shared__ __attribute__((aligned(16))) float lds_stat[kRing][64];  // lse (in log2 units) of the step's 32 rows, then their delta
   const SplitLayout L = make_split_layout(p.num_tiles);
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
@@ -476,19 +480,24 @@ __global__ __launch_bounds__(kThreads, 2) void split_key_kernel(SplitParams p) {
   // delta (lanes 32-63).  Steps past the end repeat the last one, so the count never changes.
   // (No division by the group size inside the loop: both walks are kept as counters.)
   int req_i = qend_all - 1, req_g = 0, req_buf = 0;  // the next request: query tile, head of the group, ring stage
+  // what does not change from step to step: where this wave's slots start in their images
+  // (per lane) and in a ring stage (LDS byte addresses)
+  const __bf16* slot_src[PER];
+#pragma unroll
+  for (int x = 0; x < PER; ++x) {
+    const int slot = wave * PER + x;
+    const void* image = slot < KS ? p.qn : !DK ? p.dor : slot < 2 * KS ? p.don : p.qr;
+    slot_src[x] = static_cast<const __bf16*>(image) + (slot % KS) * 512 + lane * 8;
+  }
+  const float* stat_src = (DK && h == 1 ? p.delta : p.lse2) + n;
+  const unsigned slot_lds = lds_address(&lds[0][0][0]) + wave * PER * 1024;
+  const unsigned stat_lds = lds_address(&lds_stat[0][0]);
   auto request = [&]() {
     const int hq = hkv * group + req_g;
-    const int64_t at = ((int64_t)hq * nt + req_i) * KS * 512 + lane * 8;
+    const int64_t at = ((int64_t)hq * nt + req_i) * KS * 512;
 #pragma unroll
-    for (int x = 0; x < PER; ++x) {
-      const int slot = wave * PER + x;
-      const void* image = slot < KS ? p.qn : !DK ? p.dor : slot < 2 * KS ? p.don : p.qr;
-      load_to_lds16(static_cast<const __bf16*>(image) + at + (slot % KS) * 512, &lds[req_buf][slot][0]);
-    }
-    if (wave == 0) {
-      const float* src = (DK && h == 1 ? p.delta : p.lse) + hq * padded + 32 * req_i + n;
-      load_to_lds4(src, &lds_stat[req_buf][0]);
-    }
+    for (int x = 0; x < PER; ++x) load_to_lds16(slot_src[x] + at, slot_lds + (req_buf * SLOTS + x) * 1024);
+    if (wave == 0) load_to_lds4(stat_src + hq * padded + 32 * req_i, stat_lds + req_buf * 256);
     req_buf = req_buf + 1 == kRing ? 0 : req_buf + 1;
     // past the last step the last one is requested again
     if (req_g + 1 < group)
@@ -541,7 +550,7 @@ __global__ __launch_bounds__(kThreads, 2) void split_key_kernel(SplitParams p) {
 #pragma unroll
           for (int e4 = 0; e4 < 4; ++e4) {
             const int x = 4 * q4 + e4;
-            float e = fast_exp2(__builtin_fmaf(sr[x], sc, -ls[e4] * kLog2e));
+            float e = fast_exp2(__builtin_fmaf(sr[x], sc, -ls[e4]));
             if constexpr (DK) e *= dp[x] - dl[e4];
             pb[x >> 3][x & 7] = (__bf16)e;
           }

@@ -198,7 +198,7 @@ def test_layout_arguments_are_checked():
     fwd, bwd = ctypes.c_size_t(), ctypes.c_size_t()
     assert lib.fca_split_workspace_bytes(ctypes.byref(plan), ctypes.byref(fwd), ctypes.byref(bwd)) == 0
     kv, qq = 128 * 2 * 128 * 2, 128 * 8 * 128 * 2
-    assert fwd.value == 2 * kv and bwd.value == 3 * kv + 4 * qq + 128 * 8 * 4
+    assert fwd.value == 2 * kv and bwd.value == 3 * kv + 4 * qq + 2 * 128 * 8 * 4
     with pytest.raises(RuntimeError, match="GPU"):
         L = SplitLayout([(4, [3, 2])], device="cpu")
         x = torch.zeros(9, 4, 64, dtype=torch.bfloat16)
@@ -208,9 +208,10 @@ def test_layout_arguments_are_checked():
 # ---- the kernels (GPU) ----------------------------------------------------------------------
 def _close(name, got, ref, scale_tol):
     """bf16 results of fp32 accumulations over bf16 probabilities: 2e-2 relative plus
-    ``scale_tol`` of the tensor's largest magnitude."""
+    ``scale_tol`` of the tensor's largest magnitude (plus 1e-5: a gradient that is exactly zero,
+    such as dq of a row that sees a single key, comes out as rounding noise of that size)."""
     got, ref = got.detach().cpu().double(), ref.detach().double()
-    bound = scale_tol * ref.abs().max() + 2e-2 * ref.abs()
+    bound = scale_tol * ref.abs().max() + 2e-2 * ref.abs() + 1e-5
     err = (got - ref).abs()
     assert bool((err <= bound).all()), f"{name}: max |err| {err.max():.4g}, largest reference {ref.abs().max():.4g}"
 
@@ -260,6 +261,26 @@ def test_random_layouts_match_the_oracle():
         print("layout", layout, flush=True)
         _run_case(layout, 4, 2, rng.choice([64, 128]), seed=done)
         done += 1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize(
+    "layout",
+    [
+        [(1, [0])],  # one token in all
+        [(0, [1])],
+        [(31, [1])],  # exactly one tile
+        [(32, [1])],  # one token into the second tile
+        [(0, [2, 0, 3])],  # no prompt at all
+        [(3, []), (2, [4])],  # a group without samples
+        [(127, [1]), (1, [127])],
+    ],
+)
+@pytest.mark.parametrize("heads", [(4, 1, 128), (6, 2, 64)])
+def test_smallest_and_odd_layouts(layout, heads):
+    """Fewer steps than ring stages, a single tile, empty prompts and responses; four query
+    heads per KV head take the LDS-shared kernels, three the per-wave ones."""
+    _run_case(layout, *heads, seed=33)
 
 
 @pytest.mark.gpu
