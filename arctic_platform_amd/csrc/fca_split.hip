@@ -11,20 +11,23 @@
 // one int per key.  Work is cut into tiles of 32 consecutive tokens of the packed order; a
 // tile may straddle segments, the per-element test above sorts that out.
 //
-// Kernels, one wave per (tile, head), no workgroup barrier, operands straight from global
-// memory into MFMA operand registers (mfma_f32_32x32x16_bf16):
+// Kernels (mfma_f32_32x32x16_bf16, one wave per tile and head, four waves to a workgroup
+// that share one stream of operands through LDS):
 //   forward    per query tile, over the key tiles it can see (two ranges: the prompt's
 //              tiles, then from the tile its own segment starts in up to its own):
 //              St[tok x row] = K . Qt, online softmax per lane, Ot[d x row] += Vt . Pt
 //   dq         per query tile, the same walk: Pt from the saved log-sum-exp,
 //              dPt = V . dOt, dSt = Pt (dPt - delta), dQt[d x row] += Kt . dSt
-//   dk, dv     per key tile, over the query tiles that can see it (one range) and the query
+//   dv, dk     per key tile, over the query tiles that can see it (one range) and the query
 //              heads of its KV head: S[row x tok] = Q . Kt', P, dP = dO . Vt',
-//              dVt[d x tok] += dOt . P, dKt[d x tok] += Qt . dS; a prompt's dK and dV
-//              collect every sample of the group in registers and are written once
-// The second product of each chain contracts over tokens (or rows), which a [T, H, D]
-// tensor does not hold contiguously: a transposing pass first writes the tiles
-// [H][tile][D][32] of V (forward), of K, Q and dO (backward), zero past the last token.
+//              dVt[d x tok] += dOt . P, dKt[d x tok] += Qt . dS (two launches); a prompt's
+//              dK and dV collect every sample of the group in registers and are written once
+// A [T, H, D] tensor holds neither operand of these products contiguously for a 64-lane load:
+// the first product of a chain wants 32 rows x 32 bytes per instruction, the second one
+// contracts over tokens (or rows), which lie a row stride apart.  A first pass therefore
+// writes every 32-token tile in operand order, 1 KB per operand slot ("images": rows as the
+// first product takes them, and transposed as the second takes them; zero past the last
+// token), and every operand load of the kernels is one contiguous kilobyte per wave.
 // The first product feeds its rows in the order that makes its output registers the B
 // operand of the second, so probabilities never leave registers.
 #include <algorithm>
