@@ -338,11 +338,15 @@ int check_rows(const char* name, const void* ptr, int64_t stride, int heads, int
   return FCA_OK;
 }
 struct SplitScratch {
-  size_t kv_tiles, q_tiles, delta;  // bytes
+  size_t kv_tiles, q_tiles, delta, head_slices;  // bytes
 };
 SplitScratch split_scratch(const fca_split_plan* p) {
-  const size_t padded = 32 * (size_t)((p->num_tokens + 31) / 32);
-  return {padded * p->num_kv_heads * p->head_dim * 2, padded * p->num_q_heads * p->head_dim * 2, padded * p->num_q_heads * 4};
+  const size_t tiles = (p->num_tokens + 31) / 32, padded = 32 * tiles;
+  const size_t slices = fca::split_by_head(tiles, p->num_q_heads, p->num_kv_heads)
+                            ? (size_t)(p->num_q_heads / p->num_kv_heads) * p->num_tokens * p->num_kv_heads * p->head_dim * 4
+                            : 0;
+  return {padded * p->num_kv_heads * p->head_dim * 2, padded * p->num_q_heads * p->head_dim * 2, padded * p->num_q_heads * 4,
+          (slices + 15) / 16 * 16};
 }
 }  // namespace
 
@@ -381,7 +385,7 @@ int fca_split_workspace_bytes(const fca_split_plan* plan, size_t* forward_bytes,
   if (int rc = check_split(plan)) return rc;
   const SplitScratch s = split_scratch(plan);
   if (forward_bytes) *forward_bytes = 2 * s.kv_tiles;
-  if (backward_bytes) *backward_bytes = 3 * s.kv_tiles + 4 * s.q_tiles + 2 * s.delta;
+  if (backward_bytes) *backward_bytes = 3 * s.kv_tiles + 4 * s.q_tiles + 2 * s.delta + 2 * s.head_slices;
   return FCA_OK;
 }
 
@@ -451,6 +455,9 @@ int fca_split_attention_backward(const fca_split_plan* plan, const void* q_dev, 
   p.dor = ws + 3 * s.kv_tiles + 3 * s.q_tiles;
   p.delta = reinterpret_cast<float*>(ws + 3 * s.kv_tiles + 4 * s.q_tiles);
   p.lse2 = reinterpret_cast<float*>(ws + 3 * s.kv_tiles + 4 * s.q_tiles + s.delta);
+  p.head_split = s.head_slices > 0;
+  p.dk_part = reinterpret_cast<float*>(ws + 3 * s.kv_tiles + 4 * s.q_tiles + 2 * s.delta);
+  p.dv_part = reinterpret_cast<float*>(ws + 3 * s.kv_tiles + 4 * s.q_tiles + 2 * s.delta + s.head_slices);
   p.lse = const_cast<float*>(lse_dev);
   p.dq = dq_dev, p.dk = dk_dev, p.dv = dv_dev;
   p.dq_stride = dq_stride, p.dk_stride = dk_stride, p.dv_stride = dv_stride;

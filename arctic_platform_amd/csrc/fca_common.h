@@ -198,7 +198,16 @@ struct SplitParams {
   const int32_t* layout;
   int32_t num_tokens, num_tiles, num_q_heads, num_kv_heads;
   float scale;
+  // small batches: dk and dv are formed per query head (fp32 slices [Hq / Hkv][T][Hkv][D]) and summed afterwards
+  int32_t head_split;
+  float *dk_part, *dv_part;
 };
+// A batch with few key tiles leaves most of the chip idle behind its longest walks (a prompt's
+// key tiles are seen by the whole group): then every query head of a KV head gets a workgroup
+// of its own, which shortens the longest walk by Hq / Hkv.
+inline bool split_by_head(int64_t tiles, int num_q_heads, int num_kv_heads) {
+  return num_q_heads > num_kv_heads && ((tiles + 3) / 4) * num_kv_heads < 1024;
+}
 // Offsets into the int32 layout array of a batch of `tiles` 32-token tiles.
 struct SplitLayout {
   int64_t kv_lim, q_tiles, kv_qend, q_order, kv_limmin, kv_order, total;

@@ -448,10 +448,14 @@ __global__ __launch_bounds__(kThreads, 2) void split_key_kernel(SplitParams p) {
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
   const int hkv = blockIdx.x % p.num_kv_heads;
-  const int group = p.num_q_heads / p.num_kv_heads;
+  const int ratio = p.num_q_heads / p.num_kv_heads;
+  int rest = blockIdx.x / p.num_kv_heads;
+  // the query heads this workgroup walks: all of the KV head, or (head_split) one of them
+  int hq0 = hkv * ratio, group = ratio;
+  if (p.head_split) hq0 += rest % ratio, rest /= ratio, group = 1;
   const int T = p.num_tokens, nt = p.num_tiles;
   const int64_t padded = 32 * (int64_t)nt;
-  const int j0 = __builtin_amdgcn_readfirstlane(p.layout[L.kv_order + blockIdx.x / p.num_kv_heads]) * kWaves;
+  const int j0 = __builtin_amdgcn_readfirstlane(p.layout[L.kv_order + rest]) * kWaves;
   const int j = min(j0 + wave, nt - 1);  // a wave past the last tile repeats it and stores nothing
   const bool live = j0 + wave < nt;
   const int qend = live ? __builtin_amdgcn_readfirstlane(p.layout[L.kv_qend + j]) : 0;
@@ -496,7 +500,7 @@ __global__ __launch_bounds__(kThreads, 2) void split_key_kernel(SplitParams p) {
   const unsigned slot_lds = lds_address(&lds[0][0][0]) + wave * PER * 1024;
   const unsigned stat_lds = lds_address(&lds_stat[0][0]);
   auto request = [&]() {
-    const int hq = hkv * group + req_g;
+    const int hq = hq0 + req_g;
     const int64_t at = ((int64_t)hq * nt + req_i) * KS * 512;
 #pragma unroll
     for (int x = 0; x < PER; ++x) load_to_lds16(slot_src[x] + at, slot_lds + (req_buf * SLOTS + x) * 1024);
@@ -571,11 +575,40 @@ __global__ __launch_bounds__(kThreads, 2) void split_key_kernel(SplitParams p) {
     FCA_WAIT_VMCNT(0);  // the repeated requests past the last step
   }
   if (live && t < T) {
-    if constexpr (DK)
-      store_rows<D>(p.dk, (int64_t)t * p.dk_stride + hkv * D, h, acc, p.scale);
-    else
-      store_rows<D>(p.dv, (int64_t)t * p.dv_stride + hkv * D, h, acc, 1.f);
+    const float mul = DK ? p.scale : 1.f;
+    if (p.head_split) {
+      float* part = (DK ? p.dk_part : p.dv_part) + (((int64_t)(hq0 - hkv * ratio) * T + t) * p.num_kv_heads + hkv) * D + 4 * h;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          f32x4 w;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[e] = acc[db][4 * q4 + e] * mul;
+          *reinterpret_cast<f32x4*>(part + 32 * db + 8 * q4) = w;
+        }
+    } else if constexpr (DK) {
+      store_rows<D>(p.dk, (int64_t)t * p.dk_stride + hkv * D, h, acc, mul);
+    } else {
+      store_rows<D>(p.dv, (int64_t)t * p.dv_stride + hkv * D, h, acc, mul);
+    }
   }
+}
+
+// out[t][c] = sum over the slices of part[slice][t][c], c over the Hkv * D values of a token.
+__global__ __launch_bounds__(kThreads) void split_reduce_kernel(const float* part, int slices, int64_t tokens, int row,
+                                                               __bf16* out, int64_t out_stride) {
+  const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const int per_row = row / 4;
+  if (idx >= tokens * per_row) return;
+  const int64_t t = idx / per_row;
+  const int c = (int)(idx % per_row) * 4;
+  f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < slices; ++s) sum += *reinterpret_cast<const f32x4*>(part + ((int64_t)s * tokens + t) * row + c);
+  bf16x4 w;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) w[e] = (__bf16)sum[e];
+  *reinterpret_cast<bf16x4*>(out + t * out_stride + c) = w;
 }
 
 template <typename F>
@@ -634,10 +667,19 @@ hipError_t launch_split_backward(const SplitParams& p, int head_dim, hipStream_t
     else
       split_query_kernel<D, true, false><<<qgrid, kThreads, 0, stream>>>(p);
     if (hipError_t e = hipGetLastError()) return e;
-    const unsigned kgrid = (unsigned)((nt + kWaves - 1) / kWaves) * p.num_kv_heads;
+    const int ratio = p.num_q_heads / p.num_kv_heads;
+    const unsigned kgrid = (unsigned)((nt + kWaves - 1) / kWaves) * p.num_kv_heads * (p.head_split ? ratio : 1);
     split_key_kernel<D, false><<<kgrid, kThreads, 0, stream>>>(p);
     if (hipError_t e = hipGetLastError()) return e;
     split_key_kernel<D, true><<<kgrid, kThreads, 0, stream>>>(p);
+    if (hipError_t e = hipGetLastError()) return e;
+    if (p.head_split) {
+      const int row = p.num_kv_heads * D;
+      const unsigned rgrid = (unsigned)(((int64_t)T * (row / 4) + kThreads - 1) / kThreads);
+      split_reduce_kernel<<<rgrid, kThreads, 0, stream>>>(p.dv_part, ratio, T, row, static_cast<__bf16*>(p.dv), p.dv_stride);
+      if (hipError_t e = hipGetLastError()) return e;
+      split_reduce_kernel<<<rgrid, kThreads, 0, stream>>>(p.dk_part, ratio, T, row, static_cast<__bf16*>(p.dk), p.dk_stride);
+    }
     return hipGetLastError();
   });
 }

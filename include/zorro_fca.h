@@ -254,7 +254,8 @@ int fca_split_layout_ints(int32_t num_tokens, int64_t* num_ints);
  * device once per batch; every layer's forward and backward reads it. */
 int fca_split_layout_build(int32_t num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,
                            const int32_t* response_tokens, int32_t num_tokens, int32_t* layout_host);
-/* Bytes of device scratch a forward / a backward call needs (transposed operand tiles). */
+/* Bytes of device scratch a forward / a backward call needs: operand tiles in MFMA order,
+ * per-row sums, and for small batches fp32 slices of dk and dv per query head of a KV head. */
 int fca_split_workspace_bytes(const fca_split_plan* plan, size_t* forward_bytes, size_t* backward_bytes);
 /* out [T, Hq, D] bf16; lse fp32 [Hq][32 * ceil(T / 32)], natural log (kept for backward). */
 int fca_split_attention_forward(const fca_split_plan* plan, const void* q_dev, int64_t q_stride, const void* k_dev,

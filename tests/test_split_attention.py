@@ -198,7 +198,11 @@ def test_layout_arguments_are_checked():
     fwd, bwd = ctypes.c_size_t(), ctypes.c_size_t()
     assert lib.fca_split_workspace_bytes(ctypes.byref(plan), ctypes.byref(fwd), ctypes.byref(bwd)) == 0
     kv, qq = 128 * 2 * 128 * 2, 128 * 8 * 128 * 2
-    assert fwd.value == 2 * kv and bwd.value == 3 * kv + 4 * qq + 2 * 128 * 8 * 4
+    # a batch this small forms dk and dv per query head: two sets of fp32 slices [Hq / Hkv][T][Hkv][D] on top
+    assert fwd.value == 2 * kv and bwd.value == 3 * kv + 4 * qq + 2 * 128 * 8 * 4 + 2 * 4 * 100 * 2 * 128 * 4
+    big = _lib.FcaSplitPlan(32 * 1024, 32, 8, 128)
+    assert lib.fca_split_workspace_bytes(ctypes.byref(big), ctypes.byref(fwd), ctypes.byref(bwd)) == 0
+    assert bwd.value == 3 * (32768 * 8 * 256) + 4 * (32768 * 32 * 256) + 2 * 32768 * 32 * 4
     with pytest.raises(RuntimeError, match="GPU"):
         L = SplitLayout([(4, [3, 2])], device="cpu")
         x = torch.zeros(9, 4, 64, dtype=torch.bfloat16)
