@@ -220,8 +220,9 @@ def _close(name, got, ref, scale_tol):
     assert bool((err <= bound).all()), f"{name}: max |err| {err.max():.4g}, largest reference {ref.abs().max():.4g}"
 
 
-def _run_case(layout, hq, hkv, d, seed, strided=False):
+def _run_case(layout, hq, hkv, d, seed, strided=False, q_gain=1.0):
     q, k, v = _inputs(layout, hq, hkv, d, seed, torch.bfloat16)
+    q = (q.float() * q_gain).bfloat16()
     t = q.shape[0]
     scale = d**-0.5
     L = SplitLayout(layout)
@@ -285,6 +286,14 @@ def test_smallest_and_odd_layouts(layout, heads):
     """Fewer steps than ring stages, a single tile, empty prompts and responses; four query
     heads per KV head take the LDS-shared kernels, three the per-wave ones."""
     _run_case(layout, *heads, seed=33)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("q_gain", [8.0, 1 / 64])
+def test_sharp_and_flat_score_distributions(q_gain):
+    """Scores of magnitude ~100 (softmax close to one-hot, row maxima that jump from tile to
+    tile, so the running reference of the forward is rescaled often) and scores near zero."""
+    _run_case([(150, [90, 40]), (64, [33])], 8, 2, 128, seed=17, q_gain=q_gain)
 
 
 @pytest.mark.gpu
