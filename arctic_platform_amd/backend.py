@@ -37,6 +37,7 @@ from .config import ModelConfig, validate_fca_support
 from .forest import ForestMetadata, build_forest_metadata, rows_from_query_runs
 from .kv_layout import BLOCK_SIZE, kv_cache_shape
 from .ops import forest_cascade_decode
+from .split_attention import SplitLayout, split_attention_forward
 
 
 @dataclasses.dataclass
@@ -50,13 +51,20 @@ class CommonAttentionMetadata:
     num_reqs: int
     max_query_len: int
     num_actual_tokens: int | None = None
+    # host copies, as the engine keeps them; with them a step of fresh prompts only is recognised
+    # without a device round trip
+    query_start_loc_cpu: torch.Tensor | None = None
+    seq_lens_cpu: torch.Tensor | None = None
 
 
 @dataclasses.dataclass
 class ForestCascadeMetadata:
-    forest: ForestMetadata
+    forest: ForestMetadata | None
     slot_mapping: torch.Tensor
     num_decode_tokens: int
+    # set instead of ``forest`` for a step of fresh prompts only: causal attention of every
+    # prompt over itself, straight from the step's own K and V
+    fresh_prefill: SplitLayout | None = None
 
 
 def parse_forest_cascade_configs(value) -> dict:
@@ -112,6 +120,10 @@ class ForestCascadeMetadataBuilder:
     (a new request with a cached prompt) is picked up."""
 
     MAX_KEPT_WORKSPACES = 16
+    # a step of fresh prompts with at least this many tokens runs on the trainer's split
+    # attention kernels (each prompt a group of its own): operands shared through LDS, about
+    # twice the rate of the query-run path, which stays for everything that reads the cache
+    FRESH_PREFILL_MIN_TOKENS = 256
 
     def __init__(self, num_q_heads, num_kv_heads, head_dim, device="cuda", forest_cascade_attn_configs=None):
         cfg = parse_forest_cascade_configs(forest_cascade_attn_configs)
@@ -150,6 +162,17 @@ class ForestCascadeMetadataBuilder:
         bt, sl = m.block_table_tensor[: m.num_reqs], m.seq_lens[: m.num_reqs]
         num_tokens = m.num_reqs
         row_table = row_group = None
+        if m.max_query_len > 1 and m.query_start_loc_cpu is not None and m.seq_lens_cpu is not None and self.enabled:
+            q_lens = (m.query_start_loc_cpu[1 : m.num_reqs + 1] - m.query_start_loc_cpu[: m.num_reqs]).tolist()
+            if q_lens == m.seq_lens_cpu[: m.num_reqs].tolist() and sum(q_lens) >= self.FRESH_PREFILL_MIN_TOKENS:
+                key = ("fresh", tuple(q_lens))
+                if key not in self._workspaces:
+                    self._keep(key, SplitLayout([(0, [n]) for n in q_lens], device=self.device))
+                self._workspaces.move_to_end(key)
+                total = sum(q_lens)
+                return ForestCascadeMetadata(
+                    forest=None, slot_mapping=m.slot_mapping[:total], num_decode_tokens=total, fresh_prefill=self._workspaces[key]
+                )
         if m.max_query_len > 1:
             # one row per query token: the row of its sequence, cut off behind the token itself;
             # the tokens of a run that fall into one cache block form a tile
@@ -240,6 +263,14 @@ class ForestCascadeAttentionImpl:
             )
         if output is None:
             output = torch.empty_like(query)
+        if attn_metadata.fresh_prefill is not None:
+            if key is None:
+                raise ValueError("a step of fresh prompts needs the step's key and value")
+            split_attention_forward(
+                q, key[:t].view(t, self.num_kv_heads, self.head_size), value[:t].view(t, self.num_kv_heads, self.head_size),
+                attn_metadata.fresh_prefill, self.scale, out=output[:t].view(t, self.num_heads, self.head_size),
+            )
+            return output
         forest_cascade_decode(
             q, kv_cache, attn_metadata.forest, self.scale, k_scale, v_scale,
             out=output[:t].view(t, self.num_heads, self.head_size), return_lse=False,

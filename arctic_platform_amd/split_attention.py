@@ -122,15 +122,18 @@ def _plan(q, k):
     return _lib.FcaSplitPlan(q.shape[0], q.shape[1], k.shape[1], q.shape[2])
 
 
-def split_attention_forward(q, k, v, layout: SplitLayout, scale: float):
+def split_attention_forward(q, k, v, layout: SplitLayout, scale: float, out=None):
     """q ``[T, Hq, D]``, k, v ``[T, Hkv, D]`` bf16 in deduplicated order.  Returns
     ``(out [T, Hq, D] bf16, lse fp32 [Hq, 32 * ceil(T / 32)])``; ``lse[:, :T]`` is the
-    natural-log log-sum-exp of every row's scores."""
+    natural-log log-sum-exp of every row's scores.  ``out`` may be given to write into."""
     t = layout.num_tokens
     for name, x in (("q", q), ("k", k), ("v", v)):
         _check_rows(name, x, t)
     plan = _plan(q, k)
-    out = torch.empty((t, q.shape[1], q.shape[2]), dtype=torch.bfloat16, device=q.device)
+    if out is None:
+        out = torch.empty((t, q.shape[1], q.shape[2]), dtype=torch.bfloat16, device=q.device)
+    else:
+        _check_rows("out", out, t)
     lse = torch.empty((q.shape[1], 32 * layout.num_tiles), dtype=torch.float32, device=q.device)
     if t == 0:
         return out, lse

@@ -199,6 +199,27 @@ def main_query_runs(args):
     torch.cuda.synchronize()
     step_us = (time.perf_counter() - t0) / steps * 1e6
     kern = sum(a.elapsed_time(b) * 1e3 for a, b in events) / len(events)
+    fresh = None
+    if ctx == 0:
+        # what the adapter does for a step of fresh prompts: attention straight from the step's
+        # K and V on the split-attention kernels, each prompt a group of its own (timing only:
+        # random K and V of the same shape; checked against the oracle in the tests)
+        from arctic_platform_amd.split_attention import SplitLayout, split_attention_forward
+
+        layout = SplitLayout([(0, [ql])] * nseq, device=dev)
+        kp, vp = (torch.randn(rows_total, hkv, d, generator=gen).to(torch.bfloat16).to(dev) for _ in range(2))
+        out3 = torch.empty(rows_total, hq, d, dtype=torch.bfloat16, device=dev)
+        for _ in range(3):
+            split_attention_forward(q, kp, vp, layout, scale, out=out3)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(20):
+            split_attention_forward(q, kp, vp, layout, scale, out=out3)
+        b.record()
+        torch.cuda.synchronize()
+        fresh_us = a.elapsed_time(b) * 1e3 / 20
+        fresh = {"us_per_step": round(fresh_us, 2), "tflops": round(4.0 * d * hq * float(lens.double().sum()) / fresh_us / 1e6, 1),
+                 "what": "split_attention_forward on the step's packed K and V (operand images included)"}
     flops = 4.0 * d * hq * float(lens.double().sum())
 
     # CPU baseline and a parity spot check on a sample of rows
@@ -226,6 +247,7 @@ def main_query_runs(args):
                      "achieved": round(flops / kern / 1e6, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / kern / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None, "launches_timed": len(events)},
         "breakdown_us": {"attention_kernel": round(kern, 2)},
+        "fresh_prompts_on_split_kernels": fresh,
         "cpu_baseline": {"value": cpu_s * scale_up * 1e6, "unit": "us/step", "cores": cores, "kind": "port",
                          "sample": f"{len(sample)} of {rows_total} query rows, flat fp32 attention on torch-CPU, {cpu_s:.2f} s measured, scaled by gathered tokens x{scale_up:.1f}"},
         "max_abs_err_vs_oracle_sample": err,

@@ -168,3 +168,53 @@ def test_several_query_tokens_per_sequence(gpu, q_lens_kind):
     tiled = {r for n in nodes if n["causal"] for r in n["members"]}
     assert all(leaf["tokens"] == 0 for r, leaf in enumerate(meta.forest.leaves()) if r in tiled)
 
+
+
+@pytest.mark.gpu
+def test_fresh_prompts_take_the_split_attention_kernels(gpu):
+    """A step that brings only fresh prompts (no cached context) and host copies of the
+    lengths: the adapter attends straight from the step's K and V on the split-attention
+    kernels, still fills the cache, and a following decode step reads it.  With a cached
+    context, or without the host copies, the same call goes the query-run way."""
+    from arctic_platform_amd.kv_layout import kv_cache_shape
+    from oracle.attention import flat_decode_attention
+
+    hq, hkv, d = 8, 2, 128
+    scale = d**-0.5
+    lens = [300, 77, 512]
+    T, S = sum(lens), len(lens)
+    gen = torch.Generator().manual_seed(9)
+    max_blocks = 40
+    table = torch.randperm(S * max_blocks, generator=gen).to(torch.int32).view(S, max_blocks).to(gpu)
+    cache = torch.zeros(kv_cache_shape(S * max_blocks, 16, hkv, d), dtype=torch.bfloat16, device=gpu)
+    q, k, v = (torch.randn(T, h * d, generator=gen).to(torch.bfloat16).to(gpu) for h in (hq, hkv, hkv))
+    starts = torch.tensor([0] + lens).cumsum(0)
+    seq = torch.repeat_interleave(torch.arange(S), torch.tensor(lens))
+    pos = torch.cat([torch.arange(n) for n in lens])
+    slots = (table.cpu().long()[seq, pos // 16] * 16 + pos % 16).to(gpu)
+    builder = ForestCascadeAttentionBackend.get_builder_cls()(hq, hkv, d, device=gpu)
+    impl = ForestCascadeAttentionBackend.get_impl_cls()(hq, d, scale, hkv)
+    layer = types.SimpleNamespace(k_scale=None, v_scale=None)
+    common = CommonAttentionMetadata(
+        query_start_loc=starts.to(torch.int32).to(gpu), seq_lens=torch.tensor(lens, dtype=torch.int32, device=gpu),
+        block_table_tensor=table, slot_mapping=slots, num_reqs=S, max_query_len=max(lens), num_actual_tokens=T,
+        query_start_loc_cpu=starts.to(torch.int32), seq_lens_cpu=torch.tensor(lens, dtype=torch.int32),
+    )
+    meta = builder.build(0, common)
+    assert meta.fresh_prefill is not None and meta.forest is None
+    out = impl.forward(layer, q, k, v, cache, meta)
+    # the oracle reads the cache the call has just filled: one row per token, cut off behind it
+    ref, _ = flat_decode_attention(
+        q.view(T, hq, d).cpu(), cache.cpu(), table.cpu()[seq], (pos + 1).to(torch.int32), scale, dtype=torch.float32
+    )
+    torch.testing.assert_close(out.view(T, hq, d).cpu().float(), ref, rtol=2e-2, atol=2e-2)
+    assert builder.build(0, common).fresh_prefill is meta.fresh_prefill  # the layout is kept with the workspaces
+    # the query-run way on the same step (no host copies): same rows
+    import dataclasses
+    slow = builder.build(0, dataclasses.replace(common, query_start_loc_cpu=None, seq_lens_cpu=None))
+    assert slow.fresh_prefill is None
+    out2 = impl.forward(layer, q, None, None, cache, slow)
+    torch.testing.assert_close(out2.view(T, hq, d).cpu().float(), ref, rtol=2e-2, atol=2e-2)
+    # a cached context in front of one sequence: not fresh any more
+    longer = dataclasses.replace(common, seq_lens_cpu=torch.tensor([lens[0] + 16, lens[1], lens[2]], dtype=torch.int32))
+    assert builder.build(0, longer).fresh_prefill is None
