@@ -190,3 +190,17 @@ class _SplitAttention(torch.autograd.Function):
 def split_attention(q, k, v, layout: SplitLayout, scale: float):
     """Differentiable split attention: ``out [T, Hq, D]`` in deduplicated order."""
     return _SplitAttention.apply(q, k, v, layout, scale)
+
+
+def split_attention_padded(q, k, v, valid, layout: SplitLayout, scale: float):
+    """The same attention for a deduplicated batch that still carries its padding (the
+    trainer's padded variant, qwen_attention_patcher.py:881-1040, which masks the padding inside
+    its two attention calls): ``q``, ``k``, ``v`` are ``[T_padded, H, D]``, ``valid`` a bool
+    ``[T_padded]`` (the deduplicated attention mask, zorro_train.py:359-372), ``layout`` counts
+    the valid tokens.  The valid rows are gathered, attended, and scattered back; padding rows
+    of the result are zero and receive no gradient.  Differentiable."""
+    index = torch.nonzero(valid, as_tuple=False).squeeze(-1)
+    if index.numel() != layout.num_tokens:
+        raise ValueError(f"{index.numel()} valid tokens, the layout counts {layout.num_tokens}")
+    out = split_attention(q.index_select(0, index), k.index_select(0, index), v.index_select(0, index), layout, scale)
+    return torch.zeros_like(q).index_copy(0, index, out)

@@ -14,6 +14,7 @@ from arctic_platform_amd import _lib
 from arctic_platform_amd.split_attention import (
     SplitLayout,
     split_attention,
+    split_attention_padded,
     split_attention_backward,
     split_attention_forward,
 )
@@ -363,3 +364,37 @@ def test_large_batch_is_invariant_under_group_order():
     _close("out", forward_order[0][sl], ro, 2e-2 / max(1.0, float(ro.detach().abs().max())))
     for name, got, ref in zip(("dq", "dk", "dv"), forward_order[1:], (q64.grad, k64.grad, v64.grad)):
         _close(name, got[sl], ref, 1e-2)
+
+
+@pytest.mark.gpu
+def test_padded_batch_is_gathered_attended_and_scattered():
+    """Prompts padded on the left, responses on the right, as the trainer's padded batches are:
+    the valid rows get the oracle's values, padding rows zeros, and gradients reach only valid
+    rows."""
+    layout = [(5, [4, 1]), (6, [0, 3])]
+    prompt_len, response_len = 6, 4
+    valid = []
+    for p, rs in layout:
+        valid += [False] * (prompt_len - p) + [True] * p
+        for r in rs:
+            valid += [True] * r + [False] * (response_len - r)
+    valid = torch.tensor(valid)
+    tp, t = valid.numel(), int(valid.sum())
+    assert t == total_tokens(layout)
+    gen = torch.Generator().manual_seed(6)
+    hq, hkv, d = 4, 2, 64
+    qp, kp, vp = (torch.randn(tp, h, d, generator=gen).bfloat16() for h in (hq, hkv, hkv))
+    qd, kd, vd = (x.cuda().requires_grad_() for x in (qp, kp, vp))
+    out = split_attention_padded(qd, kd, vd, valid.cuda(), SplitLayout(layout), d**-0.5)
+    w = torch.randn(tp, hq, d, generator=gen).bfloat16()
+    (out.float() * w.cuda().float()).sum().backward()
+    q64, k64, v64 = (x[valid].double().requires_grad_() for x in (qp, kp, vp))
+    ro, _ = oracle_split(q64, k64, v64, layout, d**-0.5)
+    (ro * w[valid].double()).sum().backward()
+    assert float(out.detach()[~valid.cuda()].abs().max()) == 0.0
+    _close("out", out[valid.cuda()], ro, 2e-2)
+    for name, got, ref in (("dq", qd.grad, q64.grad), ("dk", kd.grad, k64.grad), ("dv", vd.grad, v64.grad)):
+        assert float(got[~valid.cuda()].abs().max()) == 0.0, name
+        _close(name, got[valid.cuda()], ref, 1e-2)
+    with pytest.raises(ValueError, match="valid tokens"):
+        split_attention_padded(qd, kd, vd, torch.ones(tp, dtype=torch.bool, device="cuda"), SplitLayout(layout), 0.125)
