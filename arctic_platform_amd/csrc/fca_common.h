@@ -225,8 +225,6 @@ __host__ __device__ inline SplitLayout make_split_layout(int64_t tiles) {
 }
 void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,
                         const int32_t* response_tokens, int64_t tiles, int32_t* out);
-hipError_t launch_split_images(const void* x, int64_t stride, int heads, int head_dim, int num_tokens, int tiles,
-                               void* rows_image, void* transposed_image, hipStream_t stream);
 hipError_t launch_split_forward(const SplitParams& p, int head_dim, hipStream_t stream);
 hipError_t launch_split_backward(const SplitParams& p, int head_dim, hipStream_t stream);
 

@@ -149,9 +149,13 @@ __device__ inline void store_rows(void* dst, int64_t row_elem, int h, const f32x
 //   rows image        slot s, lane (m, h):        x[fed_row(m)][16 s + 8 h .. + 7]
 //   transposed image  slot (blk, db), lane (m, h): x[16 blk + 8 h + i][32 db + m], i = 0 .. 7
 // Rows past the last token are zero.
+// With `other` (the images of dO are being made and `other` is O): also leaves, per row,
+// delta = sum_d x * other and the log-sum-exp in log2 units, which the dk and dv kernels subtract.
 template <int D>
 __global__ __launch_bounds__(kThreads) void split_images_kernel(const __bf16* x, int64_t stride, int T, int nt,
-                                                               __bf16* rows_image, __bf16* transposed_image) {
+                                                               __bf16* rows_image, __bf16* transposed_image,
+                                                               const __bf16* other, int64_t other_stride, const float* lse,
+                                                               float* delta, float* lse2) {
   __shared__ __attribute__((aligned(16))) __bf16 tile[32][D + 8];
   const int j = blockIdx.x, hh = blockIdx.y;
   for (int p = threadIdx.x; p < 32 * D / 8; p += kThreads) {
@@ -160,6 +164,21 @@ __global__ __launch_bounds__(kThreads) void split_images_kernel(const __bf16* x,
     i32x4 w = {0, 0, 0, 0};
     if (t < T) w = ld16(x, t * stride + hh * D + c);
     *reinterpret_cast<i32x4*>(&tile[tk][c]) = w;
+    if (other) {  // the D / 8 pieces of a row sit in adjacent lanes
+      float sum = 0.f;
+      if (t < T) {
+        const bf16x8 a = as_bf16(w), b = as_bf16(ld16(other, t * other_stride + hh * D + c));
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum += (float)a[i] * (float)b[i];
+      }
+#pragma unroll
+      for (int m = 1; m < D / 8; m *= 2) sum += __shfl_xor(sum, m);
+      if (c == 0) {
+        const int64_t at = (int64_t)hh * 32 * nt + t;
+        delta[at] = sum;
+        lse2[at] = lse[at] * kLog2e;
+      }
+    }
   }
   __syncthreads();
   const int64_t base = ((int64_t)hh * nt + j) * (D / 16) * 512;
@@ -174,32 +193,6 @@ __global__ __launch_bounds__(kThreads) void split_images_kernel(const __bf16* x,
       for (int i = 0; i < 8; ++i) e[i] = tile[16 * blk + 8 * h + i][32 * db + m];
       *reinterpret_cast<bf16x8*>(transposed_image + base + p * 8) = e;
     }
-  }
-}
-
-// delta[h][t] = sum_d dout[t, h, d] * out[t, h, d]; zero past the last token.  Also leaves the
-// log-sum-exp in log2 units.
-template <int D>
-__global__ __launch_bounds__(kThreads) void split_delta_kernel(SplitParams p) {
-  constexpr int LPR = D / 8;
-  const int64_t padded = 32 * (int64_t)p.num_tiles;
-  const int64_t idx = (int64_t)blockIdx.x * (kThreads / LPR) + threadIdx.x / LPR;
-  if (idx >= padded * p.num_q_heads) return;  // whole lane groups leave together
-  const int64_t t = idx % padded;
-  const int hh = (int)(idx / padded);
-  const int c = (threadIdx.x % LPR) * 8;
-  float sum = 0.f;
-  if (t < p.num_tokens) {
-    const bf16x8 a = as_bf16(ld16(p.dout, t * p.do_stride + hh * D + c));
-    const bf16x8 b = as_bf16(ld16(p.out_in, t * p.o_stride + hh * D + c));
-#pragma unroll
-    for (int i = 0; i < 8; ++i) sum += (float)a[i] * (float)b[i];
-  }
-#pragma unroll
-  for (int w = 1; w < LPR; w *= 2) sum += __shfl_xor(sum, w);
-  if (threadIdx.x % LPR == 0) {
-    p.delta[hh * padded + t] = sum;
-    p.lse2[hh * padded + t] = p.lse[hh * padded + t] * kLog2e;  // the form the dk and dv kernels subtract
   }
 }
 
@@ -620,23 +613,24 @@ hipError_t by_head_dim(int head_dim, F&& f) {
 
 }  // namespace
 
-hipError_t launch_split_images(const void* x, int64_t stride, int heads, int head_dim, int num_tokens, int tiles,
-                               void* rows_image, void* transposed_image, hipStream_t stream) {
+namespace {
+hipError_t images(const void* x, int64_t stride, int heads, int head_dim, int num_tokens, int tiles, void* rows_image,
+                  void* transposed_image, hipStream_t stream, const void* other = nullptr, int64_t other_stride = 0,
+                  const float* lse = nullptr, float* delta = nullptr, float* lse2 = nullptr) {
   return by_head_dim(head_dim, [&](auto d) {
     constexpr int D = decltype(d)::value;
-    split_images_kernel<D><<<dim3(tiles, heads), kThreads, 0, stream>>>(static_cast<const __bf16*>(x), stride, num_tokens, tiles,
-                                                                       static_cast<__bf16*>(rows_image),
-                                                                       static_cast<__bf16*>(transposed_image));
+    split_images_kernel<D><<<dim3(tiles, heads), kThreads, 0, stream>>>(
+        static_cast<const __bf16*>(x), stride, num_tokens, tiles, static_cast<__bf16*>(rows_image),
+        static_cast<__bf16*>(transposed_image), static_cast<const __bf16*>(other), other_stride, lse, delta, lse2);
     return hipGetLastError();
   });
 }
+}  // namespace
 
 hipError_t launch_split_forward(const SplitParams& p, int head_dim, hipStream_t stream) {
   const int T = p.num_tokens, nt = p.num_tiles;
-  if (hipError_t e = launch_split_images(p.k, p.k_stride, p.num_kv_heads, head_dim, T, nt, const_cast<void*>(p.kn), nullptr, stream))
-    return e;
-  if (hipError_t e = launch_split_images(p.v, p.v_stride, p.num_kv_heads, head_dim, T, nt, nullptr, const_cast<void*>(p.vr), stream))
-    return e;
+  if (hipError_t e = images(p.k, p.k_stride, p.num_kv_heads, head_dim, T, nt, const_cast<void*>(p.kn), nullptr, stream)) return e;
+  if (hipError_t e = images(p.v, p.v_stride, p.num_kv_heads, head_dim, T, nt, nullptr, const_cast<void*>(p.vr), stream)) return e;
   return by_head_dim(head_dim, [&](auto d) {
     constexpr int D = decltype(d)::value;
     const unsigned grid = (unsigned)p.num_tiles * ((p.num_q_heads + kWaves - 1) / kWaves);
@@ -651,16 +645,15 @@ hipError_t launch_split_forward(const SplitParams& p, int head_dim, hipStream_t 
 hipError_t launch_split_backward(const SplitParams& p, int head_dim, hipStream_t stream) {
   const int T = p.num_tokens, nt = p.num_tiles;
   auto V = [](const void* x) { return const_cast<void*>(x); };
-  if (hipError_t e = launch_split_images(p.k, p.k_stride, p.num_kv_heads, head_dim, T, nt, V(p.kn), V(p.kr), stream)) return e;
-  if (hipError_t e = launch_split_images(p.v, p.v_stride, p.num_kv_heads, head_dim, T, nt, V(p.vn), nullptr, stream)) return e;
-  if (hipError_t e = launch_split_images(p.q, p.q_stride, p.num_q_heads, head_dim, T, nt, V(p.qn), V(p.qr), stream)) return e;
-  if (hipError_t e = launch_split_images(p.dout, p.do_stride, p.num_q_heads, head_dim, T, nt, V(p.don), V(p.dor), stream)) return e;
+  if (hipError_t e = images(p.k, p.k_stride, p.num_kv_heads, head_dim, T, nt, V(p.kn), V(p.kr), stream)) return e;
+  if (hipError_t e = images(p.v, p.v_stride, p.num_kv_heads, head_dim, T, nt, V(p.vn), nullptr, stream)) return e;
+  if (hipError_t e = images(p.q, p.q_stride, p.num_q_heads, head_dim, T, nt, V(p.qn), V(p.qr), stream)) return e;
+  // the pass over dO also makes the per-row sums of dO * O and the log-sum-exp in log2 units
+  if (hipError_t e = images(p.dout, p.do_stride, p.num_q_heads, head_dim, T, nt, V(p.don), V(p.dor), stream, p.out_in, p.o_stride,
+                            p.lse, p.delta, p.lse2))
+    return e;
   return by_head_dim(head_dim, [&](auto d) {
     constexpr int D = decltype(d)::value;
-    const int64_t rows = 32 * (int64_t)nt * p.num_q_heads;
-    const int per_block = kThreads / (D / 8);
-    split_delta_kernel<D><<<(unsigned)((rows + per_block - 1) / per_block), kThreads, 0, stream>>>(p);
-    if (hipError_t e = hipGetLastError()) return e;
     const unsigned qgrid = (unsigned)nt * ((p.num_q_heads + kWaves - 1) / kWaves);
     if ((p.num_q_heads / p.num_kv_heads) % kWaves == 0)
       split_query_kernel<D, true, true><<<qgrid, kThreads, 0, stream>>>(p);

@@ -86,7 +86,7 @@ def test_split_attention_kernels_use_no_scratch_and_keep_their_ring_in_flight(hi
     )
     assert res.returncode == 0, res.stderr[-2000:]
     sizes = re.findall(r"ScratchSize \[bytes/lane\]: (\d+)", res.stderr)
-    assert len(sizes) >= 16 and set(sizes) == {"0"}, sizes
+    assert len(sizes) >= 14 and set(sizes) == {"0"}, sizes
     kernels = {k: v for k, v in _functions(out.read_text()).items() if "split_key_kernel" in k}
     assert len(kernels) == 4, sorted(kernels)
     for name, body in kernels.items():
