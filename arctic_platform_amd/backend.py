@@ -62,9 +62,10 @@ class ForestCascadeMetadata:
     forest: ForestMetadata | None
     slot_mapping: torch.Tensor
     num_decode_tokens: int
-    # set instead of ``forest`` for a step of fresh prompts only: causal attention of every
-    # prompt over itself, straight from the step's own K and V
+    # set when the batch ends in fresh prompts: causal attention of every such prompt over
+    # itself, straight from the step's own K and V
     fresh_prefill: SplitLayout | None = None
+    fresh_start: int = 0  # first token of the fresh prompts; the tokens before it go through ``forest``
 
 
 def parse_forest_cascade_configs(value) -> dict:
@@ -163,15 +164,33 @@ class ForestCascadeMetadataBuilder:
         num_tokens = m.num_reqs
         row_table = row_group = None
         if m.max_query_len > 1 and m.query_start_loc_cpu is not None and m.seq_lens_cpu is not None and self.enabled:
+            # The requests at the end of the batch that are fresh prompts (the engine puts decodes
+            # first): they attend on the split-attention kernels, the requests before them go on
+            # as a step of their own.
             q_lens = (m.query_start_loc_cpu[1 : m.num_reqs + 1] - m.query_start_loc_cpu[: m.num_reqs]).tolist()
-            if q_lens == m.seq_lens_cpu[: m.num_reqs].tolist() and sum(q_lens) >= self.FRESH_PREFILL_MIN_TOKENS:
-                key = ("fresh", tuple(q_lens))
+            s_lens = m.seq_lens_cpu[: m.num_reqs].tolist()
+            first = m.num_reqs
+            while first > 0 and q_lens[first - 1] == s_lens[first - 1] and q_lens[first - 1] > 1:
+                first -= 1
+            fresh = q_lens[first:]
+            if sum(fresh) >= self.FRESH_PREFILL_MIN_TOKENS:
+                key = ("fresh", tuple(fresh))
                 if key not in self._workspaces:
-                    self._keep(key, SplitLayout([(0, [n]) for n in q_lens], device=self.device))
+                    self._keep(key, SplitLayout([(0, [n]) for n in fresh], device=self.device))
                 self._workspaces.move_to_end(key)
-                total = sum(q_lens)
+                layout = self._workspaces[key]
+                total, before = sum(q_lens), sum(q_lens[:first])
+                rest = None
+                if first > 0:
+                    rest = self.build(
+                        common_prefix_len,
+                        dataclasses.replace(
+                            m, num_reqs=first, max_query_len=max(q_lens[:first]), num_actual_tokens=before,
+                            query_start_loc_cpu=None, seq_lens_cpu=None,
+                        ),
+                    ).forest
                 return ForestCascadeMetadata(
-                    forest=None, slot_mapping=m.slot_mapping[:total], num_decode_tokens=total, fresh_prefill=self._workspaces[key]
+                    forest=rest, slot_mapping=m.slot_mapping[:total], num_decode_tokens=total, fresh_prefill=layout, fresh_start=before
                 )
         if m.max_query_len > 1:
             # one row per query token: the row of its sequence, cut off behind the token itself;
@@ -265,12 +284,15 @@ class ForestCascadeAttentionImpl:
             output = torch.empty_like(query)
         if attn_metadata.fresh_prefill is not None:
             if key is None:
-                raise ValueError("a step of fresh prompts needs the step's key and value")
+                raise ValueError("a step with fresh prompts needs the step's key and value")
+            f = attn_metadata.fresh_start
             split_attention_forward(
-                q, key[:t].view(t, self.num_kv_heads, self.head_size), value[:t].view(t, self.num_kv_heads, self.head_size),
-                attn_metadata.fresh_prefill, self.scale, out=output[:t].view(t, self.num_heads, self.head_size),
+                q[f:], key[f:t].view(t - f, self.num_kv_heads, self.head_size), value[f:t].view(t - f, self.num_kv_heads, self.head_size),
+                attn_metadata.fresh_prefill, self.scale, out=output[f:t].view(t - f, self.num_heads, self.head_size),
             )
-            return output
+            if f == 0:
+                return output
+            t, q = f, q[:f]
         forest_cascade_decode(
             q, kv_cache, attn_metadata.forest, self.scale, k_scale, v_scale,
             out=output[:t].view(t, self.num_heads, self.head_size), return_lse=False,

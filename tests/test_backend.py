@@ -215,6 +215,52 @@ def test_fresh_prompts_take_the_split_attention_kernels(gpu):
     assert slow.fresh_prefill is None
     out2 = impl.forward(layer, q, None, None, cache, slow)
     torch.testing.assert_close(out2.view(T, hq, d).cpu().float(), ref, rtol=2e-2, atol=2e-2)
-    # a cached context in front of one sequence: not fresh any more
-    longer = dataclasses.replace(common, seq_lens_cpu=torch.tensor([lens[0] + 16, lens[1], lens[2]], dtype=torch.int32))
+    # a cached context in front of the last sequence: no fresh prompts at the end of the batch
+    longer = dataclasses.replace(common, seq_lens_cpu=torch.tensor([lens[0], lens[1], lens[2] + 16], dtype=torch.int32))
     assert builder.build(0, longer).fresh_prefill is None
+    # in front of the first one: the two behind it are still taken as fresh prompts
+    longer = dataclasses.replace(common, seq_lens_cpu=torch.tensor([lens[0] + 16, lens[1], lens[2]], dtype=torch.int32))
+    assert builder.build(0, longer).fresh_start == lens[0]
+
+
+@pytest.mark.gpu
+def test_decodes_followed_by_fresh_prompts_in_one_step(gpu):
+    """The usual serving step: running sequences bring one token each, and two new prompts
+    arrive behind them.  The decodes go through the forest, the prompts through the
+    split-attention kernels, every row is checked against the oracle on the filled cache."""
+    from arctic_platform_amd.kv_layout import kv_cache_shape
+    from oracle.attention import flat_decode_attention
+
+    hq, hkv, d = 8, 2, 128
+    scale = d**-0.5
+    gen = torch.Generator().manual_seed(21)
+    context = [70, 33, 128, 5, 200, 64]  # tokens already cached of the running sequences
+    q_lens = [1] * len(context) + [300, 150]
+    s_lens = [c + 1 for c in context] + [300, 150]
+    S, T = len(q_lens), sum(q_lens)
+    max_blocks = 24
+    table = torch.randperm(S * max_blocks, generator=gen).to(torch.int32).view(S, max_blocks).to(gpu)
+    cache = torch.randn(kv_cache_shape(S * max_blocks, 16, hkv, d), generator=gen).to(torch.bfloat16).to(gpu)
+    q, k, v = (torch.randn(T, h * d, generator=gen).to(torch.bfloat16).to(gpu) for h in (hq, hkv, hkv))
+    starts = torch.tensor([0] + q_lens).cumsum(0)
+    seq = torch.repeat_interleave(torch.arange(S), torch.tensor(q_lens))
+    pos = torch.cat([torch.arange(s - n, s) for n, s in zip(q_lens, s_lens)])
+    slots = (table.cpu().long()[seq, pos // 16] * 16 + pos % 16).to(gpu)
+    builder = ForestCascadeAttentionBackend.get_builder_cls()(hq, hkv, d, device=gpu)
+    impl = ForestCascadeAttentionBackend.get_impl_cls()(hq, d, scale, hkv)
+    layer = types.SimpleNamespace(k_scale=None, v_scale=None)
+    common = CommonAttentionMetadata(
+        query_start_loc=starts.to(torch.int32).to(gpu), seq_lens=torch.tensor(s_lens, dtype=torch.int32, device=gpu),
+        block_table_tensor=table, slot_mapping=slots, num_reqs=S, max_query_len=max(q_lens), num_actual_tokens=T,
+        query_start_loc_cpu=starts.to(torch.int32), seq_lens_cpu=torch.tensor(s_lens, dtype=torch.int32),
+    )
+    meta = builder.build(0, common)
+    assert meta.fresh_prefill is not None and meta.fresh_start == len(context) and meta.forest is not None
+    assert meta.forest.plan.num_seqs == len(context)
+    out = impl.forward(layer, q, k, v, cache, meta)
+    torch.cuda.synchronize()
+    meta.forest.check()
+    ref, _ = flat_decode_attention(
+        q.view(T, hq, d).cpu(), cache.cpu(), table.cpu()[seq], (pos + 1).to(torch.int32), scale, dtype=torch.float32
+    )
+    torch.testing.assert_close(out.view(T, hq, d).cpu().float(), ref, rtol=2e-2, atol=2e-2)
