@@ -122,6 +122,13 @@ def test_header_is_plain_c_and_links(tmp_path):
         "  size_t m = 0, o = 0, l = 0;\n"
         "  if (fca_workspace_bytes(&p, &m, &o, &l) != 0) { puts(fca_last_error()); return 1; }\n"
         '  printf("%d %zu %zu %zu\\n", fca_version(), m, o, l);\n'
+        "  /* the trainer's layout array is host code: two prompts of 3 and 2 tokens, responses 2, 1 | 4 */\n"
+        "  int32_t prompts[2] = {3, 2}, sizes[2] = {2, 1}, responses[3] = {2, 1, 4};\n"
+        "  int64_t n = 0;\n"
+        "  int32_t layout[64];\n"
+        "  if (fca_split_layout_ints(12, &n) != 0 || n > 64) return 2;\n"
+        "  if (fca_split_layout_build(2, prompts, sizes, responses, 12, layout) != 0) { puts(fca_last_error()); return 3; }\n"
+        '  for (int i = 0; i < 12; ++i) printf("%d ", layout[i]);\n'
         "  p.head_dim = 96;\n"
         "  return fca_workspace_bytes(&p, &m, &o, &l) == 0;  /* must be refused */\n"
         "}\n"
@@ -133,3 +140,5 @@ def test_header_is_plain_c_and_links(tmp_path):
     subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", f"-I{inc}", str(src), f"-L{libdir}", "-lzorro_fca", f"-Wl,-rpath,{libdir}", "-o", str(exe)], check=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
     assert int(out[0]) >= 1 and int(out[2]) == 512 * (320 * 16 // 1024 + 6) * 32 * 128 * 2
+    # lim of every key: a prompt token is seen up to the end of its group, a response token up to its own end
+    assert [int(x) for x in out[4:16]] == [6, 6, 6, 5, 5, 6, 12, 12, 12, 12, 12, 12]
