@@ -233,7 +233,7 @@ def _run_case(layout, hq, hkv, d, seed, strided=False, q_gain=1.0):
         qd = fused[:, : hq * d].view(t, hq, d)
         kd = fused[:, hq * d : (hq + hkv) * d].view(t, hkv, d)
         vd = fused[:, (hq + hkv) * d :].view(t, hkv, d)
-        assert qd.stride(0) == (hq + 2 * hkv) * d
+        assert t == 1 or qd.stride(0) == (hq + 2 * hkv) * d
     else:
         qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
     out, lse = split_attention_forward(qd, kd, vd, L, scale)
