@@ -1,4 +1,5 @@
-"""MI355X-native forest cascade decode attention (ZoRRo inference path)."""
+"""MI355X-native forest cascade decode attention (ZoRRo inference path) and the trainer's
+split attention over deduplicated batches (ZoRRo Train)."""
 
 from .config import ModelConfig, build_model_config, parse_arctic_inference_rollout, validate_fca_support
 from .kv_layout import BLOCK_SIZE, convert_cache, kv_cache_shape, pack_blocks, unpack_blocks
@@ -16,6 +17,8 @@ __all__ = [
     "build_forest_metadata",
     "forest_cascade_decode",
     "append_kv",
+    "SplitLayout",
+    "split_attention",
 ]
 
 
@@ -34,6 +37,10 @@ def __getattr__(name):
         from . import backend
 
         return getattr(backend, name)
+    if name in ("SplitLayout", "split_attention", "split_attention_forward", "split_attention_backward", "split_attention_padded"):
+        from . import split_attention as module
+
+        return getattr(module, name)
     if name == "append_kv":
         from . import cache
 
