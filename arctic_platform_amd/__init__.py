@@ -18,7 +18,8 @@ __all__ = [
     "forest_cascade_decode",
     "append_kv",
     "SplitLayout",
-    "split_attention",
+    "split_attention_forward",
+    "split_attention_backward",
 ]
 
 
@@ -37,10 +38,12 @@ def __getattr__(name):
         from . import backend
 
         return getattr(backend, name)
-    if name in ("SplitLayout", "split_attention", "split_attention_forward", "split_attention_backward", "split_attention_padded"):
-        from . import split_attention as module
+    if name in ("SplitLayout", "split_attention_forward", "split_attention_backward", "split_attention_padded"):
+        # (the operator `split_attention` itself is reached as split_attention.split_attention:
+        # the name belongs to the submodule)
+        import importlib
 
-        return getattr(module, name)
+        return getattr(importlib.import_module(".split_attention", __name__), name)
     if name == "append_kv":
         from . import cache
 
