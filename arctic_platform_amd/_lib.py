@@ -32,6 +32,7 @@ EXPORTS = (
     "fca_merge",
     "fca_decode_step",
     "fca_append_kv",
+    "fca_gather_kv",
     "fca_calibration_copy",
     "fca_split_layout_ints",
     "fca_split_layout_build",
@@ -157,6 +158,7 @@ def load_library() -> ctypes.CDLL:
     lib.fca_merge.argtypes = [P(FcaPlan), VP, VP, VP, VP, I64, I64, I32, VP, VP]
     lib.fca_decode_step.argtypes = [P(FcaPlan), P(FcaTensors), VP, VP, VP, VP, I64, I64, I32, VP, VP]
     lib.fca_append_kv.argtypes = [VP, VP, I64, I64, I32, I32, I32, VP, VP, VP, I64, I64, I32, VP, VP, VP]
+    lib.fca_gather_kv.argtypes = lib.fca_append_kv.argtypes
     lib.fca_calibration_copy.argtypes = [VP, VP, ctypes.c_size_t, VP]
     F32 = ctypes.c_float
     lib.fca_split_layout_ints.argtypes = [I32, P(I64)]

@@ -18,8 +18,23 @@ from .forest import _stream_ptr
 from .kv_layout import BLOCK_SIZE
 
 
+def gather_kv(kv_cache, slot_mapping, head_dim, k_scale=None, v_scale=None, out=None):
+    """The way back: bf16 ``(key, value)`` rows ``[T, Hkv, D]`` of the tokens at ``slot_mapping``
+    (fp8 caches times their scales: the values decode attention sees; negative slot = zeros)."""
+    hkv = kv_cache.shape[2]
+    t = slot_mapping.shape[0]
+    if out is None:
+        out = tuple(torch.empty(t, hkv, head_dim, dtype=torch.bfloat16, device=kv_cache.device) for _ in range(2))
+    _cache_rows(True, out[0], out[1], kv_cache, slot_mapping, k_scale, v_scale)
+    return out
+
+
 def append_kv(key, value, kv_cache, slot_mapping, k_scale=None, v_scale=None) -> None:
     """key, value: bf16 ``[T, Hkv, D]``; slot_mapping: int64 ``[T]``; kv_cache as in kv_layout."""
+    _cache_rows(False, key, value, kv_cache, slot_mapping, k_scale, v_scale)
+
+
+def _cache_rows(gather, key, value, kv_cache, slot_mapping, k_scale, v_scale) -> None:
     if key.dtype != torch.bfloat16 or value.dtype != torch.bfloat16 or key.shape != value.shape or key.dim() != 3:
         raise TypeError("key and value must be bfloat16 tensors of the same shape [tokens, kv_heads, head_dim]")
     if key.stride() != value.stride() or key.stride(2) != 1:
@@ -43,7 +58,7 @@ def append_kv(key, value, kv_cache, slot_mapping, k_scale=None, v_scale=None) ->
     lib = _lib.load_library()
     esz = kv_cache.element_size()
     _lib.check(
-        lib.fca_append_kv(
+        (lib.fca_gather_kv if gather else lib.fca_append_kv)(
             key.data_ptr(), value.data_ptr(), key.stride(0), key.stride(1), t, hkv, d, slot_mapping.data_ptr(),
             kv_cache.data_ptr(), kv_cache.data_ptr() + kv_cache.stride(0) * esz, kv_cache.stride(1), kv_cache.stride(2),
             code, k_scale.data_ptr() if k_scale is not None else None, v_scale.data_ptr() if v_scale is not None else None,

@@ -273,10 +273,10 @@ int fca_decode_step(const fca_plan* plan, const fca_tensors* t, void* meta_dev, 
                    lse_dev, stream);
 }
 
-int fca_append_kv(const void* key_dev, const void* value_dev, int64_t token_stride, int64_t head_stride,
-                  int32_t num_tokens, int32_t num_kv_heads, int32_t head_dim, const int64_t* slot_mapping_dev,
-                  void* k_cache_dev, void* v_cache_dev, int64_t kv_block_stride, int64_t kv_head_stride, int32_t kv_dtype,
-                  const float* k_scale_dev, const float* v_scale_dev, void* stream) {
+static int cache_rows(bool gather, const void* key_dev, const void* value_dev, int64_t token_stride, int64_t head_stride,
+                      int32_t num_tokens, int32_t num_kv_heads, int32_t head_dim, const int64_t* slot_mapping_dev,
+                      void* k_cache_dev, void* v_cache_dev, int64_t kv_block_stride, int64_t kv_head_stride, int32_t kv_dtype,
+                      const float* k_scale_dev, const float* v_scale_dev, void* stream) {
   if (num_tokens < 0 || num_kv_heads < 1) return fail(FCA_ERR_INVALID_ARG, "num_tokens must be >= 0 and num_kv_heads >= 1");
   if (head_dim != 64 && head_dim != 128) return fail(FCA_ERR_UNSUPPORTED, "head_dim %d is not supported (64 or 128)", head_dim);
   if (kv_dtype != FCA_BF16 && kv_dtype != FCA_FP8_E4M3)
@@ -306,8 +306,26 @@ int fca_append_kv(const void* key_dev, const void* value_dev, int64_t token_stri
   a.num_tokens = num_tokens;
   a.num_kv_heads = num_kv_heads;
   a.head_dim = head_dim;
-  hipError_t e = fca::launch_append(a, kv_dtype, static_cast<hipStream_t>(stream));
-  return e == hipSuccess ? FCA_OK : hip_fail(e, "cache append launch");
+  hipError_t e = gather ? fca::launch_gather(a, kv_dtype, static_cast<hipStream_t>(stream))
+                        : fca::launch_append(a, kv_dtype, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? FCA_OK : hip_fail(e, gather ? "cache gather launch" : "cache append launch");
+}
+
+int fca_append_kv(const void* key_dev, const void* value_dev, int64_t token_stride, int64_t head_stride,
+                  int32_t num_tokens, int32_t num_kv_heads, int32_t head_dim, const int64_t* slot_mapping_dev,
+                  void* k_cache_dev, void* v_cache_dev, int64_t kv_block_stride, int64_t kv_head_stride, int32_t kv_dtype,
+                  const float* k_scale_dev, const float* v_scale_dev, void* stream) {
+  return cache_rows(false, key_dev, value_dev, token_stride, head_stride, num_tokens, num_kv_heads, head_dim, slot_mapping_dev,
+                    k_cache_dev, v_cache_dev, kv_block_stride, kv_head_stride, kv_dtype, k_scale_dev, v_scale_dev, stream);
+}
+
+int fca_gather_kv(void* key_dev, void* value_dev, int64_t token_stride, int64_t head_stride, int32_t num_tokens,
+                  int32_t num_kv_heads, int32_t head_dim, const int64_t* slot_mapping_dev, const void* k_cache_dev,
+                  const void* v_cache_dev, int64_t kv_block_stride, int64_t kv_head_stride, int32_t kv_dtype,
+                  const float* k_scale_dev, const float* v_scale_dev, void* stream) {
+  return cache_rows(true, key_dev, value_dev, token_stride, head_stride, num_tokens, num_kv_heads, head_dim, slot_mapping_dev,
+                    const_cast<void*>(k_cache_dev), const_cast<void*>(v_cache_dev), kv_block_stride, kv_head_stride, kv_dtype,
+                    k_scale_dev, v_scale_dev, stream);
 }
 
 int fca_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void* stream) {

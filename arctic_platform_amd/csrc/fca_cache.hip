@@ -59,6 +59,71 @@ __global__ __launch_bounds__(256) void fca_append_kernel(AppendParams p) {
   }
 }
 
+// The way back: the tokens at the given slots leave the cache as bf16 rows [T, Hkv, D] (fp8
+// tiles are multiplied by their per-head scales, i.e. the values decode attention sees).  A
+// negative slot gives a row of zeros.  Same thread mapping as the append.
+template <bool FP8>
+__global__ __launch_bounds__(256) void fca_gather_kernel(AppendParams p) {
+  constexpr int XW = FP8 ? 16 : 8;
+  const int groups = p.head_dim / XW;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = (int64_t)p.num_tokens * p.num_kv_heads * groups;
+  if (idx >= total) return;
+  const int c = (int)(idx % groups);
+  const int h = (int)((idx / groups) % p.num_kv_heads);
+  const int t = (int)(idx / ((int64_t)groups * p.num_kv_heads));
+  const int64_t slot = p.slot_mapping[t];
+  __hip_bfloat16* kdst = reinterpret_cast<__hip_bfloat16*>(const_cast<void*>(p.key)) + (int64_t)t * p.token_stride +
+                         (int64_t)h * p.head_stride + c * XW;
+  __hip_bfloat16* vdst = reinterpret_cast<__hip_bfloat16*>(const_cast<void*>(p.value)) + (int64_t)t * p.token_stride +
+                         (int64_t)h * p.head_stride + c * XW;
+  __hip_bfloat16 kv[XW], vv[XW];
+  if (slot < 0) {
+#pragma unroll
+    for (int e = 0; e < XW; ++e) kv[e] = vv[e] = __float2bfloat16(0.f);
+  } else {
+    const int64_t blk = slot / kBlock;
+    const int off = (int)(slot - blk * kBlock);
+    const int64_t tile = blk * p.cache_block_stride + (int64_t)h * p.cache_head_stride;  // elements
+    if constexpr (FP8) {
+      const float ks = p.k_scale ? p.k_scale[h] : 1.f;
+      const float vs = p.v_scale ? p.v_scale[h] : 1.f;
+      const unsigned char* ksrc = reinterpret_cast<const unsigned char*>(p.k_cache) + tile + ((int64_t)c * kBlock + off) * XW;
+      const unsigned char* vsrc = reinterpret_cast<const unsigned char*>(p.v_cache) + tile + (int64_t)c * XW * kBlock + off;
+      unsigned char kq[XW];
+      *reinterpret_cast<int4*>(kq) = *reinterpret_cast<const int4*>(ksrc);
+#pragma unroll
+      for (int e = 0; e < XW; ++e) {
+        kv[e] = __float2bfloat16(__builtin_amdgcn_cvt_f32_fp8((int)kq[e], 0) * ks);
+        vv[e] = __float2bfloat16(__builtin_amdgcn_cvt_f32_fp8((int)vsrc[e * kBlock], 0) * vs);
+      }
+    } else {
+      const __hip_bfloat16* ksrc = reinterpret_cast<const __hip_bfloat16*>(p.k_cache) + tile + ((int64_t)c * kBlock + off) * XW;
+      const __hip_bfloat16* vsrc = reinterpret_cast<const __hip_bfloat16*>(p.v_cache) + tile + (int64_t)c * XW * kBlock + off;
+      *reinterpret_cast<int4*>(kv) = *reinterpret_cast<const int4*>(ksrc);
+#pragma unroll
+      for (int e = 0; e < XW; ++e) vv[e] = vsrc[e * kBlock];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < XW; e += 8) {
+    *reinterpret_cast<int4*>(kdst + e) = *reinterpret_cast<const int4*>(kv + e);
+    *reinterpret_cast<int4*>(vdst + e) = *reinterpret_cast<const int4*>(vv + e);
+  }
+}
+
+hipError_t launch_gather(const AppendParams& p, int kv_dtype, hipStream_t stream) {
+  const bool fp8 = kv_dtype == FCA_FP8_E4M3;
+  const int64_t total = (int64_t)p.num_tokens * p.num_kv_heads * (p.head_dim / (fp8 ? 16 : 8));
+  if (total == 0) return hipSuccess;
+  const int grid = (int)((total + 255) / 256);
+  if (fp8)
+    hipLaunchKernelGGL(fca_gather_kernel<true>, dim3(grid), dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL(fca_gather_kernel<false>, dim3(grid), dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+
 hipError_t launch_append(const AppendParams& p, int kv_dtype, hipStream_t stream) {
   const bool fp8 = kv_dtype == FCA_FP8_E4M3;
   const int64_t total = (int64_t)p.num_tokens * p.num_kv_heads * (p.head_dim / (fp8 ? 16 : 8));

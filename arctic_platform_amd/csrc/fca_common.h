@@ -232,6 +232,7 @@ hipError_t launch_build(const BuildParams& p, hipStream_t stream);
 hipError_t launch_rows(const int32_t* query_start_loc, const int32_t* seq_lens, int num_reqs, int num_rows, int max_blocks,
                        int32_t* row_table, int32_t* row_lens, int32_t* row_group, hipStream_t stream);
 hipError_t launch_append(const AppendParams& p, int kv_dtype, hipStream_t stream);
+hipError_t launch_gather(const AppendParams& p, int kv_dtype, hipStream_t stream);  // key / value are written
 hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, hipStream_t stream);
 hipError_t launch_attend32(const AttendParams& p, const fca_plan& plan, int kv_dtype, int grid, hipStream_t stream);
 hipError_t launch_merge(const MergeParams& p, hipStream_t stream);

@@ -227,6 +227,15 @@ int fca_append_kv(const void* key_dev, const void* value_dev, int64_t token_stri
                   int32_t num_tokens, int32_t num_kv_heads, int32_t head_dim, const int64_t* slot_mapping_dev,
                   void* k_cache_dev, void* v_cache_dev, int64_t kv_block_stride, int64_t kv_head_stride, int32_t kv_dtype,
                   const float* k_scale_dev, const float* v_scale_dev, void* stream);
+/* The way back: the tokens at slot_mapping[t] leave the cache as bf16 rows key[t], value[t]
+ * ([T, Hkv, D]; fp8 tiles times their per-head scales, i.e. the values decode attention
+ * sees; a negative slot gives zeros).  Used by the adapter to hand a prompt's cached context
+ * to the split-attention kernels; like fca_append_kv it stands for an op of the external
+ * engine and has no in-tree counterpart in the reference. */
+int fca_gather_kv(void* key_dev, void* value_dev, int64_t token_stride, int64_t head_stride, int32_t num_tokens,
+                  int32_t num_kv_heads, int32_t head_dim, const int64_t* slot_mapping_dev, const void* k_cache_dev,
+                  const void* v_cache_dev, int64_t kv_block_stride, int64_t kv_head_stride, int32_t kv_dtype,
+                  const float* k_scale_dev, const float* v_scale_dev, void* stream);
 
 /* ---- split attention of the trainer (forward and backward) ---------------------------
  * Attention over a deduplicated, unpadded training batch: q [T, Hq, D], k and v

@@ -73,6 +73,28 @@ def test_kernel_is_bit_exact(gpu, dtype, d):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 64), (torch.bfloat16, 128), (torch.float8_e4m3fn, 64), (torch.float8_e4m3fn, 128)])
+def test_gather_is_the_way_back(gpu, dtype, d):
+    """Rows gathered from the cache are, bit for bit, what the oracle's cache holds at those
+    slots (times the per-head scales for fp8, rounded to bf16); a negative slot gives zeros."""
+    from arctic_platform_amd.cache import gather_kv
+
+    cache, key, value, slots, ks, vs = _case(dtype, d, 12)
+    want_cache = append_kv_reference(cache, key, value, slots, ks, vs)
+    k_blocks, v_blocks = unpack_blocks(want_cache, d)  # [blocks, 16, Hkv, D]
+    pick = slots.clone()
+    pick[1] = -1
+    got_k, got_v = gather_kv(want_cache.to(gpu), pick.to(gpu), d, None if ks is None else ks.to(gpu), None if vs is None else vs.to(gpu))
+    for got, blocks, scale in ((got_k, k_blocks, ks), (got_v, v_blocks, vs)):
+        rows = blocks[pick.clamp(min=0) // 16, pick.clamp(min=0) % 16].float()
+        if dtype == torch.float8_e4m3fn:
+            rows = rows * scale[None, :, None]
+        rows = rows.to(torch.bfloat16)
+        rows[pick < 0] = 0
+        assert torch.equal(got.cpu().view(torch.int16), rows.view(torch.int16))
+
+
+@pytest.mark.gpu
 def test_append_then_attend(gpu):
     """Decode step end to end: append the new token of every sequence, then attend."""
     from arctic_platform_amd.cache import append_kv
