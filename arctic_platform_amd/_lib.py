@@ -162,7 +162,7 @@ def load_library() -> ctypes.CDLL:
     lib.fca_calibration_copy.argtypes = [VP, VP, ctypes.c_size_t, VP]
     F32 = ctypes.c_float
     lib.fca_split_layout_ints.argtypes = [I32, P(I64)]
-    lib.fca_split_layout_build.argtypes = [I32, VP, VP, VP, I32, VP]
+    lib.fca_split_layout_build.argtypes = [I32, VP, VP, VP, I32, I32, VP]
     lib.fca_split_workspace_bytes.argtypes = [P(FcaSplitPlan), SZ, SZ]
     lib.fca_split_attention_forward.argtypes = [P(FcaSplitPlan), VP, I64, VP, I64, VP, I64, VP, F32, VP, VP, I64, VP, VP]
     lib.fca_split_attention_backward.argtypes = (

@@ -377,7 +377,7 @@ int fca_split_layout_ints(int32_t num_tokens, int64_t* num_ints) {
 }
 
 int fca_split_layout_build(int32_t num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,
-                           const int32_t* response_tokens, int32_t num_tokens, int32_t* layout_host) {
+                           const int32_t* response_tokens, int32_t num_tokens, int32_t responses_only, int32_t* layout_host) {
   if (num_groups < 0 || num_tokens < 0) return fail(FCA_ERR_INVALID_ARG, "num_groups and num_tokens must be >= 0");
   if (num_groups > 0 && (!prompt_tokens || !group_sizes)) return fail(FCA_ERR_INVALID_ARG, "prompt_tokens and group_sizes must be non-NULL");
   int64_t total = 0, samples = 0;
@@ -395,7 +395,8 @@ int fca_split_layout_build(int32_t num_groups, const int32_t* prompt_tokens, con
     return fail(FCA_ERR_INVALID_ARG, "the layout holds %lld tokens, num_tokens says %d", (long long)total, num_tokens);
   if (num_tokens == 0) return FCA_OK;
   if (!layout_host) return fail(FCA_ERR_INVALID_ARG, "layout_host is NULL");
-  fca::build_split_layout(num_groups, prompt_tokens, group_sizes, response_tokens, (num_tokens + 31) / 32, layout_host);
+  fca::build_split_layout(num_groups, prompt_tokens, group_sizes, response_tokens, (num_tokens + 31) / 32, responses_only != 0,
+                          layout_host);
   return FCA_OK;
 }
 

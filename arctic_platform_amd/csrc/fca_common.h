@@ -210,7 +210,7 @@ inline bool split_by_head(int64_t tiles, int num_q_heads, int num_kv_heads) {
 }
 // Offsets into the int32 layout array of a batch of `tiles` 32-token tiles.
 struct SplitLayout {
-  int64_t kv_lim, q_tiles, kv_qend, q_order, kv_limmin, kv_order, total;
+  int64_t kv_lim, q_tiles, kv_qend, q_order, kv_limmin, kv_order, q_index, total;
 };
 __host__ __device__ inline SplitLayout make_split_layout(int64_t tiles) {
   SplitLayout L;
@@ -220,11 +220,12 @@ __host__ __device__ inline SplitLayout make_split_layout(int64_t tiles) {
   L.q_order = L.kv_qend + tiles;
   L.kv_limmin = L.q_order + tiles;
   L.kv_order = L.kv_limmin + tiles;  // ceil(tiles / 4) entries used
-  L.total = L.kv_order + tiles;
+  L.q_index = L.kv_order + tiles;  // row of q and out that belongs to a packed token, -1 = none
+  L.total = L.q_index + 32 * tiles;
   return L;
 }
 void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,
-                        const int32_t* response_tokens, int64_t tiles, int32_t* out);
+                        const int32_t* response_tokens, int64_t tiles, bool responses_only, int32_t* out);
 hipError_t launch_split_forward(const SplitParams& p, int head_dim, hipStream_t stream);
 hipError_t launch_split_backward(const SplitParams& p, int head_dim, hipStream_t stream);
 

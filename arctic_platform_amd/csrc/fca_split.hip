@@ -41,7 +41,7 @@ namespace fca {
 
 // ---- host: the layout array ------------------------------------------------------------
 void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,
-                        const int32_t* response_tokens, int64_t tiles, int32_t* out) {
+                        const int32_t* response_tokens, int64_t tiles, bool responses_only, int32_t* out) {
   const SplitLayout L = make_split_layout(tiles);
   const int64_t padded = 32 * tiles;
   std::vector<int32_t> own(padded, 0), pstart(padded, 0), pend(padded, 0), group_of(padded, 0);
@@ -49,8 +49,12 @@ void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int3
   int64_t t = 0;
   int64_t ri = 0;
   int group = 0;
+  int32_t* q_index = out + L.q_index;
+  int32_t next_q = 0;
+  bool in_prompt = false;
   auto fill = [&](int64_t from, int64_t to, int64_t limit, int64_t p0, int64_t p1) {
     for (int64_t x = from; x < to; ++x) {
+      q_index[x] = responses_only && in_prompt ? -1 : next_q++;
       group_of[x] = group;
       lim[x] = (int32_t)limit;
       own[x] = (int32_t)from;
@@ -63,7 +67,9 @@ void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int3
     const int64_t p0 = t, p1 = t + prompt_tokens[g];
     int64_t gend = p1;
     for (int s = 0; s < group_sizes[g]; ++s) gend += response_tokens[ri + s];
+    in_prompt = true;
     fill(p0, p1, gend, p0, p1);
+    in_prompt = false;
     t = p1;
     for (int s = 0; s < group_sizes[g]; ++s) {
       const int64_t s1 = t + response_tokens[ri + s];
@@ -72,7 +78,7 @@ void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int3
     }
     ri += group_sizes[g];
   }
-  for (int64_t x = t; x < padded; ++x) lim[x] = 0;
+  for (int64_t x = t; x < padded; ++x) lim[x] = 0, q_index[x] = -1;
   std::vector<int64_t> qcost(tiles);
   for (int64_t i = 0; i < tiles; ++i) {
     // The needs of a tile's first row cover those of the rows behind it: they belong to
@@ -85,6 +91,7 @@ void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int3
     a1 = std::max(a0, std::min(a1, b0));
     int32_t* rec = out + L.q_tiles + 4 * i;
     rec[0] = a0, rec[1] = a1, rec[2] = b0, rec[3] = 0;
+    for (int x = 0; x < 32; ++x) rec[3] |= q_index[r0 + x] >= 0;  // any row of the tile that has a query
     qcost[i] = (a1 - a0) + (i - b0 + 1);
     int32_t mx = 0;
     for (int x = 0; x < 32; ++x) mx = std::max(mx, lim[r0 + x]);
@@ -220,15 +227,17 @@ __global__ __launch_bounds__(kThreads, SHARED ? 2 : 1) void split_query_kernel(S
     if (hq >= p.num_q_heads) return;
   }
   const int hkv = hq / (p.num_q_heads / p.num_kv_heads);
-  const int T = p.num_tokens, nt = p.num_tiles;
+  const int nt = p.num_tiles;
   const int64_t padded = 32 * (int64_t)nt;
   const int i = __builtin_amdgcn_readfirstlane(p.layout[L.q_order + blockIdx.x / quads]);
   const int a0 = __builtin_amdgcn_readfirstlane(p.layout[L.q_tiles + 4 * i]);
   const int a1 = __builtin_amdgcn_readfirstlane(p.layout[L.q_tiles + 4 * i + 1]);
   const int b0 = __builtin_amdgcn_readfirstlane(p.layout[L.q_tiles + 4 * i + 2]);
+  if (__builtin_amdgcn_readfirstlane(p.layout[L.q_tiles + 4 * i + 3]) == 0) return;  // a tile of rows without queries
   const int na = a1 - a0, ntile = na + i - b0 + 1;
   const int r = 32 * i + n;
-  const int64_t rc = min(r, T - 1);
+  const int qi = p.layout[L.q_index + r];  // this lane's row of q and out, -1 = none
+  const int64_t rc = max(qi, 0);
 
   bf16x8 qreg[KS], doreg[BWD ? KS : 1];
 #pragma unroll
@@ -384,10 +393,10 @@ __global__ __launch_bounds__(kThreads, SHARED ? 2 : 1) void split_query_kernel(S
   if constexpr (!BWD) {
     const float l = lrow + __shfl_xor(lrow, 32);
     const float inv = l > 0.f ? 1.f / l : 0.f;
-    if (r < T) store_rows<D>(p.out, (int64_t)r * p.o_stride + hq * D, h, acc, inv);
+    if (qi >= 0) store_rows<D>(p.out, (int64_t)qi * p.o_stride + hq * D, h, acc, inv);
     if (h == 0) p.lse[hq * padded + r] = l > 0.f ? (mrow + fast_log2(l)) * kLn2 : 0.f;
   } else {
-    if (r < T) store_rows<D>(p.dq, (int64_t)r * p.dq_stride + hq * D, h, acc, p.scale);
+    if (qi >= 0) store_rows<D>(p.dq, (int64_t)qi * p.dq_stride + hq * D, h, acc, p.scale);
   }
 }
 

@@ -31,12 +31,17 @@ def _stream_ptr(device) -> int:
 class SplitLayout:
     """Token layout of one deduplicated batch: ``[(prompt_tokens, [response_tokens, ...]), ...]``."""
 
-    def __init__(self, groups, device="cuda"):
+    def __init__(self, groups, device="cuda", responses_only=False):
+        """``responses_only`` (forward only): ``k`` and ``v`` hold every token, ``q`` and ``out`` only
+        the response rows, in packed order, and the prompts' own attention is not computed (a
+        prefill chunk behind a cached context, with the context as the prompt)."""
         self.groups = [(int(p), [int(n) for n in rs]) for p, rs in groups]
+        self.responses_only = bool(responses_only)
         prompt = np.asarray([p for p, _ in self.groups], dtype=np.int32)
         sizes = np.asarray([len(rs) for _, rs in self.groups], dtype=np.int32)
         resp = np.asarray([n for _, rs in self.groups for n in rs], dtype=np.int32)
         self.num_tokens = int(prompt.sum()) + int(resp.sum())
+        self.num_query_rows = int(resp.sum()) if self.responses_only else self.num_tokens
         self.num_tiles = (self.num_tokens + 31) // 32
         lib = _lib.load_library()
         n = ctypes.c_int64()
@@ -44,7 +49,8 @@ class SplitLayout:
         self.host = np.zeros(max(int(n.value), 1), dtype=np.int32)
         _lib.check(
             lib.fca_split_layout_build(
-                len(self.groups), prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, self.num_tokens, self.host.ctypes.data
+                len(self.groups), prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, self.num_tokens,
+                1 if self.responses_only else 0, self.host.ctypes.data,
             )
         )
         self.device = torch.device(device)
@@ -97,6 +103,10 @@ class SplitLayout:
         o = 39 * self.num_tiles
         return self.host[o : o + (self.num_tiles + 3) // 4]
 
+    def q_index(self):
+        o = 40 * self.num_tiles
+        return self.host[o : o + 32 * self.num_tiles]
+
     def scratch(self, plan, backward: bool) -> torch.Tensor:
         """Scratch of a call, kept with the layout: layers run one after the other on a stream."""
         fwd, bwd = ctypes.c_size_t(), ctypes.c_size_t()
@@ -126,14 +136,15 @@ def split_attention_forward(q, k, v, layout: SplitLayout, scale: float, out=None
     """q ``[T, Hq, D]``, k, v ``[T, Hkv, D]`` bf16 in deduplicated order.  Returns
     ``(out [T, Hq, D] bf16, lse fp32 [Hq, 32 * ceil(T / 32)])``; ``lse[:, :T]`` is the
     natural-log log-sum-exp of every row's scores.  ``out`` may be given to write into."""
-    t = layout.num_tokens
-    for name, x in (("q", q), ("k", k), ("v", v)):
+    t, rows = layout.num_tokens, layout.num_query_rows
+    _check_rows("q", q, rows)
+    for name, x in (("k", k), ("v", v)):
         _check_rows(name, x, t)
-    plan = _plan(q, k)
+    plan = _lib.FcaSplitPlan(t, q.shape[1], k.shape[1], q.shape[2])
     if out is None:
-        out = torch.empty((t, q.shape[1], q.shape[2]), dtype=torch.bfloat16, device=q.device)
+        out = torch.empty((rows, q.shape[1], q.shape[2]), dtype=torch.bfloat16, device=q.device)
     else:
-        _check_rows("out", out, t)
+        _check_rows("out", out, rows)
     lse = torch.empty((q.shape[1], 32 * layout.num_tiles), dtype=torch.float32, device=q.device)
     if t == 0:
         return out, lse
@@ -150,6 +161,8 @@ def split_attention_forward(q, k, v, layout: SplitLayout, scale: float, out=None
 def split_attention_backward(dout, q, k, v, out, lse, layout: SplitLayout, scale: float):
     """Gradients ``(dq, dk, dv)`` of ``split_attention_forward``'s ``out`` with respect to
     its inputs, for the upstream gradient ``dout``."""
+    if layout.responses_only:
+        raise ValueError("a layout with responses_only serves the forward only")
     t = layout.num_tokens
     for name, x in (("q", q), ("k", k), ("v", v), ("out", out), ("dout", dout)):
         _check_rows(name, x, t)

@@ -260,9 +260,14 @@ int fca_split_layout_ints(int32_t num_tokens, int64_t* num_ints);
  * the token layout of ZoRRoTrain.get_group_token_layout (zorro_train.py:2413-2436):
  * prompt_tokens[g], group_sizes[g] samples per group, response_tokens one per sample in
  * group order.  The counts must add up to num_tokens.  The caller copies the array to the
- * device once per batch; every layer's forward and backward reads it. */
+ * device once per batch; every layer's forward and backward reads it.
+ * responses_only != 0 (forward only, no counterpart in the reference): k and v still hold
+ * all num_tokens rows, but q and out hold the response rows only, in packed order, and the
+ * prompts' own attention is not computed -- a prefill chunk behind a cached context, with
+ * the context as the prompt. */
 int fca_split_layout_build(int32_t num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,
-                           const int32_t* response_tokens, int32_t num_tokens, int32_t* layout_host);
+                           const int32_t* response_tokens, int32_t num_tokens, int32_t responses_only,
+                           int32_t* layout_host);
 /* Bytes of device scratch a forward / a backward call needs: operand tiles in MFMA order,
  * per-row sums, and for small batches fp32 slices of dk and dv per query head of a KV head. */
 int fca_split_workspace_bytes(const fca_split_plan* plan, size_t* forward_bytes, size_t* backward_bytes);

@@ -125,9 +125,9 @@ def test_header_is_plain_c_and_links(tmp_path):
         "  /* the trainer's layout array is host code: two prompts of 3 and 2 tokens, responses 2, 1 | 4 */\n"
         "  int32_t prompts[2] = {3, 2}, sizes[2] = {2, 1}, responses[3] = {2, 1, 4};\n"
         "  int64_t n = 0;\n"
-        "  int32_t layout[64];\n"
-        "  if (fca_split_layout_ints(12, &n) != 0 || n > 64) return 2;\n"
-        "  if (fca_split_layout_build(2, prompts, sizes, responses, 12, layout) != 0) { puts(fca_last_error()); return 3; }\n"
+        "  int32_t layout[512];\n"
+        "  if (fca_split_layout_ints(12, &n) != 0 || n > 512) return 2;\n"
+        "  if (fca_split_layout_build(2, prompts, sizes, responses, 12, 0, layout) != 0) { puts(fca_last_error()); return 3; }\n"
         '  for (int i = 0; i < 12; ++i) printf("%d ", layout[i]);\n'
         "  p.head_dim = 96;\n"
         "  return fca_workspace_bytes(&p, &m, &o, &l) == 0;  /* must be refused */\n"

@@ -182,17 +182,31 @@ def test_layout_from_the_trainers_reconstruction_info():
     assert unpadded.kv_lim()[:19].tolist() == [10] * 5 + [9] * 4 + [10] + [19] * 6 + [19] * 3
 
 
+def test_layout_for_response_rows_only():
+    """A prefill chunk behind a cached context: the context is the prompt, q and out hold the
+    chunk's rows only, numbered in packed order; tiles of nothing but context rows are skipped."""
+    L = SplitLayout([(70, [5]), (0, [3]), (33, [40])], device="cpu", responses_only=True)
+    assert L.num_tokens == 151 and L.num_query_rows == 48
+    qi = L.q_index()
+    assert qi[:70].tolist() == [-1] * 70 and qi[70:78].tolist() == list(range(8))
+    assert qi[78:111].tolist() == [-1] * 33 and qi[111:151].tolist() == list(range(8, 48)) and (qi[151:] == -1).all()
+    assert [int(rec[3]) for rec in L.q_tiles()] == [0, 0, 1, 1, 1]
+    full = SplitLayout([(70, [5]), (0, [3]), (33, [40])], device="cpu")
+    assert full.q_index()[:151].tolist() == list(range(151)) and all(rec[3] == 1 for rec in full.q_tiles())
+    assert (full.kv_lim() == L.kv_lim()).all()
+
+
 def test_layout_arguments_are_checked():
     lib = _lib.load_library()
     prompt = np.asarray([4], dtype=np.int32)
     sizes = np.asarray([2], dtype=np.int32)
     resp = np.asarray([3, 2], dtype=np.int32)
-    out = np.zeros(64, dtype=np.int32)
-    assert lib.fca_split_layout_build(1, prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, 9, out.ctypes.data) == 0
-    assert lib.fca_split_layout_build(1, prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, 10, out.ctypes.data) < 0
+    out = np.zeros(128, dtype=np.int32)
+    assert lib.fca_split_layout_build(1, prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, 9, 0, out.ctypes.data) == 0
+    assert lib.fca_split_layout_build(1, prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, 10, 0, out.ctypes.data) < 0
     assert b"holds 9 tokens" in lib.fca_last_error()
     resp[1] = -1
-    assert lib.fca_split_layout_build(1, prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, 6, out.ctypes.data) < 0
+    assert lib.fca_split_layout_build(1, prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, 6, 0, out.ctypes.data) < 0
     plan = _lib.FcaSplitPlan(100, 6, 4, 128)
     assert lib.fca_split_workspace_bytes(ctypes.byref(plan), None, None) < 0
     plan = _lib.FcaSplitPlan(100, 8, 2, 128)
@@ -398,3 +412,22 @@ def test_padded_batch_is_gathered_attended_and_scattered():
         _close(name, got[valid.cuda()], ref, 1e-2)
     with pytest.raises(ValueError, match="valid tokens"):
         split_attention_padded(qd, kd, vd, torch.ones(tp, dtype=torch.bool, device="cuda"), SplitLayout(layout), 0.125)
+
+
+@pytest.mark.gpu
+def test_chunks_behind_a_context_attend_as_responses():
+    """responses_only: k and v hold context + chunk of every sequence, q only the chunks.
+    The rows equal the response rows of the full computation (the oracle), the context's own
+    attention is never formed."""
+    layout = [(70, [45]), (0, [33]), (200, [64]), (16, [1])]
+    hq, hkv, d = 8, 2, 128
+    scale = d**-0.5
+    q_all, k, v = _inputs(layout, hq, hkv, d, 5, torch.bfloat16)
+    ro, _ = oracle_split(q_all.double(), k.double(), v.double(), layout, scale)
+    L = SplitLayout(layout, responses_only=True)
+    rows = torch.tensor(L.q_index()[: L.num_tokens] >= 0)
+    assert int(rows.sum()) == L.num_query_rows == 143
+    out, _ = split_attention_forward(q_all[rows].cuda(), k.cuda(), v.cuda(), L, scale)
+    _close("out", out, ro[rows], 2e-2 / max(1.0, float(ro.abs().max())))
+    with pytest.raises(ValueError, match="forward only"):
+        split_attention_backward(out, out, k.cuda(), v.cuda(), out, out, L, scale)
