@@ -32,7 +32,7 @@ import json
 
 import torch
 
-from .cache import append_kv
+from .cache import append_kv, gather_kv
 from .config import ModelConfig, validate_fca_support
 from .forest import ForestMetadata, build_forest_metadata, rows_from_query_runs
 from .kv_layout import BLOCK_SIZE, kv_cache_shape
@@ -66,6 +66,9 @@ class ForestCascadeMetadata:
     # itself, straight from the step's own K and V
     fresh_prefill: SplitLayout | None = None
     fresh_start: int = 0  # first token of the fresh prompts; the tokens before it go through ``forest``
+    # when some of those prompts have a cached context: cache slots of context + chunk of each,
+    # in the layout's packed order; K and V are then gathered from the cache per layer
+    context_slots: torch.Tensor | None = None
 
 
 def parse_forest_cascade_configs(value) -> dict:
@@ -125,6 +128,10 @@ class ForestCascadeMetadataBuilder:
     # attention kernels (each prompt a group of its own): operands shared through LDS, about
     # twice the rate of the query-run path, which stays for everything that reads the cache
     FRESH_PREFILL_MIN_TOKENS = 256
+    # a prefill chunk behind a cached context joins them when it is at least this long: its
+    # context has to be gathered from the cache into packed rows first (several passes over
+    # the context's KV per layer), which only a long chunk pays back
+    CONTEXT_PREFILL_MIN_QUERY = 512
 
     def __init__(self, num_q_heads, num_kv_heads, head_dim, device="cuda", forest_cascade_attn_configs=None):
         cfg = parse_forest_cascade_configs(forest_cascade_attn_configs)
@@ -170,15 +177,27 @@ class ForestCascadeMetadataBuilder:
             q_lens = (m.query_start_loc_cpu[1 : m.num_reqs + 1] - m.query_start_loc_cpu[: m.num_reqs]).tolist()
             s_lens = m.seq_lens_cpu[: m.num_reqs].tolist()
             first = m.num_reqs
-            while first > 0 and q_lens[first - 1] == s_lens[first - 1] and q_lens[first - 1] > 1:
+            while first > 0 and q_lens[first - 1] > 1 and (
+                q_lens[first - 1] == s_lens[first - 1] or q_lens[first - 1] >= self.CONTEXT_PREFILL_MIN_QUERY
+            ):
                 first -= 1
             fresh = q_lens[first:]
+            context = [s - q for s, q in zip(s_lens[first:], fresh)]
             if sum(fresh) >= self.FRESH_PREFILL_MIN_TOKENS:
-                key = ("fresh", tuple(fresh))
+                key = ("fresh", tuple(fresh), tuple(context))
                 if key not in self._workspaces:
-                    self._keep(key, SplitLayout([(0, [n]) for n in fresh], device=self.device))
+                    if any(context):
+                        layout = SplitLayout([(c, [n]) for c, n in zip(context, fresh)], device=self.device, responses_only=True)
+                        req = torch.repeat_interleave(torch.arange(first, m.num_reqs), torch.tensor(s_lens[first:]))
+                        pos = torch.cat([torch.arange(n) for n in s_lens[first:]])
+                        self._keep(key, (layout, req.to(self.device), pos.to(self.device)))
+                    else:
+                        self._keep(key, (SplitLayout([(0, [n]) for n in fresh], device=self.device), None, None))
                 self._workspaces.move_to_end(key)
-                layout = self._workspaces[key]
+                layout, req, pos = self._workspaces[key]
+                slots = None
+                if req is not None:
+                    slots = m.block_table_tensor[req, pos // BLOCK_SIZE].to(torch.int64) * BLOCK_SIZE + pos % BLOCK_SIZE
                 total, before = sum(q_lens), sum(q_lens[:first])
                 rest = None
                 if first > 0:
@@ -190,7 +209,8 @@ class ForestCascadeMetadataBuilder:
                         ),
                     ).forest
                 return ForestCascadeMetadata(
-                    forest=rest, slot_mapping=m.slot_mapping[:total], num_decode_tokens=total, fresh_prefill=layout, fresh_start=before
+                    forest=rest, slot_mapping=m.slot_mapping[:total], num_decode_tokens=total, fresh_prefill=layout, fresh_start=before,
+                    context_slots=slots,
                 )
         if m.max_query_len > 1:
             # one row per query token: the row of its sequence, cut off behind the token itself;
@@ -283,12 +303,17 @@ class ForestCascadeAttentionImpl:
         if output is None:
             output = torch.empty_like(query)
         if attn_metadata.fresh_prefill is not None:
-            if key is None:
+            if key is None and attn_metadata.context_slots is None:
                 raise ValueError("a step with fresh prompts needs the step's key and value")
             f = attn_metadata.fresh_start
+            if attn_metadata.context_slots is not None:  # context and chunk alike, from the cache just filled
+                k_rows, v_rows = gather_kv(kv_cache, attn_metadata.context_slots, self.head_size, k_scale, v_scale)
+            else:
+                k_rows = key[f:t].view(t - f, self.num_kv_heads, self.head_size)
+                v_rows = value[f:t].view(t - f, self.num_kv_heads, self.head_size)
             split_attention_forward(
-                q[f:], key[f:t].view(t - f, self.num_kv_heads, self.head_size), value[f:t].view(t - f, self.num_kv_heads, self.head_size),
-                attn_metadata.fresh_prefill, self.scale, out=output[f:t].view(t - f, self.num_heads, self.head_size),
+                q[f:], k_rows, v_rows, attn_metadata.fresh_prefill, self.scale,
+                out=output[f:t].view(t - f, self.num_heads, self.head_size),
             )
             if f == 0:
                 return output

@@ -216,6 +216,8 @@ def test_fresh_prompts_take_the_split_attention_kernels(gpu):
     out2 = impl.forward(layer, q, None, None, cache, slow)
     torch.testing.assert_close(out2.view(T, hq, d).cpu().float(), ref, rtol=2e-2, atol=2e-2)
     # a cached context in front of the last sequence: no fresh prompts at the end of the batch
+    # (a chunk behind a context only joins them when it is long; ruled out here)
+    builder.CONTEXT_PREFILL_MIN_QUERY = 10**9
     longer = dataclasses.replace(common, seq_lens_cpu=torch.tensor([lens[0], lens[1], lens[2] + 16], dtype=torch.int32))
     assert builder.build(0, longer).fresh_prefill is None
     # in front of the first one: the two behind it are still taken as fresh prompts
@@ -264,3 +266,51 @@ def test_decodes_followed_by_fresh_prompts_in_one_step(gpu):
         q.view(T, hq, d).cpu(), cache.cpu(), table.cpu()[seq], (pos + 1).to(torch.int32), scale, dtype=torch.float32
     )
     torch.testing.assert_close(out.view(T, hq, d).cpu().float(), ref, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.gpu
+def test_long_chunk_behind_a_cached_context(gpu):
+    """Decodes, then a long prefill chunk whose sequence already has 130 tokens in the cache
+    (a cached prefix or an earlier chunk), then a fresh prompt: the two prompts attend on the
+    split-attention kernels with K and V gathered from the cache, context included."""
+    from arctic_platform_amd.kv_layout import kv_cache_shape
+    from oracle.attention import flat_decode_attention
+
+    hq, hkv, d = 8, 2, 128
+    scale = d**-0.5
+    gen = torch.Generator().manual_seed(22)
+    q_lens = [1, 1, 1, 600, 300]
+    s_lens = [50, 17, 200, 730, 300]
+    S, T = len(q_lens), sum(q_lens)
+    max_blocks = 48
+    table = torch.randperm(S * max_blocks, generator=gen).to(torch.int32).view(S, max_blocks).to(gpu)
+    cache = torch.randn(kv_cache_shape(S * max_blocks, 16, hkv, d), generator=gen).to(torch.bfloat16).to(gpu)
+    q, k, v = (torch.randn(T, h * d, generator=gen).to(torch.bfloat16).to(gpu) for h in (hq, hkv, hkv))
+    starts = torch.tensor([0] + q_lens).cumsum(0)
+    seq = torch.repeat_interleave(torch.arange(S), torch.tensor(q_lens))
+    pos = torch.cat([torch.arange(s - n, s) for n, s in zip(q_lens, s_lens)])
+    slots = (table.cpu().long()[seq, pos // 16] * 16 + pos % 16).to(gpu)
+    builder = ForestCascadeAttentionBackend.get_builder_cls()(hq, hkv, d, device=gpu)
+    impl = ForestCascadeAttentionBackend.get_impl_cls()(hq, d, scale, hkv)
+    layer = types.SimpleNamespace(k_scale=None, v_scale=None)
+    common = CommonAttentionMetadata(
+        query_start_loc=starts.to(torch.int32).to(gpu), seq_lens=torch.tensor(s_lens, dtype=torch.int32, device=gpu),
+        block_table_tensor=table, slot_mapping=slots, num_reqs=S, max_query_len=max(q_lens), num_actual_tokens=T,
+        query_start_loc_cpu=starts.to(torch.int32), seq_lens_cpu=torch.tensor(s_lens, dtype=torch.int32),
+    )
+    meta = builder.build(0, common)
+    assert meta.fresh_start == 3 and meta.context_slots is not None and meta.context_slots.numel() == 730 + 300
+    assert meta.fresh_prefill.responses_only and meta.fresh_prefill.num_query_rows == 900
+    out = impl.forward(layer, q, k, v, cache, meta)
+    torch.cuda.synchronize()
+    ref, _ = flat_decode_attention(
+        q.view(T, hq, d).cpu(), cache.cpu(), table.cpu()[seq], (pos + 1).to(torch.int32), scale, dtype=torch.float32
+    )
+    torch.testing.assert_close(out.view(T, hq, d).cpu().float(), ref, rtol=2e-2, atol=2e-2)
+    # a short chunk behind a context stays on the query-run path
+    short = CommonAttentionMetadata(
+        query_start_loc=torch.tensor([0, 100], dtype=torch.int32, device=gpu), seq_lens=torch.tensor([730], dtype=torch.int32, device=gpu),
+        block_table_tensor=table[3:4], slot_mapping=slots[:100], num_reqs=1, max_query_len=100, num_actual_tokens=100,
+        query_start_loc_cpu=torch.tensor([0, 100], dtype=torch.int32), seq_lens_cpu=torch.tensor([730], dtype=torch.int32),
+    )
+    assert builder.build(0, short).fresh_prefill is None
