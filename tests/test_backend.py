@@ -269,7 +269,8 @@ def test_decodes_followed_by_fresh_prompts_in_one_step(gpu):
 
 
 @pytest.mark.gpu
-def test_long_chunk_behind_a_cached_context(gpu):
+@pytest.mark.parametrize("kv_dtype", [torch.bfloat16, torch.float8_e4m3fn])
+def test_long_chunk_behind_a_cached_context(gpu, kv_dtype):
     """Decodes, then a long prefill chunk whose sequence already has 130 tokens in the cache
     (a cached prefix or an earlier chunk), then a fresh prompt: the two prompts attend on the
     split-attention kernels with K and V gathered from the cache, context included."""
@@ -284,15 +285,18 @@ def test_long_chunk_behind_a_cached_context(gpu):
     S, T = len(q_lens), sum(q_lens)
     max_blocks = 48
     table = torch.randperm(S * max_blocks, generator=gen).to(torch.int32).view(S, max_blocks).to(gpu)
-    cache = torch.randn(kv_cache_shape(S * max_blocks, 16, hkv, d), generator=gen).to(torch.bfloat16).to(gpu)
+    cache = torch.randn(kv_cache_shape(S * max_blocks, 16, hkv, d), generator=gen).to(kv_dtype).to(gpu)
     q, k, v = (torch.randn(T, h * d, generator=gen).to(torch.bfloat16).to(gpu) for h in (hq, hkv, hkv))
     starts = torch.tensor([0] + q_lens).cumsum(0)
     seq = torch.repeat_interleave(torch.arange(S), torch.tensor(q_lens))
     pos = torch.cat([torch.arange(s - n, s) for n, s in zip(q_lens, s_lens)])
     slots = (table.cpu().long()[seq, pos // 16] * 16 + pos % 16).to(gpu)
     builder = ForestCascadeAttentionBackend.get_builder_cls()(hq, hkv, d, device=gpu)
-    impl = ForestCascadeAttentionBackend.get_impl_cls()(hq, d, scale, hkv)
-    layer = types.SimpleNamespace(k_scale=None, v_scale=None)
+    fp8 = kv_dtype == torch.float8_e4m3fn
+    impl = ForestCascadeAttentionBackend.get_impl_cls()(hq, d, scale, hkv, kv_cache_dtype="fp8" if fp8 else "auto")
+    ks = torch.tensor([0.9, 1.3], device=gpu) if fp8 else None
+    vs = torch.tensor([1.1, 0.7], device=gpu) if fp8 else None
+    layer = types.SimpleNamespace(k_scale=ks, v_scale=vs)
     common = CommonAttentionMetadata(
         query_start_loc=starts.to(torch.int32).to(gpu), seq_lens=torch.tensor(s_lens, dtype=torch.int32, device=gpu),
         block_table_tensor=table, slot_mapping=slots, num_reqs=S, max_query_len=max(q_lens), num_actual_tokens=T,
@@ -304,7 +308,8 @@ def test_long_chunk_behind_a_cached_context(gpu):
     out = impl.forward(layer, q, k, v, cache, meta)
     torch.cuda.synchronize()
     ref, _ = flat_decode_attention(
-        q.view(T, hq, d).cpu(), cache.cpu(), table.cpu()[seq], (pos + 1).to(torch.int32), scale, dtype=torch.float32
+        q.view(T, hq, d).cpu(), cache.cpu(), table.cpu()[seq], (pos + 1).to(torch.int32), scale,
+        None if ks is None else ks.cpu(), None if vs is None else vs.cpu(), dtype=torch.float32,
     )
     torch.testing.assert_close(out.view(T, hq, d).cpu().float(), ref, rtol=2e-2, atol=2e-2)
     # a short chunk behind a context stays on the query-run path
