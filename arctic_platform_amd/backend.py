@@ -153,6 +153,7 @@ class ForestCascadeMetadataBuilder:
         if group > self.rows_per_item:
             raise ValueError(f"{group} query heads per KV head do not fit rows_per_item={self.rows_per_item}")
         self._workspaces: collections.OrderedDict = collections.OrderedDict()
+        self._split_scratch: dict = {}  # shared by the layouts of prompt steps, which change every step
         self._steps_since_build: dict = {}
 
     def _keep(self, key, value):
@@ -187,12 +188,15 @@ class ForestCascadeMetadataBuilder:
                 key = ("fresh", tuple(fresh), tuple(context))
                 if key not in self._workspaces:
                     if any(context):
-                        layout = SplitLayout([(c, [n]) for c, n in zip(context, fresh)], device=self.device, responses_only=True)
+                        layout = SplitLayout(
+                            [(c, [n]) for c, n in zip(context, fresh)], device=self.device, responses_only=True,
+                            scratch_pool=self._split_scratch,
+                        )
                         req = torch.repeat_interleave(torch.arange(first, m.num_reqs), torch.tensor(s_lens[first:]))
                         pos = torch.cat([torch.arange(n) for n in s_lens[first:]])
                         self._keep(key, (layout, req.to(self.device), pos.to(self.device)))
                     else:
-                        self._keep(key, (SplitLayout([(0, [n]) for n in fresh], device=self.device), None, None))
+                        self._keep(key, (SplitLayout([(0, [n]) for n in fresh], device=self.device, scratch_pool=self._split_scratch), None, None))
                 self._workspaces.move_to_end(key)
                 layout, req, pos = self._workspaces[key]
                 slots = None

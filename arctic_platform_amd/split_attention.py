@@ -31,8 +31,10 @@ def _stream_ptr(device) -> int:
 class SplitLayout:
     """Token layout of one deduplicated batch: ``[(prompt_tokens, [response_tokens, ...]), ...]``."""
 
-    def __init__(self, groups, device="cuda", responses_only=False):
-        """``responses_only`` (forward only): ``k`` and ``v`` hold every token, ``q`` and ``out`` only
+    def __init__(self, groups, device="cuda", responses_only=False, scratch_pool=None):
+        """``scratch_pool``: a dict shared by layouts whose calls run one after the other on one
+        stream (the adapter makes a layout per step), so that they share their scratch buffers.
+        ``responses_only`` (forward only): ``k`` and ``v`` hold every token, ``q`` and ``out`` only
         the response rows, in packed order, and the prompts' own attention is not computed (a
         prefill chunk behind a cached context, with the context as the prompt)."""
         self.groups = [(int(p), [int(n) for n in rs]) for p, rs in groups]
@@ -55,7 +57,7 @@ class SplitLayout:
         )
         self.device = torch.device(device)
         self.dev = torch.from_numpy(self.host).to(self.device) if self.device.type == "cuda" else None
-        self._scratch = {}
+        self._scratch = {} if scratch_pool is None else scratch_pool
 
     @classmethod
     def from_group_token_layout(cls, layout, device="cuda"):
