@@ -16,6 +16,7 @@ CSRC_DIR = os.path.join(_HERE, "csrc")
 
 FCA_BF16, FCA_FP8_E4M3, FCA_F32 = 0, 1, 2
 FCA_MAX_LEVELS = 8
+FCA_STATIC_SCRATCH_BYTES = 40 << 20
 
 EXPORTS = (
     "fca_version",
@@ -31,6 +32,7 @@ EXPORTS = (
     "fca_forest_pass",
     "fca_merge",
     "fca_decode_step",
+    "fca_decode_step_static",
     "fca_append_kv",
     "fca_gather_kv",
     "fca_calibration_copy",
@@ -157,6 +159,7 @@ def load_library() -> ctypes.CDLL:
     lib.fca_forest_pass.argtypes = attend
     lib.fca_merge.argtypes = [P(FcaPlan), VP, VP, VP, VP, I64, I64, I32, VP, VP]
     lib.fca_decode_step.argtypes = [P(FcaPlan), P(FcaTensors), VP, VP, VP, VP, I64, I64, I32, VP, VP]
+    lib.fca_decode_step_static.argtypes = [P(FcaPlan), P(FcaTensors), VP, VP, I64, I64, I32, VP, VP]
     lib.fca_append_kv.argtypes = [VP, VP, I64, I64, I32, I32, I32, VP, VP, VP, I64, I64, I32, VP, VP, VP]
     lib.fca_gather_kv.argtypes = lib.fca_append_kv.argtypes
     lib.fca_calibration_copy.argtypes = [VP, VP, ctypes.c_size_t, VP]

@@ -2,6 +2,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "fca_common.h"
 
@@ -271,6 +272,62 @@ int fca_decode_step(const fca_plan* plan, const fca_tensors* t, void* meta_dev, 
   if (int rc = run_attend(plan, t, meta_dev, partial_out_dev, partial_lse_dev, 0, stream)) return rc;
   return run_merge(plan, meta_dev, partial_out_dev, partial_lse_dev, out_dev, out_seq_stride, out_head_stride, out_dtype,
                    lse_dev, stream);
+}
+
+}  // extern "C"
+
+// ---- decode step on the library's own partial buffers ----------------------------------
+// The partial rows of fca_decode_step_static live in this array instead of caller memory.
+// Every GPU the library runs on holds its own copy at its own address; host code may only
+// use the address hipGetSymbolAddress reports for the current device, never the name.
+static __device__ __align__(256) unsigned char scratch[FCA_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];  // device address of `scratch`, per device, once looked up
+std::mutex g_scratch_mutex;
+
+// Address of the current device's copy of `scratch` (looked up on the first call per device).
+int static_scratch(unsigned char** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+  if (dev < 0 || dev >= kMaxDevices) return fail(FCA_ERR_UNSUPPORTED, "device ordinal %d is beyond %d", dev, kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    if (!p || (reinterpret_cast<uintptr_t>(p) & 255)) return fail(FCA_ERR_HIP, "static scratch has no usable device address");
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = static_cast<unsigned char*>(g_scratch_ptr[dev]);
+  return FCA_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int fca_decode_step_static(const fca_plan* plan, const fca_tensors* t, void* meta_dev, void* out_dev,
+                           int64_t out_seq_stride, int64_t out_head_stride, int32_t out_dtype, float* lse_dev,
+                           void* stream) {
+  size_t po = 0, pl = 0;
+  if (int rc = fca_workspace_bytes(plan, nullptr, &po, &pl)) return rc;
+  const size_t lse_at = (po + 255) / 256 * 256;
+  if (lse_at + pl > (size_t)FCA_STATIC_SCRATCH_BYTES)
+    return fail(FCA_ERR_UNSUPPORTED,
+                "the partial rows of this plan need %zu bytes, the static scratch holds %zu: use fca_decode_step with "
+                "caller-owned partial buffers (or a larger chunk_tokens / fewer sequences)",
+                lse_at + pl, (size_t)FCA_STATIC_SCRATCH_BYTES);
+  unsigned char* base = nullptr;
+  if (int rc = static_scratch(&base)) return rc;
+  // Every partial slot the merge reads (ord < partial count of its sequence) is written by
+  // the attention launch of the same call, so nothing of the last call's contents is read.
+  void* partial_out = base;
+  float* partial_lse = reinterpret_cast<float*>(base + lse_at);
+  if (int rc = run_attend(plan, t, meta_dev, partial_out, partial_lse, 0, stream)) return rc;
+  return run_merge(plan, meta_dev, partial_out, partial_lse, out_dev, out_seq_stride, out_head_stride, out_dtype, lse_dev,
+                   stream);
 }
 
 static int cache_rows(bool gather, const void* key_dev, const void* value_dev, int64_t token_stride, int64_t head_stride,

@@ -108,6 +108,26 @@ def forest_cascade_decode(
     return (out, lse) if return_lse else out
 
 
+def forest_cascade_decode_static(q, kv_cache, meta: ForestMetadata, scale, k_scale=None, v_scale=None, *, out, lse=None):
+    """``forest_cascade_decode`` on the library's own partial buffers
+    (``fca_decode_step_static``): nothing is allocated, so ``out`` (and ``lse`` if wanted)
+    must be passed in, and ``meta.partial_out`` / ``meta.partial_lse`` are not touched.
+    Plans whose partial rows exceed ``_lib.FCA_STATIC_SCRATCH_BYTES`` raise.  All calls on
+    one GPU share the buffers: keep them in stream order."""
+    lib = _lib.load_library()
+    t = _tensors(q, kv_cache, meta, scale, k_scale, v_scale)
+    out, code = _out_args(q, meta, out, None)
+    if lse is not None and (lse.dtype != torch.float32 or lse.shape != (meta.plan.num_seqs, meta.plan.num_q_heads) or not lse.is_contiguous()):
+        raise ValueError("lse must be a contiguous fp32 tensor [num_seqs, num_q_heads]")
+    _lib.check(
+        lib.fca_decode_step_static(
+            ctypes.byref(meta.plan), ctypes.byref(t), meta.meta.data_ptr(), out.data_ptr(), out.stride(0), out.stride(1),
+            code, lse.data_ptr() if lse is not None else None, _stream_ptr(q.device),
+        )
+    )
+    return out if lse is None else (out, lse)
+
+
 def prefix_pass(q, kv_cache, meta: ForestMetadata, scale, k_scale=None, v_scale=None):
     """Shared-node work items only; fills their slots of the partial buffers."""
     lib = _lib.load_library()

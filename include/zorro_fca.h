@@ -217,6 +217,22 @@ int fca_decode_step(const fca_plan* plan, const fca_tensors* t, void* meta_dev,
                     void* partial_out_dev, float* partial_lse_dev, void* out_dev, int64_t out_seq_stride,
                     int64_t out_head_stride, int32_t out_dtype, float* lse_dev, void* stream);
 
+/* fca_decode_step for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the partial rows live in
+ * a file-scope device array of FCA_STATIC_SCRATCH_BYTES inside the library instead of
+ * caller-owned partial buffers, and the call allocates nothing.  No counterpart in the
+ * reference.  The caller still passes q, the cache, the built metadata workspace and out.
+ * Plans whose partial buffers (fca_workspace_bytes) do not fit are refused with
+ * FCA_ERR_UNSUPPORTED.  Results are those of fca_decode_step bit for bit.  Each GPU holds
+ * one such array from the first call on it until the process ends, and every call on a GPU
+ * uses it: calls that overlap in time on one GPU (two streams, two threads) race; stream
+ * order is enough.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress); make that call outside graph capture. */
+#define FCA_STATIC_SCRATCH_BYTES (40u << 20)
+int fca_decode_step_static(const fca_plan* plan, const fca_tensors* t, void* meta_dev, void* out_dev,
+                           int64_t out_seq_stride, int64_t out_head_stride, int32_t out_dtype, float* lse_dev,
+                           void* stream);
+
 /* KV-cache append, the step before decode attention in every layer: scatter the new
  * tokens' K and V (bf16 [T, Hkv, D]) into the cache tiles at slot = block * 16 + offset
  * (negative slot = padding, skipped), quantising to fp8 e4m3 with per-KV-head scales
