@@ -124,6 +124,11 @@ class ForestCascadeMetadataBuilder:
     (a new request with a cached prompt) is picked up."""
 
     MAX_KEPT_WORKSPACES = 16
+    MAX_KEPT_BYTES = 8 << 30  # device memory of the kept forest workspaces (partial rows dominate)
+    # layouts of prompt steps are keyed by the exact token counts of a step, so nearly every
+    # prefill step makes a new one: they live in a small store of their own and never push a
+    # decode shape's workspaces out
+    MAX_KEPT_LAYOUTS = 8
     # a step of fresh prompts with at least this many tokens runs on the trainer's split
     # attention kernels (each prompt a group of its own): operands shared through LDS, about
     # twice the rate of the query-run path, which stays for everything that reads the cache
@@ -153,15 +158,25 @@ class ForestCascadeMetadataBuilder:
         if group > self.rows_per_item:
             raise ValueError(f"{group} query heads per KV head do not fit rows_per_item={self.rows_per_item}")
         self._workspaces: collections.OrderedDict = collections.OrderedDict()
+        self._layouts: collections.OrderedDict = collections.OrderedDict()
         self._split_scratch: dict = {}  # shared by the layouts of prompt steps, which change every step
         self._steps_since_build: dict = {}
 
+    @staticmethod
+    def _bytes_of(value) -> int:
+        if isinstance(value, ForestMetadata):
+            return sum(t.numel() * t.element_size() for t in (value.meta, value.partial_out, value.partial_lse))
+        return 0
+
     def _keep(self, key, value):
-        """Remember a workspace; forget the least recently used ones beyond the cap."""
+        """Remember a workspace; forget the least recently used ones beyond the cap on their
+        number and on the device memory they hold (the one just stored always stays)."""
         self._workspaces[key] = value
         self._workspaces.move_to_end(key)
-        while len(self._workspaces) > self.MAX_KEPT_WORKSPACES:
-            old, _ = self._workspaces.popitem(last=False)
+        held = sum(self._bytes_of(v) for v in self._workspaces.values())
+        while len(self._workspaces) > 1 and (len(self._workspaces) > self.MAX_KEPT_WORKSPACES or held > self.MAX_KEPT_BYTES):
+            old, gone = self._workspaces.popitem(last=False)
+            held -= self._bytes_of(gone)
             self._steps_since_build.pop(old, None)
 
     def build(self, common_prefix_len: int, common_attn_metadata: CommonAttentionMetadata) -> ForestCascadeMetadata:
@@ -170,6 +185,18 @@ class ForestCascadeMetadataBuilder:
             raise ValueError(f"max_query_len must be at least 1, got {m.max_query_len}")
         bt, sl = m.block_table_tensor[: m.num_reqs], m.seq_lens[: m.num_reqs]
         num_tokens = m.num_reqs
+        if m.seq_lens_cpu is not None:
+            # the device builder can only flag bad lengths in its header; with the engine's host
+            # copy at hand they are refused here, before anything is launched
+            lens = m.seq_lens_cpu[: m.num_reqs]
+            if int(lens.min()) < 0 or int(lens.max()) > bt.shape[1] * BLOCK_SIZE:
+                raise ValueError(
+                    f"seq_lens must lie in [0, max_blocks * {BLOCK_SIZE} = {bt.shape[1] * BLOCK_SIZE}], got [{int(lens.min())}, {int(lens.max())}]"
+                )
+            if m.query_start_loc_cpu is not None:
+                ql = m.query_start_loc_cpu[1 : m.num_reqs + 1] - m.query_start_loc_cpu[: m.num_reqs]
+                if int(ql.min()) < 0 or bool((ql > lens).any()):
+                    raise ValueError("every request's query length must lie in [0, seq_len]")
         row_table = row_group = None
         if m.max_query_len > 1 and m.query_start_loc_cpu is not None and m.seq_lens_cpu is not None and self.enabled:
             # The requests at the end of the batch that are fresh prompts (the engine puts decodes
@@ -185,23 +212,30 @@ class ForestCascadeMetadataBuilder:
             fresh = q_lens[first:]
             context = [s - q for s, q in zip(s_lens[first:], fresh)]
             if sum(fresh) >= self.FRESH_PREFILL_MIN_TOKENS:
-                key = ("fresh", tuple(fresh), tuple(context))
-                if key not in self._workspaces:
+                # Kept per (query, context) lengths: the layout and, for prompts behind a context,
+                # the position of every packed token and its request counted from the first of
+                # these prompts.  The number of requests in front of them is not part of the key,
+                # so it is added when the slots are computed.
+                key = (tuple(fresh), tuple(context))
+                if key not in self._layouts:
                     if any(context):
                         layout = SplitLayout(
                             [(c, [n]) for c, n in zip(context, fresh)], device=self.device, responses_only=True,
                             scratch_pool=self._split_scratch,
                         )
-                        req = torch.repeat_interleave(torch.arange(first, m.num_reqs), torch.tensor(s_lens[first:]))
+                        rel = torch.repeat_interleave(torch.arange(len(fresh)), torch.tensor(s_lens[first:]))
                         pos = torch.cat([torch.arange(n) for n in s_lens[first:]])
-                        self._keep(key, (layout, req.to(self.device), pos.to(self.device)))
+                        entry = (layout, rel.to(self.device), pos.to(self.device))
                     else:
-                        self._keep(key, (SplitLayout([(0, [n]) for n in fresh], device=self.device, scratch_pool=self._split_scratch), None, None))
-                self._workspaces.move_to_end(key)
-                layout, req, pos = self._workspaces[key]
+                        entry = (SplitLayout([(0, [n]) for n in fresh], device=self.device, scratch_pool=self._split_scratch), None, None)
+                    self._layouts[key] = entry
+                    while len(self._layouts) > self.MAX_KEPT_LAYOUTS:
+                        self._layouts.popitem(last=False)
+                self._layouts.move_to_end(key)
+                layout, rel, pos = self._layouts[key]
                 slots = None
-                if req is not None:
-                    slots = m.block_table_tensor[req, pos // BLOCK_SIZE].to(torch.int64) * BLOCK_SIZE + pos % BLOCK_SIZE
+                if rel is not None:
+                    slots = m.block_table_tensor[rel + first, pos // BLOCK_SIZE].to(torch.int64) * BLOCK_SIZE + pos % BLOCK_SIZE
                 total, before = sum(q_lens), sum(q_lens[:first])
                 rest = None
                 if first > 0:

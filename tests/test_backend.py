@@ -52,6 +52,92 @@ def test_workspace_cache_is_bounded():
     assert list(b._workspaces)[0] == 2 * b.MAX_KEPT_WORKSPACES  # the oldest went first
 
 
+def test_workspace_cache_is_bounded_by_bytes():
+    from arctic_platform_amd.forest import ForestMetadata
+
+    b = ForestCascadeMetadataBuilder(32, 8, 128, device="cpu")
+    b.MAX_KEPT_BYTES = 3000
+
+    def fake(n):
+        return ForestMetadata(None, None, torch.zeros(n, dtype=torch.int32), torch.zeros(0), torch.zeros(0), None, None)
+
+    for i in range(5):
+        b._keep(i, fake(250))  # 1000 bytes each
+    assert list(b._workspaces) == [2, 3, 4]
+    b._keep("big", fake(5000))  # beyond the cap on its own: everything else goes, it stays
+    assert list(b._workspaces) == ["big"]
+
+
+def test_prompt_layouts_never_evict_forest_workspaces(monkeypatch):
+    import arctic_platform_amd.backend as backend
+
+    b = ForestCascadeMetadataBuilder(8, 2, 128, device="cpu")
+    b._keep("decode-shape", object())
+    for n in range(300, 300 + 3 * b.MAX_KEPT_LAYOUTS):
+        starts = torch.tensor([0, n], dtype=torch.int32)
+        lens = torch.tensor([n], dtype=torch.int32)
+        common = CommonAttentionMetadata(
+            starts, lens, torch.zeros(1, 64, dtype=torch.int32), torch.zeros(n, dtype=torch.int64), num_reqs=1, max_query_len=n,
+            num_actual_tokens=n, query_start_loc_cpu=starts, seq_lens_cpu=lens,
+        )
+        assert b.build(0, common).fresh_prefill is not None
+    assert "decode-shape" in b._workspaces and len(b._layouts) == b.MAX_KEPT_LAYOUTS
+
+
+def test_cached_prompt_layout_follows_the_number_of_decodes_in_front(monkeypatch):
+    """Two steps with the same (query, context) lengths of their prompts but a different
+    number of decode requests in front: the cache slots of the context must come from the
+    prompt's own block-table row both times."""
+    import arctic_platform_amd.backend as backend
+
+    monkeypatch.setattr(backend, "build_forest_metadata", lambda *a, **k: None)
+    monkeypatch.setattr(backend, "rows_from_query_runs", lambda *a, **k: (None, None, None))
+    b = ForestCascadeMetadataBuilder(8, 2, 128, device="cpu")
+    max_blocks = 128
+    table = torch.arange(2 * max_blocks, dtype=torch.int32).view(2, max_blocks)
+
+    def step(q_lens, s_lens):
+        n = len(q_lens)
+        starts = torch.tensor([0] + q_lens, dtype=torch.int32).cumsum(0).to(torch.int32)
+        lens = torch.tensor(s_lens, dtype=torch.int32)
+        common = CommonAttentionMetadata(
+            starts, lens, table[:n], torch.zeros(sum(q_lens), dtype=torch.int64), num_reqs=n, max_query_len=max(q_lens),
+            num_actual_tokens=sum(q_lens), query_start_loc_cpu=starts, seq_lens_cpu=lens,
+        )
+        return b.build(0, common)
+
+    for q_lens, s_lens in (([512], [1536]), ([1, 512], [40, 1536]), ([512], [1536])):
+        meta = step(q_lens, s_lens)
+        first = len(q_lens) - 1
+        assert meta.fresh_start == sum(q_lens[:first])
+        pos = torch.arange(1536)
+        want = table[first, pos // 16].long() * 16 + pos % 16
+        assert torch.equal(meta.context_slots, want), q_lens
+    assert len(b._layouts) == 1  # one layout served all three steps
+
+
+def test_lengths_beyond_the_block_table_are_refused_on_the_host():
+    b = ForestCascadeMetadataBuilder(8, 2, 128, device="cpu")
+    starts = torch.tensor([0, 1, 2], dtype=torch.int32)
+    table = torch.zeros(2, 4, dtype=torch.int32)
+    for lens in ([10, 65], [-1, 5]):
+        lens = torch.tensor(lens, dtype=torch.int32)
+        common = CommonAttentionMetadata(
+            starts, lens, table, torch.zeros(2, dtype=torch.int64), num_reqs=2, max_query_len=1,
+            query_start_loc_cpu=starts, seq_lens_cpu=lens,
+        )
+        with pytest.raises(ValueError, match="seq_lens must lie in"):
+            b.build(0, common)
+    lens = torch.tensor([10, 20], dtype=torch.int32)
+    starts = torch.tensor([0, 11, 12], dtype=torch.int32)
+    common = CommonAttentionMetadata(
+        starts, lens, table, torch.zeros(12, dtype=torch.int64), num_reqs=2, max_query_len=11,
+        query_start_loc_cpu=starts, seq_lens_cpu=lens,
+    )
+    with pytest.raises(ValueError, match="query length"):
+        b.build(0, common)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("index", [2, 5])
 def test_decode_loop_through_backend(gpu, index):
