@@ -16,7 +16,7 @@ CSRC_DIR = os.path.join(_HERE, "csrc")
 
 FCA_BF16, FCA_FP8_E4M3, FCA_F32 = 0, 1, 2
 FCA_MAX_LEVELS = 8
-FCA_STATIC_SCRATCH_BYTES = 40 << 20
+FCA_STATIC_SCRATCH_BYTES = 48 << 20
 
 EXPORTS = (
     "fca_version",
@@ -107,6 +107,7 @@ class FcaMetaLayout(ctypes.Structure):
             "total_int32",
             "node_tok",
             "node_causal",
+            "coop_ctr",
         )
     ]
 

@@ -98,6 +98,9 @@ fca::AttendParams attend_params(const fca_plan* p, const fca_tensors* t, void* m
   a.max_partials = (int32_t)L.max_partials;
   a.select = select;
   a.kv_reread = t->kv_reread;
+  a.coop_ctr = a.meta + L.coop_ctr;
+  a.coop_pairs = (int32_t)fca::coop_pairs_for(*p, L);
+  a.coop_row0 = (int64_t)p->num_seqs * L.max_partials * p->num_q_heads;
   return a;
 }
 
@@ -122,6 +125,7 @@ int run_merge(const fca_plan* p, const void* meta, const void* po, const float* 
     return fail(FCA_ERR_INVALID_ARG, "partial workspaces must be 16-byte aligned");
   const fca::MetaLayout L = fca::make_layout(*p);
   fca::MergeParams m{};
+  m.header = static_cast<const int32_t*>(meta) + L.header;
   m.seq_npart = static_cast<const int32_t*>(meta) + L.seq_npart;
   m.partial_out = po;
   m.partial_lse = pl;
@@ -133,6 +137,7 @@ int run_merge(const fca_plan* p, const void* meta, const void* po, const float* 
   m.num_q_heads = p->num_q_heads;
   m.head_dim = p->head_dim;
   m.max_partials = (int32_t)L.max_partials;
+  m.coop_row0 = (int64_t)p->num_seqs * L.max_partials * p->num_q_heads;
   m.out_dtype = out_dtype;
   // whole 16-byte stores when every 8-channel group of out is 16-byte aligned
   const int64_t esz = out_dtype == FCA_F32 ? 4 : 2;
@@ -152,10 +157,11 @@ const char* fca_last_error(void) { return g_error; }
 int fca_workspace_bytes(const fca_plan* plan, size_t* meta_bytes, size_t* partial_out_bytes, size_t* partial_lse_bytes) {
   if (int rc = check_plan(plan)) return rc;
   const fca::MetaLayout L = fca::make_layout(*plan);
-  const size_t slots = (size_t)plan->num_seqs * (size_t)L.max_partials;
+  // one row per (partial slot, query head), then 32 rows per pair of waves that may share an item
+  const size_t rows = (size_t)plan->num_seqs * (size_t)L.max_partials * plan->num_q_heads + 32 * (size_t)fca::coop_pairs_for(*plan, L);
   if (meta_bytes) *meta_bytes = (size_t)L.total * sizeof(int32_t);
-  if (partial_out_bytes) *partial_out_bytes = slots * plan->num_q_heads * plan->head_dim * 2;  // half
-  if (partial_lse_bytes) *partial_lse_bytes = slots * plan->num_q_heads * 2 * sizeof(float);    // {lse, scale}
+  if (partial_out_bytes) *partial_out_bytes = rows * plan->head_dim * 2;  // half
+  if (partial_lse_bytes) *partial_lse_bytes = rows * 2 * sizeof(float);    // {lse, scale}
   return FCA_OK;
 }
 
@@ -180,6 +186,7 @@ int fca_meta_describe(const fca_plan* plan, fca_meta_layout* out) {
   out->total_int32 = L.total;
   out->node_tok = L.node_tok;
   out->node_causal = L.node_causal;
+  out->coop_ctr = L.coop_ctr;
   return FCA_OK;
 }
 

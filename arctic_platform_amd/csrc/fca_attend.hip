@@ -31,6 +31,7 @@
 // token) follow arctic_platform/model/implementations/qwen35/models/qwen3_5_moe/
 // modeling_qwen3_5_moe.py:368-373, :385, :440-454.
 #include <cstring>
+#include <cstdlib>
 #include <type_traits>
 
 #include "fca_attend_common.h"
@@ -448,6 +449,12 @@ hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dty
                               ((int64_t)plan.max_blocks * kBlock / plan.chunk_tokens + plan.max_levels + 2) *
                               plan.num_kv_heads;
   int grid = cached_cu_count() * workgroups_per_cu(plan.head_dim, fp8, plan.rows_per_item);
+  // FCA_ATTEND_WORKGROUPS caps the grid (tests use it to reach the many-items-per-wave
+  // schedules of a large batch with a small one)
+  if (const char* cap = getenv("FCA_ATTEND_WORKGROUPS")) {
+    const int n = atoi(cap);
+    if (n > 0 && n < grid) grid = n;
+  }
   if ((int64_t)grid * kWaves > max_tickets) grid = (int)((max_tickets + kWaves - 1) / kWaves);
   if (grid < 1) grid = 1;
   if (nrt == 1) return launch_attend32(p, plan, kv_dtype, grid, stream);

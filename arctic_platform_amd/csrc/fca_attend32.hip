@@ -11,6 +11,17 @@
 // with the next item's first tiles as soon as the current item's last tiles have been
 // consumed, exactly as they are refilled inside an item.
 //
+// The last item of a wave is shared with a wave of another XCD.  XCDs stream at different
+// speeds (the slowest takes about a sixth longer per tile than the fastest, and which is
+// which differs from box to box), and with a handful of items per wave, drawn four items
+// ahead of use, the draws come too early to tell a fast wave from a slow one.  So the
+// largest items of the list are set aside, one per pair of waves: both waves of a pair take
+// the item as their last, one from its first pair of tiles upwards, the other from its last
+// pair downwards, each claiming the next pair of tiles from a counter of the pair until the
+// claims meet.  Whichever wave arrives earlier or streams faster takes more of the item,
+// and each wave writes a partial of its own (the second one into rows set aside behind the
+// ordinary partial rows; the first one's row scale carries the second one's address).
+//
 // All loads sit at fixed places of the instruction stream (none inside a data-dependent
 // branch): the hardware counts outstanding vector memory operations in order and the
 // compiler picks each wait's count for the shortest path, so a load issued on only some
@@ -63,9 +74,25 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
   // list shorter than five rounds is dealt statically as a whole.  Every wave draws until
   // its first failing draw; the draw that returns the last possible value resets the
   // counter for the next launch.
-  const int static_tickets = ntickets < 5 * nwaves ? ntickets : (ntickets / nwaves - 1) * nwaves;
-  const int dynamic_draws = ntickets - static_tickets + nwaves;
-  bool drawing = static_tickets < ntickets;
+  // Cooperative last items: tickets [0, coop) are set aside, one per pair of waves; the rest
+  // of the list (nmain tickets, numbered from coop upwards) is dealt as described above.
+  // Workgroup b pairs with workgroup b ^ 3, which the dispatcher places on another XCD (an
+  // even one with an odd one, an outer one with an inner one); its wave w pairs with wave w
+  // there.  The lower half of each quad of workgroups takes its item from the front.
+  const int quad_pos = (int)blockIdx.x & 3;
+  const bool coop_back = quad_pos >= 2;
+  const int pair_id = (((int)blockIdx.x >> 2) * 2 + ((quad_pos == 1 || quad_pos == 2) ? 1 : 0)) * kWaves + wave;
+  // (not where two workgroups share a CU: the second wave per SIMD evens the speeds out, and
+  // the kernel has no registers to spare there)
+  constexpr bool COOP = workgroups_per_cu(D, FP8, 32) == 1;
+  const bool coop_on = COOP && p.coop_ctr != nullptr && (gridDim.x & 3) == 0 && nwaves / 2 <= p.coop_pairs &&
+                       ntickets >= nwaves / 2 + 3 * nwaves;
+  const int coop = coop_on ? nwaves / 2 : 0;
+  const int nmain = ntickets - coop;
+  const int static_tickets = nmain < 5 * nwaves ? nmain : (nmain / nwaves - 1) * nwaves;
+  const int dynamic_draws = nmain - static_tickets + nwaves;
+  bool drawing = static_tickets < nmain;
+  bool coop_pending = coop_on;
   // A zero the compiler cannot see through; it makes an address look lane-dependent.
   int opaque_zero;
   asm volatile("v_mov_b32 %0, 0" : "=v"(opaque_zero));
@@ -79,15 +106,27 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
     if (r * nwaves >= static_tickets && drawing && lane == 0)
       tv_drawn = atomicAdd(&hdr[H_TICKET + opaque_zero], 1);
   };
+  // what follows a wave's last ticket of the main list: its pair's item, then nothing
+  auto after_main = [&]() -> int {
+    if (!coop_pending) return ntickets;
+    coop_pending = false;
+    return pair_id;
+  };
   // ticket of round r; ntickets or more = none
   auto resolve_ticket = [&](int r) -> int {
-    if (r * nwaves < static_tickets) return r * nwaves + ((r & 1) ? nwaves - 1 - my_wave : my_wave);
-    if (!drawing) return ntickets;
+    if (r * nwaves < static_tickets) {
+      const int t = r * nwaves + ((r & 1) ? nwaves - 1 - my_wave : my_wave);
+      return t < nmain ? coop + t : after_main();
+    }
+    if (!drawing) return after_main();
     const int drawn = __builtin_amdgcn_readfirstlane(tv_drawn);
     if (drawn == dynamic_draws - 1 && lane == 0) hdr[H_TICKET] = 0;  // nobody draws after this one
     const int t = static_tickets + drawn;
-    if (t >= ntickets) drawing = false;
-    return t;
+    if (t >= nmain) {
+      drawing = false;
+      return after_main();
+    }
+    return coop + t;
   };
 
   // The opaque zero in the record address keeps the compiler from moving the record's
@@ -151,9 +190,10 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
   int4 r0, r1, a0, a1, b0, b1;  // records of the current item and the two after it
   int kvh, akvh, bkvh;
   int my_blk, seq, a_blk, a_seq;  // per-lane data of the current and the next item
-  int ta = resolve_ticket(1);  // rounds 0 to 3 are static, or the whole list is
+  int t_cur = resolve_ticket(0);  // rounds 0 to 3 are static, or the whole list is
+  int ta = resolve_ticket(1);
   int tb = resolve_ticket(2);
-  load_record(my_wave, r0, r1, kvh);
+  load_record(t_cur, r0, r1, kvh);
   load_record(ta, a0, a1, akvh);
   load_record(tb, b0, b1, bkvh);
   load_lane_meta(r0, r1, my_blk, seq);
@@ -185,16 +225,163 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
     load_tile(kb1, vb1, my_blk, nb, kvh, min(1, lt));
   }
 
+  // ---- state of the item being attended
+  struct Item {
+    int tok_len;  // KV tokens of the chunk
+    // Last chunk of a query-run tile: member i sees the first `sees + i` tokens of the chunk
+    // (its own token and what is before it).  All members end inside the last tile, which
+    // then takes the masking path even when the chunk fills it.
+    int sees;
+    f32x16 acc[NDB];
+    float mrow, lrow;  // reference maximum (scaled, log2 domain) and running sum
+    float sc;
+  };
+  auto begin_item = [&](Item& it) {
+    it.tok_len = __builtin_amdgcn_readfirstlane(r0.z);
+    it.sees = __builtin_amdgcn_readfirstlane(r1.w);
+    it.mrow = -INFINITY, it.lrow = 0.f;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) it.acc[db][r] = 0.f;
+    it.sc = p.scale * kLog2e;
+    if (FP8) it.sc *= k_scale;
+  };
+
+  // One 32-token tile.  RAGGED is the variant for the single tile that may run past the
+  // end of the chunk: it masks scores and zeroes V there; full tiles carry no mask code.
+  auto compute_tile = [&](Item& it, const KT& kt, const VT& vt, int ti, auto ragged) {
+    constexpr bool RAGGED = decltype(ragged)::value;
+    f32x16(&acc)[NDB] = it.acc;
+    float &mrow = it.mrow, &lrow = it.lrow;
+    const float sc = it.sc;
+    const int tok_len = it.tok_len, sees = it.sees;
+    const int tok0 = ti * kTile;
+    f32x16 sr;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sr[r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < KS; ++i) {
+      bf16x8 a;
+      if constexpr (FP8) {
+        const i32x4 w = kt.k[i >> 1];
+        a = (i & 1) ? fp8x8_to_bf16(w[2], w[3]) : fp8x8_to_bf16(w[0], w[1]);
+      } else {
+        a = __builtin_bit_cast(bf16x8, kt.k[i]);
+      }
+      sr = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[i], sr, 0, 0, 0);
+    }
+    // register r holds token 16 * (r / 8) + 8 * h + r % 8 of the tile
+    if constexpr (RAGGED) {
+      // every score register of a lane belongs to the lane's own query row
+      const int row_lim = sees > 0 ? min(tok_len, sees + row_member) : tok_len;
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (tok0 + 16 * (r >> 3) + 8 * h + (r & 7) >= row_lim) sr[r] = -INFINITY;
+    }
+    float mx = sr[0];
+#pragma unroll
+    for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sr[r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    // sc > 0, so the maximum of the scaled scores is the scaled maximum.  mrow is the
+    // reference the exponentials are taken against, not the exact running maximum: it
+    // moves (and the accumulators are rescaled) only when a row's maximum rises more than
+    // kRescaleSlack above it, so probabilities stay below 2^kRescaleSlack and the rescale,
+    // which touches every accumulator register, is rare.  The log-sum-exp m + log2(l)
+    // does not depend on the reference.
+    // The first tile sets the reference without a rescale (the accumulators are zero).
+    const float mtile = mx * sc;
+    if (ti == 0) mrow = mtile;
+    if (__builtin_amdgcn_readfirstlane(__any(mtile > mrow + kRescaleSlack))) {
+      const float mnew = fmaxf(mrow, mtile);
+      const float alpha = fast_exp2(mrow - mnew);
+      lrow *= alpha;
+      mrow = mnew;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[db][r] *= alpha;
+    }
+    const float mref = mrow;
+    float sum = 0.f;
+    bf16x8 pb[2];  // probabilities of the tile as B operands
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float e = fast_exp2(__builtin_fmaf(sr[r], sc, -mref));
+      sum += e;
+      pb[r >> 3][r & 7] = (__bf16)e;
+    }
+    lrow += sum;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      // tokens this lane feeds for this block: 8h .. 8h+7; on the ragged tile zero the
+      // ones past the end so stale cache contents (possibly NaN) cannot leak through 0 * x
+      const int nv = tok_len - (tok0 + 16 * blk + 8 * h);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) {
+        bf16x8 a;
+        if constexpr (FP8) {
+          // rows of channel blocks 2 * pair and 2 * pair + 1 sit in the lower and upper
+          // lane halves; the swap hands every lane its tokens 8h..8h+7 of both blocks:
+          // dwords 0,1 become the operand of block 2 * pair, dwords 2,3 of 2 * pair + 1
+          const i32x4 raw = vt.v[blk][db >> 1];
+          const auto s0 = __builtin_amdgcn_permlane32_swap((unsigned)raw[0], (unsigned)raw[2], false, false);
+          const auto s1 = __builtin_amdgcn_permlane32_swap((unsigned)raw[1], (unsigned)raw[3], false, false);
+          i32x2 w = {(int)s0[db & 1], (int)s1[db & 1]};
+          if constexpr (RAGGED) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              unsigned keep = 0;
+#pragma unroll
+              for (int b = 0; b < 4; ++b)
+                if (4 * j + b < nv) keep |= 0xffu << (8 * b);
+              w[j] &= keep;
+            }
+          }
+          a = fp8x8_to_bf16(w[0], w[1]);
+        } else {
+          i32x4 w = vt.v[blk][db];
+          if constexpr (RAGGED) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              unsigned keep = (2 * j < nv ? 0xffffu : 0u) | (2 * j + 1 < nv ? 0xffff0000u : 0u);
+              w[j] &= keep;
+            }
+          }
+          a = __builtin_bit_cast(bf16x8, w);
+        }
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[blk], acc[db], 0, 0, 0);
+      }
+    }
+  };
+
+  // Write the partial of the item just attended: rows of a live member go to `prow` (-1: dead
+  // row), `tag` rides in the mantissa of the stored row scale.  Every accumulator register of
+  // a lane belongs to the lane's own query row, so normalisation is per lane.  The rows then
+  // pass through a wave-private strip of LDS so that they leave as whole rows: stored
+  // straight from the accumulator layout a row goes out in sixteen pieces, and back-to-back
+  // partial writes to one cache line cost a wave several microseconds per item.
+  auto write_partial = [&](Item& it, int64_t prow, int live_rows, int tag) {
+    const float vs = FP8 ? v_scale : 1.f;
+    const float l = it.lrow + __shfl_xor(it.lrow, 32);
+    // an item half of which nobody attended here (the other wave of the pair took all of it)
+    // leaves an empty partial: log-sum-exp -inf, weight 0 in the merge
+    const float inv = l > 0.f ? vs / l : 0.f;
+    stage_partial_row<D>(strip, m, h, it.acc, inv, prow, (it.mrow + fast_log2(l)) * kLn2, p.partial_lse, tag);
+    __builtin_amdgcn_wave_barrier();
+    store_partial_rows<D, STREAM>(strip, live_rows, lane, p.partial_out);
+    __builtin_amdgcn_wave_barrier();
+  };
+
+  bool to_pair_item = false;
   for (int round = 0;; ++round) {
-    const int tok_len = __builtin_amdgcn_readfirstlane(r0.z);
+    Item it;
+    begin_item(it);
+    const int tok_len = it.tok_len, sees = it.sees;
     const int mcnt = __builtin_amdgcn_readfirstlane(r1.x);
     const int ord = __builtin_amdgcn_readfirstlane(r1.y);
     const int nblk = (tok_len + kBlock - 1) / kBlock;
     const int ntiles = (tok_len + kTile - 1) / kTile;
-    // Last chunk of a query-run tile: member i sees the first `sees + i` tokens of the chunk
-    // (its own token and what is before it).  All members end inside the last tile, which
-    // then takes the masking path even when the chunk fills it.
-    const int sees = __builtin_amdgcn_readfirstlane(r1.w);
     const int nfull = (tok_len - (sees > 0 ? 1 : 0)) / kTile;  // tiles without masking; at most one masked tile follows
     const int last = ntiles - 1;
     const int npairs = (ntiles + 1) >> 1;
@@ -205,127 +392,20 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
     const int a_len = __builtin_amdgcn_readfirstlane(a0.z);
     const int a_nblk = (a_len + kBlock - 1) / kBlock;
     const int a_last = (a_len + kTile - 1) / kTile - 1;
-
-    f32x16 acc[NDB];
-    float mrow = -INFINITY, lrow = 0.f;  // reference maximum (scaled, log2 domain) and running sum
-#pragma unroll
-    for (int db = 0; db < NDB; ++db)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
-    float sc = p.scale * kLog2e;
-    if (FP8) sc *= k_scale;
-
-    // One 32-token tile.  RAGGED is the variant for the single tile that may run past the
-    // end of the chunk: it masks scores and zeroes V there; full tiles carry no mask code.
-    auto compute_tile = [&](const KT& kt, const VT& vt, int ti, auto ragged) {
-      constexpr bool RAGGED = decltype(ragged)::value;
-      const int tok0 = ti * kTile;
-      f32x16 sr;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sr[r] = 0.f;
-#pragma unroll
-      for (int i = 0; i < KS; ++i) {
-        bf16x8 a;
-        if constexpr (FP8) {
-          const i32x4 w = kt.k[i >> 1];
-          a = (i & 1) ? fp8x8_to_bf16(w[2], w[3]) : fp8x8_to_bf16(w[0], w[1]);
-        } else {
-          a = __builtin_bit_cast(bf16x8, kt.k[i]);
-        }
-        sr = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[i], sr, 0, 0, 0);
-      }
-      // register r holds token 16 * (r / 8) + 8 * h + r % 8 of the tile
-      if constexpr (RAGGED) {
-        // every score register of a lane belongs to the lane's own query row
-        const int row_lim = sees > 0 ? min(tok_len, sees + row_member) : tok_len;
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          if (tok0 + 16 * (r >> 3) + 8 * h + (r & 7) >= row_lim) sr[r] = -INFINITY;
-      }
-      float mx = sr[0];
-#pragma unroll
-      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sr[r]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
-      // sc > 0, so the maximum of the scaled scores is the scaled maximum.  mrow is the
-      // reference the exponentials are taken against, not the exact running maximum: it
-      // moves (and the accumulators are rescaled) only when a row's maximum rises more than
-      // kRescaleSlack above it, so probabilities stay below 2^kRescaleSlack and the rescale,
-      // which touches every accumulator register, is rare.  The log-sum-exp m + log2(l)
-      // does not depend on the reference.
-      // The first tile sets the reference without a rescale (the accumulators are zero).
-      const float mtile = mx * sc;
-      if (ti == 0) mrow = mtile;
-      if (__builtin_amdgcn_readfirstlane(__any(mtile > mrow + kRescaleSlack))) {
-        const float mnew = fmaxf(mrow, mtile);
-        const float alpha = fast_exp2(mrow - mnew);
-        lrow *= alpha;
-        mrow = mnew;
-#pragma unroll
-        for (int db = 0; db < NDB; ++db)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[db][r] *= alpha;
-      }
-      const float mref = mrow;
-      float sum = 0.f;
-      bf16x8 pb[2];  // probabilities of the tile as B operands
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float e = fast_exp2(__builtin_fmaf(sr[r], sc, -mref));
-        sum += e;
-        pb[r >> 3][r & 7] = (__bf16)e;
-      }
-      lrow += sum;
-#pragma unroll
-      for (int blk = 0; blk < 2; ++blk) {
-        // tokens this lane feeds for this block: 8h .. 8h+7; on the ragged tile zero the
-        // ones past the end so stale cache contents (possibly NaN) cannot leak through 0 * x
-        const int nv = tok_len - (tok0 + 16 * blk + 8 * h);
-#pragma unroll
-        for (int db = 0; db < NDB; ++db) {
-          bf16x8 a;
-          if constexpr (FP8) {
-            // rows of channel blocks 2 * pair and 2 * pair + 1 sit in the lower and upper
-            // lane halves; the swap hands every lane its tokens 8h..8h+7 of both blocks:
-            // dwords 0,1 become the operand of block 2 * pair, dwords 2,3 of 2 * pair + 1
-            const i32x4 raw = vt.v[blk][db >> 1];
-            const auto s0 = __builtin_amdgcn_permlane32_swap((unsigned)raw[0], (unsigned)raw[2], false, false);
-            const auto s1 = __builtin_amdgcn_permlane32_swap((unsigned)raw[1], (unsigned)raw[3], false, false);
-            i32x2 w = {(int)s0[db & 1], (int)s1[db & 1]};
-            if constexpr (RAGGED) {
-#pragma unroll
-              for (int j = 0; j < 2; ++j) {
-                unsigned keep = 0;
-#pragma unroll
-                for (int b = 0; b < 4; ++b)
-                  if (4 * j + b < nv) keep |= 0xffu << (8 * b);
-                w[j] &= keep;
-              }
-            }
-            a = fp8x8_to_bf16(w[0], w[1]);
-          } else {
-            i32x4 w = vt.v[blk][db];
-            if constexpr (RAGGED) {
-#pragma unroll
-              for (int j = 0; j < 4; ++j) {
-                unsigned keep = (2 * j < nv ? 0xffffu : 0u) | (2 * j + 1 < nv ? 0xffff0000u : 0u);
-                w[j] &= keep;
-              }
-            }
-            a = __builtin_bit_cast(bf16x8, w);
-          }
-          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[blk], acc[db], 0, 0, 0);
-        }
-      }
-    };
+    // first tiles of the next item: its first pair, or, for the wave that takes its pair's
+    // item from the back, its last pair
+    const bool a_from_back = COOP && coop_back && ta < coop && a_last >= 2 * kCoopMinPairs - 2;
+    const int a_t0 = a_from_back ? (a_last & ~1) : 0;
+    const int a_t1 = min(a_t0 + 1, a_last);
 
     // ---- all pairs of tiles but the last: both tiles full, refills from this item.
     // Buffer 0 holds tile ti, buffer 1 tile ti + 1; a refill past the end (odd tile count)
     // repeats the last tile so that the number of loads in flight never varies.
     for (int pr = 0; pr < npairs - 1; ++pr) {
       const int ti = 2 * pr;
-      compute_tile(kb0, vb0, ti, std::false_type{});
+      compute_tile(it, kb0, vb0, ti, std::false_type{});
       load_tile(kb0, vb0, my_blk, nblk, kvh, ti + 2);
-      compute_tile(kb1, vb1, ti + 1, std::false_type{});
+      compute_tile(it, kb1, vb1, ti + 1, std::false_type{});
       load_tile(kb1, vb1, my_blk, nblk, kvh, min(ti + 3, last));
     }
 
@@ -344,31 +424,19 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
     // the last record of the list, loads nobody uses)
     const int ti = 2 * (npairs - 1);
     if (ti < nfull)
-      compute_tile(kb0, vb0, ti, std::false_type{});
+      compute_tile(it, kb0, vb0, ti, std::false_type{});
     else
-      compute_tile(kb0, vb0, ti, std::true_type{});
-    load_tile(kb0, vb0, a_blk, a_nblk, akvh, 0);
+      compute_tile(it, kb0, vb0, ti, std::true_type{});
+    load_tile(kb0, vb0, a_blk, a_nblk, akvh, a_t0);
     if (ti + 1 < nfull)
-      compute_tile(kb1, vb1, ti + 1, std::false_type{});
+      compute_tile(it, kb1, vb1, ti + 1, std::false_type{});
     else if (ti + 1 <= last)
-      compute_tile(kb1, vb1, ti + 1, std::true_type{});
+      compute_tile(it, kb1, vb1, ti + 1, std::true_type{});
 
     // Write the partial (before the second refill: stores count as outstanding memory
     // operations too, and behind the refill they would be waited for together with it).
-    // Every accumulator register of a lane belongs to the lane's own query row, so
-    // normalisation is per lane.  The rows then pass through a wave-private strip of LDS
-    // so that they leave as whole rows: stored straight from the accumulator layout a row
-    // goes out in sixteen pieces, and back-to-back partial writes to one cache line cost a
-    // wave several microseconds per item.
-    {
-      const float vs = FP8 ? v_scale : 1.f;
-      const float l = lrow + __shfl_xor(lrow, 32);
-      stage_partial_row<D>(strip, m, h, acc, vs / l, prow, (mrow + fast_log2(l)) * kLn2, p.partial_lse);
-      __builtin_amdgcn_wave_barrier();
-      store_partial_rows<D, STREAM>(strip, mcnt * G, lane, p.partial_out);
-      __builtin_amdgcn_wave_barrier();
-    }
-    load_tile(kb1, vb1, a_blk, a_nblk, akvh, min(1, a_last));
+    write_partial(it, prow, mcnt * G, 0);
+    load_tile(kb1, vb1, a_blk, a_nblk, akvh, a_t1);
 
     // ---- move on
     if (ta >= ntickets) break;
@@ -378,8 +446,84 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
     r0 = a0, r1 = a1, kvh = akvh, my_blk = a_blk, seq = a_seq;
     a0 = b0, a1 = b1, akvh = bkvh, a_blk = b_blk, a_seq = b_seq;
     b0 = c0, b1 = c1, bkvh = ckvh;
+    t_cur = ta;
     ta = tb;
     tb = tc;
+    if constexpr (COOP) {
+      if (t_cur < coop) {
+        to_pair_item = true;
+        break;
+      }
+    }
+  }
+
+  // ---- the item shared with the other wave of the pair, the last one of both.  Pairs of
+  // tiles are claimed from a counter of the pair: bits 0-9 count the claims from the front,
+  // bits 10-19 those from the back; the first two pairs at either end are granted without a
+  // claim.  A claim is good while the counts do not meet.  A wave that is through replaces its
+  // own count by a marker (+2^20 from the front, -2^20 from the back) that makes every later
+  // claim of the other wave fail, so that after both the counter is zero again for the next
+  // launch.  Claims run two pairs ahead of the arithmetic, refills one pair ahead, so a claim
+  // has a whole pair of tiles to come back.  An item of fewer than four pairs is attended by
+  // its front wave alone.
+  if (COOP && to_pair_item) {
+    Item it;
+    begin_item(it);
+    const int tok_len = it.tok_len, sees = it.sees;
+    const int mcnt = __builtin_amdgcn_readfirstlane(r1.x);
+    const int ord = __builtin_amdgcn_readfirstlane(r1.y);
+    const int nblk = (tok_len + kBlock - 1) / kBlock;
+    const int ntiles = (tok_len + kTile - 1) / kTile;
+    const int nfull = (tok_len - (sees > 0 ? 1 : 0)) / kTile;
+    const int last = ntiles - 1;
+    const int npairs = (ntiles + 1) >> 1;
+    const bool shared_item = npairs >= kCoopMinPairs;
+    if (shared_item || !coop_back) {
+      const bool from_back = shared_item && coop_back;
+      const int64_t front_row = ((int64_t)seq * p.max_partials + ord) * p.num_q_heads + kvh * G + row_head;
+      const int64_t back_row = p.coop_row0 + (int64_t)pair_id * 32 + m;
+      const int64_t prow = row_member < mcnt ? (from_back ? back_row : front_row) : -1;
+      // the front partial says where the back partial of the same query row is
+      const int tag = shared_item && !coop_back ? ((pair_id + 1) << 5) | m : 0;
+      const int inc = shared_item ? (coop_back ? 1 << 10 : 1) : 0;
+      int* ctr = p.coop_ctr + pair_id;
+      int added = 0, claim_v = 0;
+      auto issue_claim = [&](int by) {
+        if (lane == 0) claim_v = atomicAdd(ctr + opaque_zero, by);
+        added += by;
+      };
+      // the pair of tiles after `cur`, or -1 when there is none left for this wave
+      auto next_pair = [&](int cur) -> int {
+        if (!shared_item) return cur + 1 < npairs ? cur + 1 : -1;
+        const int old = __builtin_amdgcn_readfirstlane(claim_v);
+        const int f = old & 1023, b = (old >> 10) & 1023;
+        if ((old >> 20) != 0 || 4 + f + b >= npairs) return -1;
+        return coop_back ? npairs - 3 - b : 2 + f;
+      };
+      auto compute_any = [&](const KT& kt, const VT& vt, int ti) {
+        if (ti > last) return;
+        if (ti < nfull)
+          compute_tile(it, kt, vt, ti, std::false_type{});
+        else
+          compute_tile(it, kt, vt, ti, std::true_type{});
+      };
+      int cur = from_back ? npairs - 1 : 0;
+      int nxt = from_back ? npairs - 2 : (npairs > 1 ? 1 : -1);  // granted
+      issue_claim(inc);
+      for (;;) {
+        const int refill = nxt >= 0 ? nxt : cur;  // (past the end: loads nobody uses, as above)
+        compute_any(kb0, vb0, 2 * cur);
+        load_tile(kb0, vb0, my_blk, nblk, kvh, 2 * refill);
+        compute_any(kb1, vb1, 2 * cur + 1);
+        load_tile(kb1, vb1, my_blk, nblk, kvh, min(2 * refill + 1, last));
+        if (nxt < 0) break;
+        cur = nxt;
+        nxt = next_pair(cur);
+        issue_claim(nxt >= 0 ? inc : 0);
+      }
+      write_partial(it, prow, mcnt * G, tag);
+      if (shared_item && lane == 0) atomicAdd(ctr, (coop_back ? -(1 << 20) : (1 << 20)) - added);
+    }
   }
   // loads nobody uses are still in flight: let them land before the wave ends
   __builtin_amdgcn_s_waitcnt(0);

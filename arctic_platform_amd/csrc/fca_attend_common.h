@@ -84,10 +84,12 @@ __device__ inline float pow2_ceil(float x) {
 // Lane (m, h) holds, in acc[db][4 * q4 + e], channel 32 * db + 8 * q4 + 4 * h + e of query
 // row `row` of the tile.  Normalises the row by `inv` (1 / softmax sum, times the V scale
 // of an fp8 cache), stages it in the strip as scaled halves and, from the lanes with
-// h == 0, writes {lse, scale} and leaves the destination row index in the strip.
+// h == 0, writes {lse, scale} and leaves the destination row index in the strip.  `tag`
+// (below 2^23) is stored in the mantissa bits of the scale, which is a power of two: the
+// merge reads it as the place of a second partial of the same chunk (0 = none).
 template <int D>
 __device__ inline void stage_partial_row(char* strip, int row, int h, const f32x16 (&acc)[D / 32], float inv,
-                                         int64_t prow, float lse, float* partial_lse) {
+                                         int64_t prow, float lse, float* partial_lse, int tag = 0) {
   float amax = 0.f;
 #pragma unroll
   for (int db = 0; db < D / 32; ++db)
@@ -99,7 +101,7 @@ __device__ inline void stage_partial_row(char* strip, int row, int h, const f32x
   if (prow < 0) return;
   char* dst = strip + row * strip_row_bytes<D>();
   if (h == 0) {
-    *reinterpret_cast<f32x2*>(partial_lse + 2 * prow) = f32x2{lse, scale};
+    *reinterpret_cast<f32x2*>(partial_lse + 2 * prow) = f32x2{lse, __uint_as_float(__float_as_uint(scale) | (unsigned)tag)};
     *reinterpret_cast<int64_t*>(dst + D * 2) = prow;
   }
 #pragma unroll

@@ -261,6 +261,10 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   // from that block on.
   auto declared = [&](int s) { return p.row_group && p.row_group[s] >= 0; };
 
+  // claim counters of the attention kernel: zero before the first launch on this workspace
+  // (every launch leaves them at zero again)
+  for (int i = tid; i < kCoopMaxPairs; i += kBuildThreads) meta[L.coop_ctr + i] = 0;
+
   // ---- update: is the forest of the last build on this workspace still the forest of
   // these rows?  (pos = first private block of a row, ord = chunks of its shared nodes:
   // both are left in the workspace by the build.)

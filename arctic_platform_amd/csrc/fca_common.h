@@ -15,6 +15,11 @@ constexpr int kMaxChunk = 1024;          // one lane of a wave holds one block i
 constexpr int kItemInts = 8;             // int32 per work-item record
 constexpr int kSizeBuckets = 32;         // size classes for the descending work-list order
 constexpr int kHeaderInts = 16;
+// Items that two waves of the 32-row attention kernel attend together (one from either end):
+// at most this many pairs of waves, one claim counter each in the metadata workspace, and 32
+// partial rows each behind the ordinary partial rows for the wave that comes from the back.
+constexpr int kCoopMaxPairs = 1024;
+constexpr int kCoopMinPairs = 4;  // pairs of 32-token tiles an item needs to be shared
 
 enum HeaderSlot {
   H_ITEMS = 0,
@@ -51,6 +56,7 @@ struct MetaLayout {
   int64_t hash_keys;  // 64-bit keys, 2 int32 each
   int64_t hash_min;
   int64_t hash_size;  // entries (power of two)
+  int64_t coop_ctr;   // [kCoopMaxPairs] claim counters of the attention kernel, zero between launches
   int64_t max_items;
   int64_t max_partials;
   int64_t total;
@@ -104,6 +110,7 @@ inline __host__ MetaLayout make_layout(const fca_plan& p) {
   L.hash_size = hs;
   L.hash_keys = take(2 * hs);
   L.hash_min = take(hs);
+  L.coop_ctr = take(kCoopMaxPairs);
   L.total = off;
   return L;
 }
@@ -115,6 +122,12 @@ inline __host__ __device__ int chunk_len_for(int tokens, int chunk_tokens) {
   int n = (tokens + chunk_tokens - 1) / chunk_tokens;
   int len = (tokens + n - 1) / n;
   return (len + kTile - 1) / kTile * kTile;
+}
+// Pairs of waves that can share an item under a plan: the attention grid never has more
+// than one wave per possible ticket.
+inline __host__ int64_t coop_pairs_for(const fca_plan& p, const MetaLayout& L) {
+  const int64_t waves = L.max_items * p.num_kv_heads + 3;
+  return waves / 2 < kCoopMaxPairs ? waves / 2 : kCoopMaxPairs;
 }
 inline __host__ __device__ int num_chunks_for(int tokens, int chunk_tokens) {
   if (tokens <= 0) return 0;
@@ -155,9 +168,15 @@ struct AttendParams {
   int32_t max_partials;
   int32_t select;  // 0 all items, 1 shared only, 2 leaves only
   int32_t kv_reread;  // a launch reads KV blocks more than once (query runs): keep the loads cacheable
+  // items attended by two waves (32-row kernel): claim counters, how many pairs the partial
+  // buffers have rows for, and the first of those rows
+  int32_t* coop_ctr;
+  int32_t coop_pairs;
+  int64_t coop_row0;
 };
 
 struct MergeParams {
+  const int32_t* header;  // metadata header: a non-zero error slot turns every output into NaN
   const int32_t* seq_npart;
   const void* partial_out;
   const float* partial_lse;
@@ -166,6 +185,7 @@ struct MergeParams {
   float* lse;
   int32_t num_seqs, num_q_heads, head_dim, max_partials, out_dtype;
   int32_t vector_out;  // out rows allow 16-byte stores
+  int64_t coop_row0;   // first of the partial rows written by waves that took a shared item from the back
 };
 
 struct AppendParams {

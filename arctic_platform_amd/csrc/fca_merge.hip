@@ -40,21 +40,33 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
   float acc[V];
 #pragma unroll
   for (int e = 0; e < V; ++e) acc[e] = 0.f;
+  auto take = [&](float l, float scale, const f16x8& o) {
+    if (!(l > -INFINITY)) return;  // empty partial: weight 0, whatever its output holds
+    const float m_new = fmaxf(m, l);
+    const float keep = __expf(m - m_new);  // exp(-inf) = 0 on the first live partial
+    const float w = __expf(l - m_new);
+    wsum = wsum * keep + w;
+    const float ws = w * scale;
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = acc[e] * keep + ws * (float)o[e];
+    m = m_new;
+  };
 #pragma unroll 4
   for (int i = share; i < np; i += SPLIT) {
     const int64_t pr = (base + i) * p.num_q_heads + hq;
     const float2 ls = lse_scale[pr];
     const f16x8 o = *reinterpret_cast<const f16x8*>(rows + pr * D + sub * V);
-    const float l = ls.x;
-    if (!(l > -INFINITY)) continue;  // empty partial: weight 0, whatever its output holds
-    const float m_new = fmaxf(m, l);
-    const float keep = __expf(m - m_new);  // exp(-inf) = 0 on the first live partial
-    const float w = __expf(l - m_new);
-    wsum = wsum * keep + w;
-    const float ws = w * ls.y;
-#pragma unroll
-    for (int e = 0; e < V; ++e) acc[e] = acc[e] * keep + ws * (float)o[e];
-    m = m_new;
+    // the scale is a power of two; its mantissa bits say where a second partial of the same
+    // chunk is (an item attended by two waves of the attention kernel), 0 = nowhere
+    const unsigned sbits = __float_as_uint(ls.y);
+    const unsigned tag = sbits & 0x007fffffu;
+    take(ls.x, __uint_as_float(sbits & 0xff800000u), o);
+    if (tag) {
+      const int64_t br = p.coop_row0 + (int64_t)(tag - 32);  // tag = (pair + 1) * 32 + row of the tile
+      const float2 bls = lse_scale[br];
+      const f16x8 bo = *reinterpret_cast<const f16x8*>(rows + br * D + sub * V);
+      take(bls.x, bls.y, bo);
+    }
   }
   // combine the shares: the same update with a whole running result in place of one partial
 #pragma unroll
@@ -69,7 +81,11 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
     m = m_new;
   }
   if (!live_row || share != 0) return;
-  const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
+  // The builder records input it had to clamp (a length beyond the block table, a row-table
+  // entry out of range, overflowing lists) in the header and carries on; results made from
+  // such metadata leave as NaN so that they cannot pass for attention over a cut-off sequence.
+  const bool flagged = p.header[H_ERROR] != 0;
+  const float inv = flagged ? __builtin_nanf("") : (wsum > 0.f ? 1.f / wsum : 0.f);
   const int64_t o = (int64_t)s * p.out_seq_stride + (int64_t)hq * p.out_head_stride + sub * V;
   if (p.out_dtype == FCA_F32) {
     float* dst = reinterpret_cast<float*>(p.out) + o;
@@ -95,7 +111,7 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
       for (int e = 0; e < V; ++e) dst[e] = __float2bfloat16(acc[e] * inv);
     }
   }
-  if (p.lse && sub == 0) p.lse[row] = wsum > 0.f ? m + __logf(wsum) : -INFINITY;
+  if (p.lse && sub == 0) p.lse[row] = flagged ? __builtin_nanf("") : (wsum > 0.f ? m + __logf(wsum) : -INFINITY);
 }
 
 // Plain 16-bytes-per-lane copy, the yardstick the hardware traffic counters are scaled by.

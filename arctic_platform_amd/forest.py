@@ -32,8 +32,8 @@ class ForestMetadata:
     plan: _lib.FcaPlan
     layout: _lib.FcaMetaLayout
     meta: torch.Tensor  # int32 workspace on the device
-    partial_out: torch.Tensor  # half [S * max_partials, Hq, D]: rows scaled by a power of two
-    partial_lse: torch.Tensor  # fp32 [S * max_partials, Hq, 2]: {lse, row scale}
+    partial_out: torch.Tensor  # half, fca_workspace_bytes: [S * max_partials * Hq + shared-item rows, D], rows scaled by a power of two
+    partial_lse: torch.Tensor  # fp32, fca_workspace_bytes: {lse, row scale} per row
     block_table: torch.Tensor
     seq_lens: torch.Tensor  # per query row
     row_table: torch.Tensor | None = None  # block-table row of every query row (None: the row itself)
@@ -222,20 +222,18 @@ def build_forest_metadata(
         nm, no, nl = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
         _lib.check(lib.fca_workspace_bytes(ctypes.byref(plan), ctypes.byref(nm), ctypes.byref(no), ctypes.byref(nl)))
         dev = block_table.device
-        slots = plan.num_seqs * layout.max_partials
         md = ForestMetadata(
             plan=plan,
             layout=layout,
             meta=torch.zeros(nm.value // 4, dtype=torch.int32, device=dev),
-            partial_out=torch.empty(slots, num_q_heads, head_dim, dtype=torch.float16, device=dev),
-            partial_lse=torch.empty(slots, num_q_heads, 2, dtype=torch.float32, device=dev),
+            partial_out=torch.empty(no.value // 2, dtype=torch.float16, device=dev),
+            partial_lse=torch.empty(nl.value // 4, dtype=torch.float32, device=dev),
             block_table=block_table,
             seq_lens=seq_lens,
             row_table=row_table,
             row_group=row_group,
             kv_reread=row_group is not None if kv_reread is None else bool(kv_reread),
         )
-        assert md.partial_out.numel() * 2 == no.value and md.partial_lse.numel() * 4 == nl.value
     if row_table is not None:
         _lib.check(
             lib.fca_build_metadata_rows(

@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define FCA_VERSION 100
+#define FCA_VERSION 101
 #define FCA_BLOCK_SIZE 16
 #define FCA_MAX_LEVELS 8
 
@@ -118,6 +118,8 @@ typedef struct fca_meta_layout {
   int64_t node_tok;      /* [S] KV tokens of the node: num blocks * 16, or, for a causal node, up to
                             the last token of its last member */
   int64_t node_causal;   /* [S] 1: the node is a tile of a query run (fca_build_metadata_rows) */
+  int64_t coop_ctr;      /* [1024] claim counters of the attention kernel (pairs of waves that attend
+                            an item together), zero between launches */
 } fca_meta_layout;
 
 int fca_version(void);
@@ -125,9 +127,11 @@ const char* fca_last_error(void);
 
 /* Workspace sizes for a plan: metadata (int32 arrays) and the two partial buffers.  A
  * partial output row is D half-precision values times one power-of-two scale per row:
- * partial_out is half [S * max_partials, Hq, D], partial_lse is fp32
- * [S * max_partials, Hq, 2] = {natural-log lse, scale}.  Both are opaque to the caller:
- * written by the passes, read by the merge. */
+ * partial_out is half [rows, D], partial_lse is fp32 [rows, 2] = {natural-log lse, scale},
+ * rows = S * max_partials * Hq plus 32 for each pair of waves that may attend an item
+ * together (at most 1024 pairs; the second wave of a pair writes there, and the scale of
+ * the first wave's row carries the place in its mantissa bits).  Both are opaque to the
+ * caller: written by the passes, read by the merge. */
 int fca_workspace_bytes(const fca_plan* plan, size_t* meta_bytes, size_t* partial_out_bytes, size_t* partial_lse_bytes);
 int fca_meta_describe(const fca_plan* plan, fca_meta_layout* layout);
 
@@ -228,7 +232,7 @@ int fca_decode_step(const fca_plan* plan, const fca_tensors* t, void* meta_dev,
  * uses it: calls that overlap in time on one GPU (two streams, two threads) race; stream
  * order is enough.  The first call on a device looks the array's address up
  * (hipGetSymbolAddress); make that call outside graph capture. */
-#define FCA_STATIC_SCRATCH_BYTES (40u << 20)
+#define FCA_STATIC_SCRATCH_BYTES (48u << 20)
 int fca_decode_step_static(const fca_plan* plan, const fca_tensors* t, void* meta_dev, void* out_dev,
                            int64_t out_seq_stride, int64_t out_head_stride, int32_t out_dtype, float* lse_dev,
                            void* stream);

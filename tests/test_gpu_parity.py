@@ -221,6 +221,16 @@ def test_bad_lengths_are_flagged(gpu):
     torch.cuda.synchronize()
     with pytest.raises(ValueError):
         md.check()
+    # a caller that never looks at the flag still cannot mistake the result for attention
+    # over the clamped sequence: the merge turns every output of such metadata into NaN
+    from arctic_platform_amd.kv_layout import kv_cache_shape
+    from arctic_platform_amd.ops import forest_cascade_decode
+
+    q = torch.randn(2, 8, 64, device=gpu).to(torch.bfloat16)
+    cache = torch.randn(kv_cache_shape(4, 16, 2, 64), device=gpu).to(torch.bfloat16)
+    out, lse = forest_cascade_decode(q, cache, md, 0.125)
+    torch.cuda.synchronize()
+    assert torch.isnan(out.float()).all() and torch.isnan(lse).all()
 
 
 def test_error_budget_of_fp32_outputs(gpu):
@@ -247,3 +257,31 @@ def test_error_budget_of_fp32_outputs(gpu):
         rel = float((got - want).norm() / want.norm())
         assert rel < 2.5e-3, f"KV head {kvh}: relative rms error {rel:.2e}"
     assert float((lse.cpu().double() - ref_lse).abs().max()) < 1e-5
+
+
+@pytest.mark.parametrize("index,workgroups,chunk", [(2, 8, 512), (2, 4, 1024), (5, 8, 512), (4, 16, 256)])
+def test_items_shared_by_pairs_of_waves(gpu, index, workgroups, chunk, monkeypatch):
+    """With many items per wave the 32-row kernel sets the largest items aside, one per pair of
+    waves, and both waves of a pair attend it from either end until their claims meet.  A
+    small grid brings that schedule to a small batch.  Items long enough (four pairs of tiles)
+    are shared, shorter ones go to the front wave alone; either way the result is the oracle's,
+    the claim counters are zero again after every launch, and a second launch agrees."""
+    from arctic_platform_amd.ops import forest_cascade_decode
+
+    monkeypatch.setenv("FCA_ATTEND_WORKGROUPS", str(workgroups))
+    w = make_config(index, device=gpu, shrink=4, poison_unused=True)
+    md, out, lse = _run(w, chunk_tokens=chunk)
+    items = md.items()
+    waves = 4 * workgroups
+    tickets = len(items) * w.num_kv_heads
+    assert tickets >= waves // 2 + 3 * waves, "the batch is too small to set items aside"
+    set_aside = [it["tok_len"] for it in items[: waves // 2 // w.num_kv_heads + 1]]
+    assert max(set_aside) >= 7 * 32 - 31, "no item long enough to be shared"
+    ref_out, ref_lse = oracle_for(w)
+    assert_matches_oracle(out, lse, ref_out, ref_lse, what=f"C{index}/4, {workgroups} workgroups")
+    ctr = md.meta[md.layout.coop_ctr : md.layout.coop_ctr + 1024]
+    assert int(ctr.abs().max()) == 0
+    out2, lse2 = forest_cascade_decode(w.q, w.kv_cache, md, w.scale, w.k_scale, w.v_scale)
+    torch.cuda.synchronize()
+    assert_matches_oracle(out2, lse2, ref_out, ref_lse, what="second launch")
+    assert int(ctr.abs().max()) == 0
