@@ -408,7 +408,7 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 64)) void fca_a
       for (int rt = 0; rt < NRT; ++rt) {
         if (rt > 0 && !two_tiles) continue;
         const float l = lrow[rt] + __shfl_xor(lrow[rt], 32);
-        stage_partial_row<D>(strip, rt * 32 + m, h, acc[rt], vs / l, prow[rt], (mrow[rt] + fast_log2(l)) * kLn2,
+        stage_partial_row<D, STREAM>(strip, rt * 32 + m, h, acc[rt], vs / l, prow[rt], (mrow[rt] + fast_log2(l)) * kLn2,
                              p.partial_lse);
       }
       __builtin_amdgcn_wave_barrier();

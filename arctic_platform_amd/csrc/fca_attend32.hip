@@ -367,7 +367,7 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
     // an item half of which nobody attended here (the other wave of the pair took all of it)
     // leaves an empty partial: log-sum-exp -inf, weight 0 in the merge
     const float inv = l > 0.f ? vs / l : 0.f;
-    stage_partial_row<D>(strip, m, h, it.acc, inv, prow, (it.mrow + fast_log2(l)) * kLn2, p.partial_lse, tag);
+    stage_partial_row<D, STREAM>(strip, m, h, it.acc, inv, prow, (it.mrow + fast_log2(l)) * kLn2, p.partial_lse, tag);
     __builtin_amdgcn_wave_barrier();
     store_partial_rows<D, STREAM>(strip, live_rows, lane, p.partial_out);
     __builtin_amdgcn_wave_barrier();

@@ -135,6 +135,15 @@ inline __host__ __device__ int num_chunks_for(int tokens, int chunk_tokens) {
   return (tokens + len - 1) / len;
 }
 
+// Device-scope 8-byte accesses: a store that is written through to memory, a load that does
+// not trust the L2 of the XCD it runs on.
+__device__ inline void store8_coherent(void* ptr, uint64_t v) {
+  __hip_atomic_store(reinterpret_cast<uint64_t*>(ptr), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ inline uint64_t load8_coherent(const void* ptr) {
+  return __hip_atomic_load(reinterpret_cast<const uint64_t*>(ptr), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 struct BuildParams {
   fca_plan plan;
   const int32_t* block_table;

@@ -40,6 +40,7 @@ def parse_args():
     ap.add_argument("--kv-copies", type=int, default=4, help="distinct KV caches cycled over the layers")
     ap.add_argument("--chunk", type=int, default=0, help="split-K chunk in tokens (0 = default of the configuration)")
     ap.add_argument("--rows", type=int, default=0, help="query rows per work item, 32 or 64 (0 = default)")
+    ap.add_argument("--time-every", type=int, default=0, help="bracket the attention launch of every n-th timed step with events (0 = about 24 per run)")
     ap.add_argument("--cpu-seqs", type=int, default=512, help="sequences in the CPU baseline sample (0 = skip)")
     ap.add_argument("--skip-noncascade", action="store_true")
     ap.add_argument("--split-passes", action="store_true", help="also time the shared-prefix pass and the suffix pass as launches of their own (and leave them in the trace for the profiler)")
@@ -55,32 +56,37 @@ def median(xs):
     return xs[len(xs) // 2]
 
 
-def run_steps(torch, ops, build, w, caches, md, out, lse, steps, layers, timed_events=None):
+def run_steps(torch, ops, build, w, caches, md, out, lse, steps, layers, timed_events=None, time_every=1):
     """``steps`` layer calls; metadata refreshed at every ``layers``-th one.  When
-    ``timed_events`` is a list, the attention launch of each rebuilt step is bracketed by
-    events on the launch stream."""
+    ``timed_events`` is a list, the attention launch of every ``time_every``-th step is
+    bracketed by events on the launch stream (the step is the same two launches either way)."""
     for i in range(steps):
         cache = caches[i % len(caches)]
         if i % layers == 0:
             build()
-            if timed_events is not None:
-                a = torch.cuda.Event(enable_timing=True)
-                b = torch.cuda.Event(enable_timing=True)
-                a.record()
-                ops.forest_pass(w.q, cache, md, w.scale, w.k_scale, w.v_scale)
-                b.record()
-                ops.merge_partials(md, w.q, out=out, return_lse=False)
-                timed_events.append((a, b))
-                continue
+        if timed_events is not None and i % time_every == 0:
+            a = torch.cuda.Event(enable_timing=True)
+            b = torch.cuda.Event(enable_timing=True)
+            a.record()
+            ops.forest_pass(w.q, cache, md, w.scale, w.k_scale, w.v_scale)
+            b.record()
+            ops.merge_partials(md, w.q, out=out, return_lse=False)
+            timed_events.append((a, b))
+            continue
         ops.forest_cascade_decode(w.q, cache, md, w.scale, w.k_scale, w.v_scale, out=out, return_lse=False)
 
 
-def time_steps(torch, ops, build, w, caches, md, out, lse, steps, warmup, layers):
+def time_steps(torch, ops, build, w, caches, md, out, lse, steps, warmup, layers, time_every=0):
+    """Wall time of ``steps`` steps after ``warmup`` untimed ones, and the event-timed durations
+    of the attention launches inside the timed region (``time_every`` = 0: as many as 24,
+    evenly spread, never fewer than every second step of a short run)."""
+    if time_every <= 0:
+        time_every = max(1, steps // 24)
     run_steps(torch, ops, build, w, caches, md, out, lse, warmup, layers)
     torch.cuda.synchronize()
     events = []
     t0 = time.perf_counter()
-    run_steps(torch, ops, build, w, caches, md, out, lse, steps, layers, events)
+    run_steps(torch, ops, build, w, caches, md, out, lse, steps, layers, events, time_every)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     kernel_us = [a.elapsed_time(b) * 1e3 for a, b in events]
@@ -423,7 +429,7 @@ def main():
         # device checks that the rows still carry the forest and remakes leaves and work list
         build_forest_metadata(w.block_table, w.seq_lens, out=md, update=True, **kw)
 
-    wall, kern_us = time_steps(torch, ops, refresh, w, caches, md, out, None, args.steps, args.warmup, args.layers)
+    wall, kern_us = time_steps(torch, ops, refresh, w, caches, md, out, None, args.steps, args.warmup, args.layers, args.time_every)
     step_us = wall / args.steps * 1e6
     checked_rows = out[: max(0, min(args.cpu_seqs, w.num_seqs))].clone()  # compared with the oracle below
     kern = sum(kern_us) / len(kern_us)
