@@ -36,6 +36,7 @@ EXPORTS = (
     "fca_append_kv",
     "fca_gather_kv",
     "fca_calibration_copy",
+    "fca_time_next_attention",
     "fca_split_layout_ints",
     "fca_split_layout_build",
     "fca_split_workspace_bytes",
@@ -164,6 +165,7 @@ def load_library() -> ctypes.CDLL:
     lib.fca_append_kv.argtypes = [VP, VP, I64, I64, I32, I32, I32, VP, VP, VP, I64, I64, I32, VP, VP, VP]
     lib.fca_gather_kv.argtypes = lib.fca_append_kv.argtypes
     lib.fca_calibration_copy.argtypes = [VP, VP, ctypes.c_size_t, VP]
+    lib.fca_time_next_attention.argtypes = [VP, VP]
     F32 = ctypes.c_float
     lib.fca_split_layout_ints.argtypes = [I32, P(I64)]
     lib.fca_split_layout_build.argtypes = [I32, VP, VP, VP, I32, I32, VP]

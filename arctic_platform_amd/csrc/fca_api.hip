@@ -392,6 +392,13 @@ int fca_gather_kv(void* key_dev, void* value_dev, int64_t token_stride, int64_t 
                     k_scale_dev, v_scale_dev, stream);
 }
 
+int fca_time_next_attention(void* start_event, void* stop_event) {
+  if ((start_event == nullptr) != (stop_event == nullptr))
+    return fail(FCA_ERR_INVALID_ARG, "start and stop events come as a pair (both or neither)");
+  fca::set_attend_timing(static_cast<hipEvent_t>(start_event), static_cast<hipEvent_t>(stop_event));
+  return FCA_OK;
+}
+
 int fca_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void* stream) {
   if (!src_dev || !dst_dev || (bytes & 15) || (reinterpret_cast<uintptr_t>(src_dev) & 15) ||
       (reinterpret_cast<uintptr_t>(dst_dev) & 15))

@@ -30,6 +30,8 @@
 // Semantics (softmax scale, GQA head mapping h -> h / (Hq/Hkv), no mask for the decode
 // token) follow arctic_platform/model/implementations/qwen35/models/qwen3_5_moe/
 // modeling_qwen3_5_moe.py:368-373, :385, :440-454.
+#include <hip/hip_ext.h>
+
 #include <cstring>
 #include <cstdlib>
 #include <type_traits>
@@ -425,6 +427,13 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 64)) void fca_a
   }
 }
 
+static thread_local hipEvent_t g_time_start = nullptr, g_time_stop = nullptr;
+void set_attend_timing(hipEvent_t start, hipEvent_t stop) { g_time_start = start, g_time_stop = stop; }
+void take_attend_timing(hipEvent_t* start, hipEvent_t* stop) {
+  *start = g_time_start, *stop = g_time_stop;
+  g_time_start = g_time_stop = nullptr;
+}
+
 static int cached_cu_count() {
   static int cus = 0;
   if (cus == 0) {
@@ -463,8 +472,10 @@ hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dty
   // memory-side cache serves the repeats, so the loads stay ordinary; likewise when query
   // runs make successive tiles of a sequence read the same blocks.
   const bool stream_kv = plan.max_levels > 0 && !p.kv_reread;
+  hipEvent_t ev_start, ev_stop;
+  take_attend_timing(&ev_start, &ev_stop);
 #define FCA_LAUNCH(D_, F_, S_) \
-  hipLaunchKernelGGL((fca_attend64_kernel<D_, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, p)
+  hipExtLaunchKernelGGL((fca_attend64_kernel<D_, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, ev_start, ev_stop, 0, p)
 #define FCA_PICK(D_, F_) \
   if (stream_kv) FCA_LAUNCH(D_, F_, true); else FCA_LAUNCH(D_, F_, false)
   if (plan.head_dim == 128) {

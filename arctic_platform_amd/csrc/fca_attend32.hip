@@ -26,6 +26,8 @@
 // branch): the hardware counts outstanding vector memory operations in order and the
 // compiler picks each wait's count for the shortest path, so a load issued on only some
 // paths would turn the waits behind it into full drains of the tile stream.
+#include <hip/hip_ext.h>
+
 #include <type_traits>
 
 #include "fca_attend_common.h"
@@ -536,8 +538,10 @@ hipError_t launch_attend32(const AttendParams& p, const fca_plan& plan, int kv_d
   // memory-side cache serves the repeats, so the loads stay ordinary; likewise when query
   // runs make successive tiles of a sequence read the same blocks.
   const bool stream_kv = plan.max_levels > 0 && !p.kv_reread;
+  hipEvent_t ev_start, ev_stop;
+  take_attend_timing(&ev_start, &ev_stop);
 #define FCA_LAUNCH(D_, F_, S_) \
-  hipLaunchKernelGGL((fca_attend32_kernel<D_, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, p)
+  hipExtLaunchKernelGGL((fca_attend32_kernel<D_, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, ev_start, ev_stop, 0, p)
 #define FCA_PICK(D_, F_) \
   if (stream_kv) FCA_LAUNCH(D_, F_, true); else FCA_LAUNCH(D_, F_, false)
   if (plan.head_dim == 128) {

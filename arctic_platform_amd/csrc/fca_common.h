@@ -264,6 +264,9 @@ hipError_t launch_rows(const int32_t* query_start_loc, const int32_t* seq_lens, 
 hipError_t launch_append(const AppendParams& p, int kv_dtype, hipStream_t stream);
 hipError_t launch_gather(const AppendParams& p, int kv_dtype, hipStream_t stream);  // key / value are written
 hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, hipStream_t stream);
+// Events the next attention launch of this thread records its begin and end in (NULL: none).
+void set_attend_timing(hipEvent_t start, hipEvent_t stop);
+void take_attend_timing(hipEvent_t* start, hipEvent_t* stop);
 hipError_t launch_attend32(const AttendParams& p, const fca_plan& plan, int kv_dtype, int grid, hipStream_t stream);
 hipError_t launch_merge(const MergeParams& p, hipStream_t stream);
 hipError_t launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);

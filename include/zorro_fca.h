@@ -310,6 +310,15 @@ int fca_split_attention_backward(const fca_split_plan* plan, const void* q_dev, 
  * readings of the kernels above. */
 int fca_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void* stream);
 
+/* Measurement hook, no counterpart in the reference: the next attention launch this thread
+ * makes (fca_prefix_pass, fca_suffix_pass, fca_forest_pass, or the attention launch inside
+ * fca_decode_step) records its own begin and end in the two HIP events (hipEvent_t, created
+ * by the caller with timing enabled), taken from the kernel's dispatch itself, so that
+ * hipEventElapsedTime(start, stop) is the kernel's duration and the launch is not fenced in
+ * by event records on the stream (those cost about 3 us each here).  One launch consumes the
+ * pair; NULL, NULL withdraws it. */
+int fca_time_next_attention(void* start_event, void* stop_event);
+
 #ifdef __cplusplus
 }
 #endif
