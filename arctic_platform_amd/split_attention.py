@@ -202,18 +202,33 @@ class _SplitAttention(torch.autograd.Function):
         return dq, dk, dv, None, None
 
 
-def split_attention(q, k, v, layout: SplitLayout, scale: float):
-    """Differentiable split attention: ``out [T, Hq, D]`` in deduplicated order."""
+def _refuse_unsupported(dropout, sliding_window):
+    """The trainer hands both to its attention calls on every step
+    (qwen_attention_patcher.py:1204-1206, :1224-1226); Qwen3 has no dropout in attention and
+    no window, and these kernels implement neither, so anything else is refused rather than
+    silently ignored."""
+    if dropout is not None and float(dropout) != 0.0:
+        raise NotImplementedError(f"attention dropout {dropout} is not supported by the split attention kernels (only 0.0)")
+    if sliding_window is not None:
+        raise NotImplementedError(f"sliding_window={sliding_window} is not supported by the split attention kernels (only None)")
+
+
+def split_attention(q, k, v, layout: SplitLayout, scale: float, dropout: float = 0.0, sliding_window=None):
+    """Differentiable split attention: ``out [T, Hq, D]`` in deduplicated order.  ``dropout``
+    and ``sliding_window`` are the arguments of the trainer's attention calls; only 0.0 and
+    None are accepted."""
+    _refuse_unsupported(dropout, sliding_window)
     return _SplitAttention.apply(q, k, v, layout, scale)
 
 
-def split_attention_padded(q, k, v, valid, layout: SplitLayout, scale: float):
+def split_attention_padded(q, k, v, valid, layout: SplitLayout, scale: float, dropout: float = 0.0, sliding_window=None):
     """The same attention for a deduplicated batch that still carries its padding (the
     trainer's padded variant, qwen_attention_patcher.py:881-1040, which masks the padding inside
     its two attention calls): ``q``, ``k``, ``v`` are ``[T_padded, H, D]``, ``valid`` a bool
     ``[T_padded]`` (the deduplicated attention mask, zorro_train.py:359-372), ``layout`` counts
     the valid tokens.  The valid rows are gathered, attended, and scattered back; padding rows
     of the result are zero and receive no gradient.  Differentiable."""
+    _refuse_unsupported(dropout, sliding_window)
     index = torch.nonzero(valid, as_tuple=False).squeeze(-1)
     if index.numel() != layout.num_tokens:
         raise ValueError(f"{index.numel()} valid tokens, the layout counts {layout.num_tokens}")

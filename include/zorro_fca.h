@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define FCA_VERSION 101
+#define FCA_VERSION 102
 #define FCA_BLOCK_SIZE 16
 #define FCA_MAX_LEVELS 8
 
@@ -48,6 +48,9 @@ typedef enum fca_status {
   FCA_ERR_HIP = -3
 } fca_status;
 
+/* q is bf16 and the KV cache bf16 or fp8: the products run on the bf16 matrix cores with
+ * fp32 accumulation.  An fp32 q or KV cache is refused (FCA_ERR_UNSUPPORTED) by every entry
+ * point that takes one; fp32 is available for the outputs only. */
 typedef enum fca_dtype {
   FCA_BF16 = 0,     /* q, out, KV cache */
   FCA_FP8_E4M3 = 1, /* KV cache only (OCP e4m3fn) */
@@ -148,7 +151,13 @@ int fca_build_metadata(const fca_plan* plan, const int32_t* block_table_dev, int
  * blocks of the row and no sequence got shorter; then only the private leaves and the work list are made again, at a
  * fraction of the cost.  Otherwise, or on a workspace never built or built for another
  * plan, this is fca_build_metadata.  Either way the result is valid for the given rows; a
- * kept forest may miss sharing that only a new build would find.  Header slot 14 counts
+ * kept forest may miss sharing that only a new build would find.  The comparison is by a
+ * 64-bit fingerprint of the shared block ids of each row (a sum of (id xor c) * w_j with odd
+ * weights per position): one changed id, or two ids exchanged, always change it; an arbitrary
+ * rewrite of several ids of a row goes unnoticed with probability about 2^-64 per row, in
+ * which case the row would attend to the blocks its shared nodes were built from, not the
+ * new ones.  Callers that rewrite the shared part of a row (rather than append to it) and
+ * cannot accept that call fca_build_metadata.  Header slot 14 counts
  * the updates since the last full build.  This replaces the per-step rebuild of the host-side
  * group discovery (arctic_platform/rl/zorro_train/zorro_train.py:242-285 runs once per batch). */
 int fca_update_metadata(const fca_plan* plan, const int32_t* block_table_dev, int64_t block_table_stride,

@@ -120,11 +120,18 @@ def test_config1_golden(gpu):
         seq_lens=w32.seq_lens.to(gpu),
     )
     md, out, lse = _run(w, chunk_tokens=256)
-    # the kernel sees the inputs rounded to bf16 (relative error 2^-9 per value), which moves
-    # a 64-term score by a few 1e-2 at most; the fixture itself is exact for fp32 inputs
-    err = (out.cpu().double() - torch.from_numpy(z["out"])).abs().max()
-    lerr = (lse.cpu().double() - torch.from_numpy(z["lse"])).abs().max()
-    assert err <= 2e-2 and lerr <= 5e-2, (err, lerr)
+    # The fixture holds the exact result for the generator's fp32 values; the kernels take
+    # bf16 inputs, so what they can be held to is the fixture moved by that rounding alone
+    # (the fp64 oracle on the rounded inputs says by how much: about 1e-2 on the log-sum-exp)
+    # plus the tolerance of the path on equal inputs.
+    ref_out, ref_lse = oracle_for(w)
+    gold_out, gold_lse = torch.from_numpy(z["out"]), torch.from_numpy(z["lse"])
+    moved_out = (ref_out - gold_out).abs().max()
+    moved_lse = (ref_lse - gold_lse).abs().max()
+    assert moved_lse <= 2e-2 and moved_out <= 1e-2, (moved_out, moved_lse)
+    err = (out.cpu().double() - gold_out).abs().max()
+    lerr = (lse.cpu().double() - gold_lse).abs().max()
+    assert err <= moved_out + 1e-2 and lerr <= moved_lse + 1e-3, (err, lerr, moved_out, moved_lse)
 
 
 @pytest.mark.parametrize("index", [2, 3, 4, 5])
@@ -155,6 +162,7 @@ def test_full_size_configs(gpu, index):
     _, out2, lse2 = _run(w, chunk_tokens=256, rows_per_item=96 - rows)
     assert (lse - lse2).abs().max() <= 2e-4
     assert (out.float() - out2.float()).abs().max() <= 1.6e-2
+    assert_matches_oracle(out2[sample], lse2[sample], ref_out, ref_lse, what=f"C{index} sample, {96 - rows}-row tiles")
 
 
 def test_interleaved_group_order(gpu):

@@ -43,6 +43,15 @@ CASES = [
     (8, 4, 4, 64, torch.bfloat16, 6, 2, (1, 40), (0, 20), 32, 32),  # deeper than the default level cap
     (9, 32, 2, 64, torch.bfloat16, 3, 4, (1, 120), (1, 80), 64, 64),  # GQA 16, D 64, four members per 64-row tile
     (10, 16, 2, 64, torch.float8_e4m3fn, 4, 3, (1, 100), (1, 60), 32, 64),  # fp8, D 64, 64 rows
+    # query heads per KV head that are no power of two: a tile then ends in dead rows (32 = 4 * 7 + 4)
+    (11, 28, 4, 128, torch.bfloat16, 3, 4, (1, 150), (1, 100), 64, 32),  # GQA 7
+    (12, 28, 4, 128, torch.float8_e4m3fn, 3, 4, (1, 150), (1, 100), 64, 64),  # GQA 7, fp8, 64 rows
+    (13, 12, 4, 128, torch.bfloat16, 4, 3, (1, 120), (1, 80), 32, 64),  # GQA 3, 64 rows
+    (14, 12, 4, 64, torch.float8_e4m3fn, 4, 3, (1, 120), (1, 80), 32, 32),  # GQA 3, fp8, D 64
+    (15, 10, 2, 128, torch.bfloat16, 3, 5, (1, 200), (1, 60), 96, 32),  # GQA 5: six members per 32-row tile, two dead rows
+    (16, 10, 2, 64, torch.bfloat16, 3, 5, (1, 200), (1, 60), 96, 64),  # GQA 5, D 64, 64 rows
+    (17, 24, 4, 128, torch.float8_e4m3fn, 3, 4, (1, 150), (1, 100), 128, 32),  # GQA 6, fp8
+    (18, 24, 4, 128, torch.bfloat16, 3, 4, (1, 150), (1, 100), 128, 64),  # GQA 6, 64 rows
 ]
 
 

@@ -196,6 +196,20 @@ def test_layout_for_response_rows_only():
     assert (full.kv_lim() == L.kv_lim()).all()
 
 
+def test_dropout_and_sliding_window_are_refused():
+    """The trainer passes both on every call (qwen_attention_patcher.py:1204-1206): the values
+    Qwen3 uses go through, anything else raises before a tensor is looked at."""
+    from arctic_platform_amd.split_attention import split_attention, split_attention_padded
+
+    for fn, args in ((split_attention, (None, None, None, None, 1.0)), (split_attention_padded, (None, None, None, None, None, 1.0))):
+        with pytest.raises(NotImplementedError, match="dropout"):
+            fn(*args, dropout=0.1)
+        with pytest.raises(NotImplementedError, match="sliding_window"):
+            fn(*args, sliding_window=4096)
+        with pytest.raises(NotImplementedError, match="sliding_window"):
+            fn(*args, dropout=0.0, sliding_window=128)
+
+
 def test_layout_arguments_are_checked():
     lib = _lib.load_library()
     prompt = np.asarray([4], dtype=np.int32)
