@@ -77,5 +77,6 @@ def validate_fca_support(cfg: ModelConfig, *, head_dim=None, num_q_heads=None, n
     if head_dim is not None and head_dim not in (64, 128):
         raise ValueError(f"forest cascade attention supports head_dim 64 or 128, got {head_dim}")
     if num_q_heads is not None and num_kv_heads is not None:
-        if num_q_heads % num_kv_heads or num_q_heads // num_kv_heads > 32:
-            raise ValueError("num_q_heads must be a multiple of num_kv_heads with at most 32 query heads per KV head")
+        # (a member's query heads must fit one row tile: 32 rows by default, 64 at most)
+        if num_q_heads % num_kv_heads or num_q_heads // num_kv_heads > 64:
+            raise ValueError("num_q_heads must be a multiple of num_kv_heads with at most 64 query heads per KV head")

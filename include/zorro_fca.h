@@ -61,7 +61,7 @@ typedef enum fca_dtype {
 typedef struct fca_plan {
   int32_t num_seqs;      /* S: rows of q and of the block table */
   int32_t max_blocks;    /* columns of the block table */
-  int32_t num_q_heads;   /* Hq, multiple of num_kv_heads, Hq / Hkv <= 32 */
+  int32_t num_q_heads;   /* Hq, multiple of num_kv_heads, Hq / Hkv <= rows_per_item */
   int32_t num_kv_heads;  /* Hkv */
   int32_t head_dim;      /* 64 or 128 */
   int32_t block_size;    /* must be FCA_BLOCK_SIZE */

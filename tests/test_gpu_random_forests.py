@@ -52,6 +52,9 @@ CASES = [
     (16, 10, 2, 64, torch.bfloat16, 3, 5, (1, 200), (1, 60), 96, 64),  # GQA 5, D 64, 64 rows
     (17, 24, 4, 128, torch.float8_e4m3fn, 3, 4, (1, 150), (1, 100), 128, 32),  # GQA 6, fp8
     (18, 24, 4, 128, torch.bfloat16, 3, 4, (1, 150), (1, 100), 128, 64),  # GQA 6, 64 rows
+    # more than 32 query heads per KV head: only the 64-row tiles hold a member
+    (19, 64, 1, 128, torch.bfloat16, 2, 3, (1, 100), (1, 40), 64, 64),  # GQA 64: one member fills a tile
+    (20, 96, 2, 64, torch.float8_e4m3fn, 3, 3, (1, 100), (1, 60), 32, 64),  # GQA 48, fp8, D 64: sixteen dead rows
 ]
 
 
