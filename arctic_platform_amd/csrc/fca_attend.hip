@@ -475,9 +475,10 @@ hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dty
   hipEvent_t ev_start, ev_stop;
   take_attend_timing(&ev_start, &ev_stop);
 #define FCA_LAUNCH(D_, F_, S_) \
-  hipExtLaunchKernelGGL((fca_attend64_kernel<D_, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, ev_start, ev_stop, 0, p)
+  if (ev_start) hipExtLaunchKernelGGL((fca_attend64_kernel<D_, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, ev_start, ev_stop, 0, p); \
+  else hipLaunchKernelGGL((fca_attend64_kernel<D_, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, p)
 #define FCA_PICK(D_, F_) \
-  if (stream_kv) FCA_LAUNCH(D_, F_, true); else FCA_LAUNCH(D_, F_, false)
+  if (stream_kv) { FCA_LAUNCH(D_, F_, true); } else { FCA_LAUNCH(D_, F_, false); }
   if (plan.head_dim == 128) {
     if (fp8) { FCA_PICK(128, true); } else { FCA_PICK(128, false); }
   } else {

@@ -40,7 +40,7 @@ def parse_args():
     ap.add_argument("--kv-copies", type=int, default=4, help="distinct KV caches cycled over the layers")
     ap.add_argument("--chunk", type=int, default=0, help="split-K chunk in tokens (0 = default of the configuration)")
     ap.add_argument("--rows", type=int, default=0, help="query rows per work item, 32 or 64 (0 = default)")
-    ap.add_argument("--time-every", type=int, default=0, help="time the attention launch of every n-th step with events (0 = every second step of a short run, about 24 launches of a long one)")
+    ap.add_argument("--time-every", type=int, default=0, help="time the attention launch of every n-th step with events (0 = every second step of a short run, about 24 launches of a long one; -1 = none, for runs under a profiler)")
     ap.add_argument("--cpu-seqs", type=int, default=512, help="sequences in the CPU baseline sample (0 = skip)")
     ap.add_argument("--skip-noncascade", action="store_true")
     ap.add_argument("--split-passes", action="store_true", help="also time the shared-prefix pass and the suffix pass as launches of their own (and leave them in the trace for the profiler)")
@@ -85,9 +85,11 @@ def time_steps(torch, ops, build, w, caches, md, out, lse, steps, warmup, layers
     about 5 us (measured: 305.3 against 300.5 us per step with every launch timed), so by
     default (``time_every`` = 0) every second step of a short run is timed and about 24
     launches, evenly spread, of a long one."""
-    if time_every <= 0:
+    if time_every == 0:
         time_every = max(2, steps // 24)
-    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range((steps + time_every - 1) // time_every)]
+    # (negative: no launch is timed; runs under rocprofv3 take that, the profiler has its own
+    # hold on every dispatch)
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range((steps + time_every - 1) // time_every if time_every > 0 else 0)]
     for a, b in pairs:  # a first record creates the underlying HIP events
         a.record()
         b.record()
@@ -483,7 +485,7 @@ def main():
             build_forest_metadata(w.block_table, w.seq_lens, cascade=False, out=nc, **kw)
 
         nsteps = max(args.layers, args.steps // 4)
-        nwall, _ = time_steps(torch, ops, nc_build, w, caches, nc, out, None, nsteps, args.layers, args.layers, nsteps + 1)
+        nwall, _ = time_steps(torch, ops, nc_build, w, caches, nc, out, None, nsteps, args.layers, args.layers, -1)
         nc_us = nwall / nsteps * 1e6
         noncascade["noncascade"] = {
             "us_per_step": round(nc_us, 2),
@@ -502,7 +504,7 @@ def main():
             import dataclasses
 
             w2 = dataclasses.replace(w, q=w.q[perm].contiguous(), block_table=bt2, seq_lens=sl2)
-            nwall2, _ = time_steps(torch, ops, nc2_build, w2, caches, nc2, out, None, nsteps, args.layers, args.layers, nsteps + 1)
+            nwall2, _ = time_steps(torch, ops, nc2_build, w2, caches, nc2, out, None, nsteps, args.layers, args.layers, -1)
             nc2_us = nwall2 / nsteps * 1e6
             noncascade["noncascade_interleaved"] = {
                 "us_per_step": round(nc2_us, 2),
@@ -514,7 +516,7 @@ def main():
     wall, kern_us = time_steps(torch, ops, refresh, w, caches, md, out, None, args.steps, args.warmup, args.layers, args.time_every)
     step_us = wall / args.steps * 1e6
     checked_rows = out[: max(0, min(args.cpu_seqs, w.num_seqs))].clone()  # compared with the oracle below
-    kern = sum(kern_us) / len(kern_us)
+    kern = sum(kern_us) / len(kern_us) if kern_us else float("nan")
 
     result = {
         "metric": METRIC,
@@ -561,8 +563,8 @@ def main():
             "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, chunk, rows)),
             "launches_timed": len(kern_us),
             "launch_us_mean": round(kern, 2),
-            "launch_us_min": round(min(kern_us), 2),
-            "launch_us_max": round(max(kern_us), 2),
+            "launch_us_min": round(min(kern_us), 2) if kern_us else None,
+            "launch_us_max": round(max(kern_us), 2) if kern_us else None,
         },
     }
 

@@ -325,7 +325,8 @@ int fca_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void*
  * by the caller with timing enabled), taken from the kernel's dispatch itself, so that
  * hipEventElapsedTime(start, stop) is the kernel's duration and the launch is not fenced in
  * by event records on the stream (those cost about 3 us each here).  One launch consumes the
- * pair; NULL, NULL withdraws it. */
+ * pair; NULL, NULL withdraws it.  Not for use under a profiler that intercepts dispatches
+ * (rocprofv3): it keeps its own hold on every dispatch's completion signal. */
 int fca_time_next_attention(void* start_event, void* stop_event);
 
 #ifdef __cplusplus
