@@ -18,105 +18,197 @@ __device__ inline unsigned char to_fp8(float x) {
   return (unsigned char)(__builtin_amdgcn_cvt_pk_fp8_f32(x, 0.f, 0, false) & 0xff);
 }
 
-// One thread per (token, kv head, group of XW channels), XW = channels per 16-byte K slice.
+// Both directions move 16 tokens of one KV head per workgroup through LDS, so that global
+// memory sees whole pieces on either side: the token rows [T, Hkv, D] in 16-byte pieces of
+// adjacent lanes, the K tile in 16-byte slices whose 16 tokens are adjacent lanes (256
+// contiguous bytes per slice when the tokens fill a block in order, as a prefill's do), and
+// the V tile, where a channel's 16 tokens are adjacent, in one packed store or load per
+// channel and aligned run of eight tokens.  Tokens that do not form such a run (a decode
+// step's single tokens, padding, a run that starts off an 8-token boundary) take element
+// accesses for the V tile; the result is the same either way.
+constexpr int kGroup = 16;      // tokens per workgroup
+constexpr int kRowPieces = 17;  // 16-byte pieces per staged row: D / 8 <= 16, and one of padding
+
+struct CacheStage {
+  int4 k[kGroup][kRowPieces];
+  int4 v[kGroup][kRowPieces];
+  int64_t slot[kGroup];
+  int run[2];  // tokens 8 * r .. 8 * r + 7 lie in consecutive slots from a multiple of eight on
+};
+
+__device__ inline void stage_slots(CacheStage& st, const AppendParams& p, int t0, int tid) {
+  if (tid < kGroup) st.slot[tid] = t0 + tid < p.num_tokens ? p.slot_mapping[t0 + tid] : -1;
+  __syncthreads();
+  if (tid < 2) {
+    const int64_t first = st.slot[8 * tid];
+    bool ok = first >= 0 && first % 8 == 0;
+    for (int k = 1; k < 8; ++k) ok = ok && st.slot[8 * tid + k] == first + k;
+    st.run[tid] = ok ? 1 : 0;
+  }
+}
+
 template <bool FP8>
 __global__ __launch_bounds__(256) void fca_append_kernel(AppendParams p) {
-  constexpr int XW = FP8 ? 16 : 8;
-  const int groups = p.head_dim / XW;
-  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t total = (int64_t)p.num_tokens * p.num_kv_heads * groups;
-  if (idx >= total) return;
-  const int c = (int)(idx % groups);
-  const int h = (int)((idx / groups) % p.num_kv_heads);
-  const int t = (int)(idx / ((int64_t)groups * p.num_kv_heads));
-  const int64_t slot = p.slot_mapping[t];
-  if (slot < 0) return;
-  const int64_t blk = slot / kBlock;
-  const int off = (int)(slot - blk * kBlock);
-
-  const __hip_bfloat16* ksrc = reinterpret_cast<const __hip_bfloat16*>(p.key) + (int64_t)t * p.token_stride +
-                               (int64_t)h * p.head_stride + c * XW;
-  const __hip_bfloat16* vsrc = reinterpret_cast<const __hip_bfloat16*>(p.value) + (int64_t)t * p.token_stride +
-                               (int64_t)h * p.head_stride + c * XW;
-  const int64_t tile = blk * p.cache_block_stride + (int64_t)h * p.cache_head_stride;  // elements
-  if constexpr (FP8) {
-    const float ks = p.k_scale ? p.k_scale[h] : 1.f;
-    const float vs = p.v_scale ? p.v_scale[h] : 1.f;
-    unsigned char* kdst = reinterpret_cast<unsigned char*>(p.k_cache) + tile + ((int64_t)c * kBlock + off) * XW;
-    unsigned char* vdst = reinterpret_cast<unsigned char*>(p.v_cache) + tile + (int64_t)c * XW * kBlock + off;
-    unsigned char kq[XW];
+  constexpr int XW = FP8 ? 16 : 8;  // channels per 16-byte slice of the K tile
+  const int D = p.head_dim, pieces = D / 8, slices = D / XW;
+  const int h = blockIdx.x % p.num_kv_heads, t0 = (blockIdx.x / p.num_kv_heads) * kGroup;
+  const int tid = threadIdx.x;
+  __shared__ CacheStage st;
+  stage_slots(st, p, t0, tid);
+  for (int j = tid; j < kGroup * pieces; j += 256) {
+    const int i = j / pieces, c = j - i * pieces;
+    if (t0 + i < p.num_tokens) {
+      const int64_t at = (int64_t)(t0 + i) * p.token_stride + (int64_t)h * p.head_stride + c * 8;
+      st.k[i][c] = *reinterpret_cast<const int4*>(reinterpret_cast<const __hip_bfloat16*>(p.key) + at);
+      st.v[i][c] = *reinterpret_cast<const int4*>(reinterpret_cast<const __hip_bfloat16*>(p.value) + at);
+    }
+  }
+  __syncthreads();
+  const float ks = FP8 && p.k_scale ? p.k_scale[h] : 1.f;
+  const float vs = FP8 && p.v_scale ? p.v_scale[h] : 1.f;
+  const int64_t head_at = (int64_t)h * p.cache_head_stride;  // elements
+  // K tile: slice c of token i
+  for (int j = tid; j < kGroup * slices; j += 256) {
+    const int c = j / kGroup, i = j - c * kGroup;
+    const int64_t slot = st.slot[i];
+    if (slot < 0) continue;
+    const int64_t blk = slot / kBlock;
+    const int off = (int)(slot - blk * kBlock);
+    const int64_t at = blk * p.cache_block_stride + head_at + ((int64_t)c * kBlock + off) * XW;
+    if constexpr (FP8) {
+      const __hip_bfloat16* src = reinterpret_cast<const __hip_bfloat16*>(&st.k[i][2 * c]);
+      unsigned char q[XW];
 #pragma unroll
-    for (int e = 0; e < XW; ++e) kq[e] = to_fp8(__bfloat162float(ksrc[e]) / ks);
-    *reinterpret_cast<int4*>(kdst) = *reinterpret_cast<const int4*>(kq);
+      for (int e = 0; e < XW; ++e) q[e] = to_fp8(__bfloat162float(src[e]) / ks);
+      *reinterpret_cast<int4*>(reinterpret_cast<unsigned char*>(p.k_cache) + at) = *reinterpret_cast<const int4*>(q);
+    } else {
+      *reinterpret_cast<int4*>(reinterpret_cast<__hip_bfloat16*>(p.k_cache) + at) = st.k[i][c];
+    }
+  }
+  // V tile: channel d, tokens 8 * half .. 8 * half + 7
+  for (int j = tid; j < 2 * D; j += 256) {
+    const int d = j >> 1, half = j & 1;
+    __hip_bfloat16 x[8];
 #pragma unroll
-    for (int e = 0; e < XW; ++e) vdst[e * kBlock] = to_fp8(__bfloat162float(vsrc[e]) / vs);
-  } else {
-    __hip_bfloat16* kdst = reinterpret_cast<__hip_bfloat16*>(p.k_cache) + tile + ((int64_t)c * kBlock + off) * XW;
-    __hip_bfloat16* vdst = reinterpret_cast<__hip_bfloat16*>(p.v_cache) + tile + (int64_t)c * XW * kBlock + off;
-    *reinterpret_cast<int4*>(kdst) = *reinterpret_cast<const int4*>(ksrc);
+    for (int k = 0; k < 8; ++k) x[k] = reinterpret_cast<const __hip_bfloat16*>(&st.v[8 * half + k][0])[d];
+    if (st.run[half]) {
+      const int64_t slot = st.slot[8 * half];
+      const int64_t blk = slot / kBlock;
+      const int off = (int)(slot - blk * kBlock);
+      const int64_t at = blk * p.cache_block_stride + head_at + (int64_t)d * kBlock + off;
+      if constexpr (FP8) {
+        unsigned char q[8];
 #pragma unroll
-    for (int e = 0; e < XW; ++e) vdst[e * kBlock] = vsrc[e];
+        for (int k = 0; k < 8; ++k) q[k] = to_fp8(__bfloat162float(x[k]) / vs);
+        *reinterpret_cast<uint2*>(reinterpret_cast<unsigned char*>(p.v_cache) + at) = *reinterpret_cast<const uint2*>(q);
+      } else {
+        *reinterpret_cast<int4*>(reinterpret_cast<__hip_bfloat16*>(p.v_cache) + at) = *reinterpret_cast<const int4*>(x);
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int64_t slot = st.slot[8 * half + k];
+        if (slot < 0) continue;
+        const int64_t blk = slot / kBlock;
+        const int off = (int)(slot - blk * kBlock);
+        const int64_t at = blk * p.cache_block_stride + head_at + (int64_t)d * kBlock + off;
+        if constexpr (FP8)
+          reinterpret_cast<unsigned char*>(p.v_cache)[at] = to_fp8(__bfloat162float(x[k]) / vs);
+        else
+          reinterpret_cast<__hip_bfloat16*>(p.v_cache)[at] = x[k];
+      }
+    }
   }
 }
 
 // The way back: the tokens at the given slots leave the cache as bf16 rows [T, Hkv, D] (fp8
 // tiles are multiplied by their per-head scales, i.e. the values decode attention sees).  A
-// negative slot gives a row of zeros.  Same thread mapping as the append.
+// negative slot gives a row of zeros.
 template <bool FP8>
 __global__ __launch_bounds__(256) void fca_gather_kernel(AppendParams p) {
   constexpr int XW = FP8 ? 16 : 8;
-  const int groups = p.head_dim / XW;
-  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t total = (int64_t)p.num_tokens * p.num_kv_heads * groups;
-  if (idx >= total) return;
-  const int c = (int)(idx % groups);
-  const int h = (int)((idx / groups) % p.num_kv_heads);
-  const int t = (int)(idx / ((int64_t)groups * p.num_kv_heads));
-  const int64_t slot = p.slot_mapping[t];
-  __hip_bfloat16* kdst = reinterpret_cast<__hip_bfloat16*>(const_cast<void*>(p.key)) + (int64_t)t * p.token_stride +
-                         (int64_t)h * p.head_stride + c * XW;
-  __hip_bfloat16* vdst = reinterpret_cast<__hip_bfloat16*>(const_cast<void*>(p.value)) + (int64_t)t * p.token_stride +
-                         (int64_t)h * p.head_stride + c * XW;
-  __hip_bfloat16 kv[XW], vv[XW];
-  if (slot < 0) {
+  const int D = p.head_dim, pieces = D / 8, slices = D / XW;
+  const int h = blockIdx.x % p.num_kv_heads, t0 = (blockIdx.x / p.num_kv_heads) * kGroup;
+  const int tid = threadIdx.x;
+  __shared__ CacheStage st;
+  stage_slots(st, p, t0, tid);
+  __syncthreads();
+  const float ks = FP8 && p.k_scale ? p.k_scale[h] : 1.f;
+  const float vs = FP8 && p.v_scale ? p.v_scale[h] : 1.f;
+  const int64_t head_at = (int64_t)h * p.cache_head_stride;  // elements
+  const __hip_bfloat16 zero = __float2bfloat16(0.f);
+  for (int j = tid; j < kGroup * slices; j += 256) {
+    const int c = j / kGroup, i = j - c * kGroup;
+    const int64_t slot = st.slot[i];
+    __hip_bfloat16 x[XW];
+    if (slot < 0) {
 #pragma unroll
-    for (int e = 0; e < XW; ++e) kv[e] = vv[e] = __float2bfloat16(0.f);
-  } else {
-    const int64_t blk = slot / kBlock;
-    const int off = (int)(slot - blk * kBlock);
-    const int64_t tile = blk * p.cache_block_stride + (int64_t)h * p.cache_head_stride;  // elements
-    if constexpr (FP8) {
-      const float ks = p.k_scale ? p.k_scale[h] : 1.f;
-      const float vs = p.v_scale ? p.v_scale[h] : 1.f;
-      const unsigned char* ksrc = reinterpret_cast<const unsigned char*>(p.k_cache) + tile + ((int64_t)c * kBlock + off) * XW;
-      const unsigned char* vsrc = reinterpret_cast<const unsigned char*>(p.v_cache) + tile + (int64_t)c * XW * kBlock + off;
-      unsigned char kq[XW];
-      *reinterpret_cast<int4*>(kq) = *reinterpret_cast<const int4*>(ksrc);
+      for (int e = 0; e < XW; ++e) x[e] = zero;
+    } else {
+      const int64_t blk = slot / kBlock;
+      const int off = (int)(slot - blk * kBlock);
+      const int64_t at = blk * p.cache_block_stride + head_at + ((int64_t)c * kBlock + off) * XW;
+      if constexpr (FP8) {
+        unsigned char q[XW];
+        *reinterpret_cast<int4*>(q) = *reinterpret_cast<const int4*>(reinterpret_cast<const unsigned char*>(p.k_cache) + at);
 #pragma unroll
-      for (int e = 0; e < XW; ++e) {
-        kv[e] = __float2bfloat16(__builtin_amdgcn_cvt_f32_fp8((int)kq[e], 0) * ks);
-        vv[e] = __float2bfloat16(__builtin_amdgcn_cvt_f32_fp8((int)vsrc[e * kBlock], 0) * vs);
+        for (int e = 0; e < XW; ++e) x[e] = __float2bfloat16(__builtin_amdgcn_cvt_f32_fp8((int)q[e], 0) * ks);
+      } else {
+        *reinterpret_cast<int4*>(x) = *reinterpret_cast<const int4*>(reinterpret_cast<const __hip_bfloat16*>(p.k_cache) + at);
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < XW; e += 8) st.k[i][(XW / 8) * c + e / 8] = *reinterpret_cast<const int4*>(x + e);
+  }
+  for (int j = tid; j < 2 * D; j += 256) {
+    const int d = j >> 1, half = j & 1;
+    __hip_bfloat16 x[8];
+    if (st.run[half]) {
+      const int64_t slot = st.slot[8 * half];
+      const int64_t blk = slot / kBlock;
+      const int off = (int)(slot - blk * kBlock);
+      const int64_t at = blk * p.cache_block_stride + head_at + (int64_t)d * kBlock + off;
+      if constexpr (FP8) {
+        unsigned char q[8];
+        *reinterpret_cast<uint2*>(q) = *reinterpret_cast<const uint2*>(reinterpret_cast<const unsigned char*>(p.v_cache) + at);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) x[k] = __float2bfloat16(__builtin_amdgcn_cvt_f32_fp8((int)q[k], 0) * vs);
+      } else {
+        *reinterpret_cast<int4*>(x) = *reinterpret_cast<const int4*>(reinterpret_cast<const __hip_bfloat16*>(p.v_cache) + at);
       }
     } else {
-      const __hip_bfloat16* ksrc = reinterpret_cast<const __hip_bfloat16*>(p.k_cache) + tile + ((int64_t)c * kBlock + off) * XW;
-      const __hip_bfloat16* vsrc = reinterpret_cast<const __hip_bfloat16*>(p.v_cache) + tile + (int64_t)c * XW * kBlock + off;
-      *reinterpret_cast<int4*>(kv) = *reinterpret_cast<const int4*>(ksrc);
 #pragma unroll
-      for (int e = 0; e < XW; ++e) vv[e] = vsrc[e * kBlock];
+      for (int k = 0; k < 8; ++k) {
+        const int64_t slot = st.slot[8 * half + k];
+        x[k] = zero;
+        if (slot < 0) continue;
+        const int64_t blk = slot / kBlock;
+        const int off = (int)(slot - blk * kBlock);
+        const int64_t at = blk * p.cache_block_stride + head_at + (int64_t)d * kBlock + off;
+        if constexpr (FP8)
+          x[k] = __float2bfloat16(__builtin_amdgcn_cvt_f32_fp8((int)reinterpret_cast<const unsigned char*>(p.v_cache)[at], 0) * vs);
+        else
+          x[k] = reinterpret_cast<const __hip_bfloat16*>(p.v_cache)[at];
+      }
     }
-  }
 #pragma unroll
-  for (int e = 0; e < XW; e += 8) {
-    *reinterpret_cast<int4*>(kdst + e) = *reinterpret_cast<const int4*>(kv + e);
-    *reinterpret_cast<int4*>(vdst + e) = *reinterpret_cast<const int4*>(vv + e);
+    for (int k = 0; k < 8; ++k) reinterpret_cast<__hip_bfloat16*>(&st.v[8 * half + k][0])[d] = x[k];
+  }
+  __syncthreads();
+  for (int j = tid; j < kGroup * pieces; j += 256) {
+    const int i = j / pieces, c = j - i * pieces;
+    if (t0 + i < p.num_tokens) {
+      const int64_t at = (int64_t)(t0 + i) * p.token_stride + (int64_t)h * p.head_stride + c * 8;
+      *reinterpret_cast<int4*>(reinterpret_cast<__hip_bfloat16*>(const_cast<void*>(p.key)) + at) = st.k[i][c];
+      *reinterpret_cast<int4*>(reinterpret_cast<__hip_bfloat16*>(const_cast<void*>(p.value)) + at) = st.v[i][c];
+    }
   }
 }
 
 hipError_t launch_gather(const AppendParams& p, int kv_dtype, hipStream_t stream) {
   const bool fp8 = kv_dtype == FCA_FP8_E4M3;
-  const int64_t total = (int64_t)p.num_tokens * p.num_kv_heads * (p.head_dim / (fp8 ? 16 : 8));
-  if (total == 0) return hipSuccess;
-  const int grid = (int)((total + 255) / 256);
+  if (p.num_tokens == 0) return hipSuccess;
+  const int grid = (p.num_tokens + kGroup - 1) / kGroup * p.num_kv_heads;
   if (fp8)
     hipLaunchKernelGGL(fca_gather_kernel<true>, dim3(grid), dim3(256), 0, stream, p);
   else
@@ -126,9 +218,8 @@ hipError_t launch_gather(const AppendParams& p, int kv_dtype, hipStream_t stream
 
 hipError_t launch_append(const AppendParams& p, int kv_dtype, hipStream_t stream) {
   const bool fp8 = kv_dtype == FCA_FP8_E4M3;
-  const int64_t total = (int64_t)p.num_tokens * p.num_kv_heads * (p.head_dim / (fp8 ? 16 : 8));
-  if (total == 0) return hipSuccess;
-  const int grid = (int)((total + 255) / 256);
+  if (p.num_tokens == 0) return hipSuccess;
+  const int grid = (p.num_tokens + kGroup - 1) / kGroup * p.num_kv_heads;
   if (fp8)
     hipLaunchKernelGGL(fca_append_kernel<true>, dim3(grid), dim3(256), 0, stream, p);
   else

@@ -47,6 +47,7 @@ def parse_args():
     ap.add_argument("--calibrate", action="store_true", help="also run the library's plain copy kernel over 1 GiB (counter yardstick)")
     ap.add_argument("--query-runs", default="", metavar="NxL", help="instead of a decode configuration: N sequences that each bring a run of L query tokens (a prefill chunk), e.g. 4x2048")
     ap.add_argument("--context", type=int, default=0, help="tokens already cached in front of every query run")
+    ap.add_argument("--append", default="", metavar="NxL", help="instead of a decode configuration: the cache writer and reader, N sequences that each append L tokens (512x1 = a decode step, 1x8192 = a prefill), with --context tokens cached in front")
     ap.add_argument("--split-train", default="", metavar="GxS", help="instead of a decode configuration: the trainer's split attention, forward + backward, over G prompt groups of S samples each, e.g. 8x8")
     return ap.parse_args()
 
@@ -299,6 +300,93 @@ def main_query_runs(args):
     }))
 
 
+def main_append(args):
+    """The KV-cache writer (fca_append_kv) and its way back (fca_gather_kv): N sequences append
+    L tokens each into a paged cache with a random block table.  A step is one layer's append
+    of the whole batch; bytes = what the call must move (K and V rows read, cache tiles
+    written, and the other way round for the gather).  The yardstick is the library's plain
+    copy kernel over the same number of bytes."""
+    import torch
+
+    from arctic_platform_amd import _lib
+    from arctic_platform_amd.cache import append_kv, gather_kv
+    from arctic_platform_amd.forest import _stream_ptr
+    from arctic_platform_amd.kv_layout import kv_cache_shape
+    from oracle.cache import append_kv_reference
+
+    nseq, ql = (int(v) for v in args.append.lower().split("x"))
+    ctx, hkv, d = args.context, 8, 128
+    dev = torch.device("cuda:0")
+    gen = torch.Generator().manual_seed(99)
+    max_blocks = (ctx + ql + 15) // 16
+    nblocks = nseq * max_blocks
+    table = torch.randperm(nblocks, generator=gen).view(nseq, max_blocks)
+    pos = ctx + torch.arange(ql).repeat(nseq)
+    seq = torch.arange(nseq).repeat_interleave(ql)
+    slots = (table[seq, pos // 16].to(torch.int64) * 16 + pos % 16).to(dev)
+    t = nseq * ql
+    key = torch.randn(t, hkv, d, generator=gen).to(torch.bfloat16).to(dev)
+    value = torch.randn(t, hkv, d, generator=gen).to(torch.bfloat16).to(dev)
+    lib = _lib.load_library()
+    steps, warmup = min(args.steps, 200), min(args.warmup, 20)
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(steps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e3 / steps
+
+    out = {}
+    for name, dtype in (("bf16", torch.bfloat16), ("fp8", torch.float8_e4m3fn)):
+        cache = torch.zeros(kv_cache_shape(nblocks, 16, hkv, d), dtype=torch.bfloat16, device=dev).to(dtype)
+        scales = None if dtype == torch.bfloat16 else (torch.full((hkv,), 0.05, device=dev), torch.full((hkv,), 0.04, device=dev))
+        ks, vs = scales or (None, None)
+        esz = cache.element_size()
+        moved = 2 * t * hkv * d * (2 + esz)  # K and V: bf16 rows on one side, cache elements on the other
+        us_a = timed(lambda: append_kv(key, value, cache, slots, ks, vs))
+        rows = tuple(torch.empty_like(key) for _ in range(2))
+        us_g = timed(lambda: gather_kv(cache, slots, d, ks, vs, out=rows))
+        half = (moved // 2 + 15) // 16 * 16
+        src, dst = torch.empty(half, dtype=torch.uint8, device=dev), torch.empty(half, dtype=torch.uint8, device=dev)
+        us_c = timed(lambda: _lib.check(lib.fca_calibration_copy(src.data_ptr(), dst.data_ptr(), half, _stream_ptr(dev))))
+        # the timed writer against the CPU restatement (plain loops) on a few of the blocks:
+        # every token that lands in them is written, the blocks are compared byte for byte
+        blocks = torch.unique(slots.cpu()[:: max(1, t // 6)] // 16)
+        mask = torch.isin(slots.cpu() // 16, blocks)
+        sel = mask.nonzero().squeeze(1)
+        ref = append_kv_reference(
+            torch.zeros(kv_cache_shape(nblocks, 16, hkv, d), dtype=torch.bfloat16).to(dtype), key.cpu()[sel], value.cpu()[sel], slots.cpu()[sel],
+            None if ks is None else ks.cpu(), None if vs is None else vs.cpu(),
+        )
+        ok = bool(torch.equal(cache.cpu()[:, blocks].view(torch.uint8), ref[:, blocks].view(torch.uint8)))
+        assert ok, f"{name}: the timed cache differs from the CPU restatement"
+        got_k, got_v = (r.cpu()[sel] for r in rows)
+        if dtype == torch.bfloat16:
+            assert torch.equal(got_k, key.cpu()[sel]) and torch.equal(got_v, value.cpu()[sel]), "gather does not return what was appended"
+        out[name] = {
+            "append_us": round(us_a, 2), "append_gbs": round(moved / us_a / 1e3, 1),
+            "gather_us": round(us_g, 2), "gather_gbs": round(moved / us_g / 1e3, 1),
+            "copy_same_bytes_us": round(us_c, 2), "copy_gbs": round(2 * half / us_c / 1e3, 1),
+            "bytes_moved": moved, "bit_exact_vs_cpu": ok,
+        }
+        del cache
+    print(json.dumps({
+        "metric": "KV-cache append µs/step (one layer, whole batch)", "value": out["bf16"]["append_us"], "unit": "us/step", "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": round(out["bf16"]["append_us"] / 1e3, 5), "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16 rows -> bf16 / fp8 e4m3 tiles", "data": "synthetic",
+        "config": {"workload": f"{nseq} sequences x {ql} new tokens after {ctx} cached, Hkv {hkv} / D {d}, random block table", "tokens": t},
+        "roofline": {"kernel": "fca_append_kernel", "bound": "hbm", "achieved": out["bf16"]["append_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(out["bf16"]["append_gbs"] / HBM_PEAK_GBS, 4), "traffic": None},
+        "cache_io": out, "cpu_baseline": None,
+    }))
+
+
 def main_split_train(args):
     """The trainer's split attention over a deduplicated batch: G prompt groups, S samples
     each, prompts U[1024, 4096], responses U[1, 1024] tokens, Qwen3-4B heads.  A step is one
@@ -408,6 +496,8 @@ def main():
         return main_query_runs(args)
     if args.split_train:
         return main_split_train(args)
+    if args.append:
+        return main_append(args)
     import torch
 
     from arctic_platform_amd import ops

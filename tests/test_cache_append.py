@@ -122,3 +122,49 @@ def test_append_then_attend(gpu):
         assert torch.equal(ref_cache.view(torch.uint8), w.kv_cache.cpu().view(torch.uint8))
         ref_out, ref_lse = oracle_for(w)
         assert_matches_oracle(out, lse, ref_out, ref_lse, what=f"append+attend C{index}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 128), (torch.float8_e4m3fn, 128), (torch.bfloat16, 64), (torch.float8_e4m3fn, 64)])
+@pytest.mark.parametrize("start", [0, 8, 5])
+def test_prefill_runs_take_packed_stores(gpu, dtype, d, start):
+    """Runs of consecutive tokens (a prefill chunk that starts at a block boundary, in the
+    middle of a block, and off any 8-token boundary), a padding token inside a run, and a
+    token count that is no multiple of 16: the packed V stores and the element stores must
+    leave the same bytes as the plain loops of the oracle, and the gather must read them back."""
+    from arctic_platform_amd.cache import append_kv, gather_kv
+    from arctic_platform_amd.kv_layout import kv_cache_shape
+
+    gen = torch.Generator().manual_seed(11 + start)
+    hkv, nblocks, t = 2, 12, 75
+    table = torch.randperm(nblocks, generator=gen)
+    pos = start + torch.arange(t)
+    slots = table[pos // 16].to(torch.int64) * 16 + pos % 16
+    slots[37] = -1  # padding in the middle of a run
+    key = torch.randn(t, hkv, d, generator=gen).to(torch.bfloat16)
+    value = torch.randn(t, hkv, d, generator=gen).to(torch.bfloat16)
+    fp8 = dtype == torch.float8_e4m3fn
+    ks = torch.tensor([0.02, 0.03]) if fp8 else None
+    vs = torch.tensor([0.015, 0.04]) if fp8 else None
+    base = (torch.randn(kv_cache_shape(nblocks, 16, hkv, d), generator=gen) * 0.1).to(torch.bfloat16).to(dtype)
+    want = append_kv_reference(base, key, value, slots, ks, vs)
+    cache = base.clone().to(gpu)
+    append_kv(key.to(gpu), value.to(gpu), cache, slots.to(gpu), None if ks is None else ks.to(gpu), None if vs is None else vs.to(gpu))
+    torch.cuda.synchronize()
+    assert torch.equal(cache.cpu().view(torch.uint8), want.view(torch.uint8))
+    gk, gv = gather_kv(cache, slots.to(gpu), d, None if ks is None else ks.to(gpu), None if vs is None else vs.to(gpu))
+    torch.cuda.synchronize()
+    live = slots >= 0
+    assert (gk.cpu()[~live] == 0).all() and (gv.cpu()[~live] == 0).all()
+    if not fp8:
+        assert torch.equal(gk.cpu()[live], key[live]) and torch.equal(gv.cpu()[live], value[live])
+    else:
+        x = 16
+        for tok in (0, 1, 36, 38, t - 1):
+            blk, off = divmod(int(slots[tok]), 16)
+            for h in range(hkv):
+                raw_k = want[0, blk, h].view(d // x, 16, x)[:, off].reshape(d)
+                raw_v = want[1, blk, h].view(d, 16)[:, off]
+                assert torch.equal(gk.cpu()[tok, h], (raw_k.float() * ks[h]).to(torch.bfloat16))
+                assert torch.equal(gv.cpu()[tok, h], (raw_v.float() * vs[h]).to(torch.bfloat16))
+
