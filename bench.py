@@ -606,7 +606,7 @@ def main():
     wall, kern_us = time_steps(torch, ops, refresh, w, caches, md, out, None, args.steps, args.warmup, args.layers, args.time_every)
     step_us = wall / args.steps * 1e6
     checked_rows = out[: max(0, min(args.cpu_seqs, w.num_seqs))].clone()  # compared with the oracle below
-    kern = sum(kern_us) / len(kern_us) if kern_us else float("nan")
+    kern = sum(kern_us) / len(kern_us) if kern_us else None
 
     result = {
         "metric": METRIC,
@@ -637,7 +637,7 @@ def main():
         },
         "pct_hbm_peak_unique_bytes": round(unique_bytes / (step_us * 1e-6) / 1e9 / HBM_PEAK_GBS * 100, 2),
         "breakdown_us": {
-            "attention_kernel": round(kern, 2),
+            "attention_kernel": round(kern, 2) if kern else None,
             "merge_kernel": round(merge_us, 2),
             "metadata_builder": round(build_us, 2),
             "metadata_update": round(update_us, 2),
@@ -646,13 +646,13 @@ def main():
         "roofline": {
             "kernel": "fca_attend64_kernel" if rows > 32 else "fca_attend32_kernel",
             "bound": "hbm",
-            "achieved": round(unique_bytes / (kern * 1e-6) / 1e9, 1),
+            "achieved": round(unique_bytes / (kern * 1e-6) / 1e9, 1) if kern else None,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": round(unique_bytes / (kern * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            "frac": round(unique_bytes / (kern * 1e-6) / 1e9 / HBM_PEAK_GBS, 4) if kern else None,
             "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, chunk, rows)),
             "launches_timed": len(kern_us),
-            "launch_us_mean": round(kern, 2),
+            "launch_us_mean": round(kern, 2) if kern else None,
             "launch_us_min": round(min(kern_us), 2) if kern_us else None,
             "launch_us_max": round(max(kern_us), 2) if kern_us else None,
         },
