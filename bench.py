@@ -27,6 +27,10 @@ HBM_PEAK_GBS = 8000.0
 # passes summarised in profiles/, keyed by (configuration, chunk_tokens, rows_per_item).
 # Counters cannot be read from inside this process; other shapes report null.
 MEASURED_TRAFFIC_BYTES = {(2, 1024, 32): 1_865_600_000}
+# Share of the matrix-core cycles that were busy (SQ_VALU_MFMA_BUSY_CYCLES over cycles x SIMDs)
+# in the counter passes of the same profile summary: the whole attention launch, and the
+# shared-prefix pass launched on its own (every MFMA row a live query row).
+MEASURED_MFMA_UTIL = {(2, 1024, 32): {"attention_launch": 0.074, "prefix_pass": 0.072, "source": "profiles/attend32_c2_qwen3_4b.md"}}
 METRIC = "cascade decode-attn µs/step & % of HBM peak, Qwen3-4B shape 512 seqs"
 
 
@@ -658,6 +662,7 @@ def main():
         },
     }
 
+    result["mfma_util"] = MEASURED_MFMA_UTIL.get((args.config, chunk, rows))
     if split is not None:
         result["split_passes"] = split
 
