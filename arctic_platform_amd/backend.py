@@ -153,8 +153,13 @@ class ForestCascadeMetadataBuilder:
         group = num_q_heads // num_kv_heads
         self.rows_per_item = int(cfg.get("rows_per_item", 64 if group > 32 else 32))
         # several query tokens per sequence multiply the rows of every shared node: unless the
-        # configuration fixes the tile height, such steps use 64-row tiles
-        self.rows_multi_token = int(cfg.get("rows_per_item", 64))
+        # configuration fixes the tile height, such steps use 64-row tiles (head size 256 has
+        # 32-row tiles only)
+        self.rows_multi_token = int(cfg.get("rows_per_item", 32 if head_dim == 256 else 64))
+        if head_dim == 256 and (self.rows_per_item != 32 or self.rows_multi_token != 32):
+            raise ValueError("head_dim 256 takes rows_per_item 32 only")
+        # the split attention kernels, which serve long prompts, exist for head sizes 64 and 128
+        self.prompts_on_split_kernels = head_dim in (64, 128)
         if group > self.rows_per_item:
             raise ValueError(f"{group} query heads per KV head do not fit rows_per_item={self.rows_per_item}")
         self._workspaces: collections.OrderedDict = collections.OrderedDict()
@@ -198,7 +203,7 @@ class ForestCascadeMetadataBuilder:
                 if int(ql.min()) < 0 or bool((ql > lens).any()):
                     raise ValueError("every request's query length must lie in [0, seq_len]")
         row_table = row_group = None
-        if m.max_query_len > 1 and m.query_start_loc_cpu is not None and m.seq_lens_cpu is not None and self.enabled:
+        if m.max_query_len > 1 and m.query_start_loc_cpu is not None and m.seq_lens_cpu is not None and self.enabled and self.prompts_on_split_kernels:
             # The requests at the end of the batch that are fresh prompts (the engine puts decodes
             # first): they attend on the split-attention kernels, the requests before them go on
             # as a step of their own.

@@ -74,8 +74,8 @@ def validate_fca_support(cfg: ModelConfig, *, head_dim=None, num_q_heads=None, n
         raise ValueError(f"forest cascade attention needs block_size={BLOCK_SIZE}, got {cfg.block_size}")
     if cfg.kv_cache_dtype not in ("auto", "bfloat16", "fp8", "fp8_e4m3"):
         raise ValueError(f"forest cascade attention supports bf16 and fp8 e4m3 KV caches, got {cfg.kv_cache_dtype!r}")
-    if head_dim is not None and head_dim not in (64, 128):
-        raise ValueError(f"forest cascade attention supports head_dim 64 or 128, got {head_dim}")
+    if head_dim is not None and head_dim not in (64, 128, 256):
+        raise ValueError(f"forest cascade attention supports head_dim 64, 128 or 256, got {head_dim}")
     if num_q_heads is not None and num_kv_heads is not None:
         # (a member's query heads must fit one row tile: 32 rows by default, 64 at most)
         if num_q_heads % num_kv_heads or num_q_heads // num_kv_heads > 64:

@@ -28,13 +28,15 @@ int check_plan(const fca_plan* p) {
   if (p->max_blocks < 1) return fail(FCA_ERR_INVALID_ARG, "max_blocks must be >= 1, got %d", p->max_blocks);
   if (p->block_size != FCA_BLOCK_SIZE)
     return fail(FCA_ERR_UNSUPPORTED, "block_size %d is not supported (only %d)", p->block_size, FCA_BLOCK_SIZE);
-  if (p->head_dim != 64 && p->head_dim != 128)
-    return fail(FCA_ERR_UNSUPPORTED, "head_dim %d is not supported (64 or 128)", p->head_dim);
+  if (p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256)
+    return fail(FCA_ERR_UNSUPPORTED, "head_dim %d is not supported (64, 128 or 256)", p->head_dim);
   if (p->num_kv_heads < 1 || p->num_q_heads < p->num_kv_heads || p->num_q_heads % p->num_kv_heads)
     return fail(FCA_ERR_INVALID_ARG, "num_q_heads %d must be a positive multiple of num_kv_heads %d", p->num_q_heads,
                 p->num_kv_heads);
   if (p->rows_per_item != 32 && p->rows_per_item != 64)
     return fail(FCA_ERR_UNSUPPORTED, "rows_per_item %d is not supported (32 or 64)", p->rows_per_item);
+  if (p->head_dim == 256 && p->rows_per_item != 32)
+    return fail(FCA_ERR_UNSUPPORTED, "head_dim 256 takes rows_per_item 32 only (two row tiles of accumulators do not fit)");
   if (p->num_q_heads / p->num_kv_heads > p->rows_per_item)
     return fail(FCA_ERR_UNSUPPORTED, "GQA group %d exceeds rows_per_item %d", p->num_q_heads / p->num_kv_heads,
                 p->rows_per_item);
@@ -342,7 +344,8 @@ static int cache_rows(bool gather, const void* key_dev, const void* value_dev, i
                       void* k_cache_dev, void* v_cache_dev, int64_t kv_block_stride, int64_t kv_head_stride, int32_t kv_dtype,
                       const float* k_scale_dev, const float* v_scale_dev, void* stream) {
   if (num_tokens < 0 || num_kv_heads < 1) return fail(FCA_ERR_INVALID_ARG, "num_tokens must be >= 0 and num_kv_heads >= 1");
-  if (head_dim != 64 && head_dim != 128) return fail(FCA_ERR_UNSUPPORTED, "head_dim %d is not supported (64 or 128)", head_dim);
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256)
+    return fail(FCA_ERR_UNSUPPORTED, "head_dim %d is not supported (64, 128 or 256)", head_dim);
   if (kv_dtype != FCA_BF16 && kv_dtype != FCA_FP8_E4M3)
     return fail(FCA_ERR_UNSUPPORTED, "kv_dtype %d is not supported (bf16 or fp8 e4m3)", kv_dtype);
   if (num_tokens == 0) return FCA_OK;

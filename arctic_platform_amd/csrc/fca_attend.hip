@@ -61,9 +61,12 @@ namespace fca {
 // the next item's record, block ids and member sequences; the next item's query rows and
 // first tile are requested before the current item's partial is written out, so the
 // memory pipe does not drain at item boundaries.
-template <int D, bool FP8, bool STREAM>
-__global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 64)) void fca_attend64_kernel(AttendParams p) {
-  constexpr int NRT = 2;       // row tiles of 32 query rows
+//
+// NRT = row tiles of 32 query rows per item: 2 for the 64-row items; 1 makes this the 32-row
+// kernel of head size 256, where two tile buffers and the deep lookahead of fca_attend32.hip
+// do not fit the register file.
+template <int D, bool FP8, bool STREAM, int NRT = 2>
+__global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32 * NRT)) void fca_attend64_kernel(AttendParams p) {
   constexpr int KS = D / 16;   // MFMA steps of the score product
   constexpr int NDB = D / 32;  // 32-channel blocks of the output
   using KT = KTile<D, FP8>;
@@ -466,7 +469,7 @@ hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dty
   }
   if ((int64_t)grid * kWaves > max_tickets) grid = (int)((max_tickets + kWaves - 1) / kWaves);
   if (grid < 1) grid = 1;
-  if (nrt == 1) return launch_attend32(p, plan, kv_dtype, grid, stream);
+  if (nrt == 1 && plan.head_dim != 256) return launch_attend32(p, plan, kv_dtype, grid, stream);
   // With sharing on, a launch reads every KV block once: stream it past the caches.  With
   // sharing off, sequences of a group read the same blocks again and again and the
   // memory-side cache serves the repeats, so the loads stay ordinary; likewise when query
@@ -474,15 +477,17 @@ hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dty
   const bool stream_kv = plan.max_levels > 0 && !p.kv_reread;
   hipEvent_t ev_start, ev_stop;
   take_attend_timing(&ev_start, &ev_stop);
-#define FCA_LAUNCH(D_, F_, S_) \
-  if (ev_start) hipExtLaunchKernelGGL((fca_attend64_kernel<D_, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, ev_start, ev_stop, 0, p); \
-  else hipLaunchKernelGGL((fca_attend64_kernel<D_, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, p)
-#define FCA_PICK(D_, F_) \
-  if (stream_kv) { FCA_LAUNCH(D_, F_, true); } else { FCA_LAUNCH(D_, F_, false); }
-  if (plan.head_dim == 128) {
-    if (fp8) { FCA_PICK(128, true); } else { FCA_PICK(128, false); }
+#define FCA_LAUNCH(D_, F_, S_, N_) \
+  if (ev_start) hipExtLaunchKernelGGL((fca_attend64_kernel<D_, F_, S_, N_>), dim3(grid), dim3(kThreads), 0, stream, ev_start, ev_stop, 0, p); \
+  else hipLaunchKernelGGL((fca_attend64_kernel<D_, F_, S_, N_>), dim3(grid), dim3(kThreads), 0, stream, p)
+#define FCA_PICK(D_, F_, N_) \
+  if (stream_kv) { FCA_LAUNCH(D_, F_, true, N_); } else { FCA_LAUNCH(D_, F_, false, N_); }
+  if (plan.head_dim == 256) {  // 32-row items only (checked with the plan)
+    if (fp8) { FCA_PICK(256, true, 1); } else { FCA_PICK(256, false, 1); }
+  } else if (plan.head_dim == 128) {
+    if (fp8) { FCA_PICK(128, true, 2); } else { FCA_PICK(128, false, 2); }
   } else {
-    if (fp8) { FCA_PICK(64, true); } else { FCA_PICK(64, false); }
+    if (fp8) { FCA_PICK(64, true, 2); } else { FCA_PICK(64, false, 2); }
   }
 #undef FCA_PICK
 #undef FCA_LAUNCH

@@ -27,7 +27,7 @@ __device__ inline unsigned char to_fp8(float x) {
 // step's single tokens, padding, a run that starts off an 8-token boundary) take element
 // accesses for the V tile; the result is the same either way.
 constexpr int kGroup = 16;      // tokens per workgroup
-constexpr int kRowPieces = 17;  // 16-byte pieces per staged row: D / 8 <= 16, and one of padding
+constexpr int kRowPieces = 33;  // 16-byte pieces per staged row: D / 8 <= 32, and one of padding
 
 struct CacheStage {
   int4 k[kGroup][kRowPieces];

@@ -132,12 +132,15 @@ hipError_t launch_copy(const void* src, void* dst, size_t bytes, hipStream_t str
 hipError_t launch_merge(const MergeParams& p, hipStream_t stream) {
   const int rows = p.num_seqs * p.num_q_heads;
   if (rows == 0) return hipSuccess;
-  // rows that can have many partials are merged by four lane groups each
-  const int split = p.max_partials >= 16 ? 4 : 1;
+  // rows that can have many partials are merged by four lane groups each (two at head size
+  // 256, where four would not fit a wave)
+  const int split = p.max_partials >= 16 ? (p.head_dim == 256 ? 2 : 4) : 1;
   const int per_block = kMergeThreads / (p.head_dim / 8 * split);
   const int grid = (rows + per_block - 1) / per_block;
 #define FCA_MERGE(D_, S_) hipLaunchKernelGGL((fca_merge_kernel<D_, S_>), dim3(grid), dim3(kMergeThreads), 0, stream, p)
-  if (p.head_dim == 128) {
+  if (p.head_dim == 256) {
+    if (split == 2) FCA_MERGE(256, 2); else FCA_MERGE(256, 1);
+  } else if (p.head_dim == 128) {
     if (split == 4) FCA_MERGE(128, 4); else FCA_MERGE(128, 1);
   } else {
     if (split == 4) FCA_MERGE(64, 4); else FCA_MERGE(64, 1);

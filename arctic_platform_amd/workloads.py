@@ -216,6 +216,9 @@ CONFIG_NAMES = {
     3: "C3 long-context rollout: 16 groups x 16 samples, prefix 32768, suffix U[256,4096], Hq 32 / Hkv 8 / D 128, bf16",
     4: "C4 three-level forest: system 1024, 32 segments U[2048,6144] x 8 samples, suffix U[1,2048], Hq 32 / Hkv 8 / D 128, bf16",
     5: "C5 fp8 KV Qwen3-4B decode: C2 shape, K/V fp8 e4m3 with per-KV-head scales U[0.01,0.1]",
+    # beyond the five benchmark configurations: the forest of C2 with the attention heads of the
+    # in-tree Qwen3.5 (configuration_qwen3_5_moe.py:23-35)
+    6: "C2 forest with Qwen3.5 heads: 64 groups x 8 samples, prefix U[1024,4096], suffix U[1,1024], Hq 16 / Hkv 2 / D 256, bf16",
 }
 
 
@@ -235,6 +238,9 @@ def make_config(index: int, device="cpu", *, shrink: int = 1, dtype=None, poison
         kw = dict(num_q_heads=32, num_kv_heads=8, head_dim=128, dtype=torch.bfloat16)
         if index == 5:
             kw["kv_dtype"] = torch.float8_e4m3fn
+    elif index == 6:
+        seg_len, paths = two_level_forest(gen, d(64), 8, (d(1024), d(4096)), (1, d(1024)))
+        kw = dict(num_q_heads=16, num_kv_heads=2, head_dim=256, dtype=torch.bfloat16)
     elif index == 3:
         seg_len, paths = two_level_forest(gen, d(16), 16, (d(32768), d(32768)), (d(256), d(4096)))
         kw = dict(num_q_heads=32, num_kv_heads=8, head_dim=128, dtype=torch.bfloat16)

@@ -39,7 +39,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=720)
     ap.add_argument("--warmup", type=int, default=72)
-    ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1-5 (default: the Qwen3-4B decode step)")
+    ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1-5 (default 2: the Qwen3-4B decode step); 6 = the forest of 2 with the heads of Qwen3.5 (Hq 16 / Hkv 2 / D 256)")
     ap.add_argument("--layers", type=int, default=36, help="attention layers sharing one metadata build")
     ap.add_argument("--kv-copies", type=int, default=4, help="distinct KV caches cycled over the layers")
     ap.add_argument("--chunk", type=int, default=0, help="split-K chunk in tokens (0 = default of the configuration)")
@@ -648,7 +648,7 @@ def main():
             "metadata_per_step": round(update_us / args.layers, 2),
         },
         "roofline": {
-            "kernel": "fca_attend64_kernel" if rows > 32 else "fca_attend32_kernel",
+            "kernel": "fca_attend64_kernel" if rows > 32 or w.head_dim == 256 else "fca_attend32_kernel",
             "bound": "hbm",
             "achieved": round(unique_bytes / (kern * 1e-6) / 1e9, 1) if kern else None,
             "peak": HBM_PEAK_GBS,

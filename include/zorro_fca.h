@@ -63,7 +63,7 @@ typedef struct fca_plan {
   int32_t max_blocks;    /* columns of the block table */
   int32_t num_q_heads;   /* Hq, multiple of num_kv_heads, Hq / Hkv <= rows_per_item */
   int32_t num_kv_heads;  /* Hkv */
-  int32_t head_dim;      /* 64 or 128 */
+  int32_t head_dim;      /* 64, 128 or 256 (256: rows_per_item 32 only) */
   int32_t block_size;    /* must be FCA_BLOCK_SIZE */
   int32_t chunk_tokens;  /* split-K chunk, multiple of 32 in [32, 1024] */
   int32_t rows_per_item; /* query rows stacked per work item: 32 or 64 */

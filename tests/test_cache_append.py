@@ -125,7 +125,7 @@ def test_append_then_attend(gpu):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 128), (torch.float8_e4m3fn, 128), (torch.bfloat16, 64), (torch.float8_e4m3fn, 64)])
+@pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 128), (torch.float8_e4m3fn, 128), (torch.bfloat16, 64), (torch.float8_e4m3fn, 64), (torch.bfloat16, 256), (torch.float8_e4m3fn, 256)])
 @pytest.mark.parametrize("start", [0, 8, 5])
 def test_prefill_runs_take_packed_stores(gpu, dtype, d, start):
     """Runs of consecutive tokens (a prefill chunk that starts at a block boundary, in the

@@ -55,6 +55,11 @@ CASES = [
     # more than 32 query heads per KV head: only the 64-row tiles hold a member
     (19, 64, 1, 128, torch.bfloat16, 2, 3, (1, 100), (1, 40), 64, 64),  # GQA 64: one member fills a tile
     (20, 96, 2, 64, torch.float8_e4m3fn, 3, 3, (1, 100), (1, 60), 32, 64),  # GQA 48, fp8, D 64: sixteen dead rows
+    # head size 256 (the reference's in-tree Qwen3.5: configuration_qwen3_5_moe.py:35), 32-row tiles only
+    (21, 16, 2, 256, torch.bfloat16, 3, 3, (1, 150), (1, 100), 64, 32),  # GQA 8
+    (22, 16, 4, 256, torch.float8_e4m3fn, 3, 4, (1, 150), (1, 100), 96, 32),  # GQA 4, fp8
+    (23, 4, 4, 256, torch.bfloat16, 4, 3, (1, 200), (1, 60), 1024, 32),  # MHA, one chunk per node
+    (24, 32, 2, 256, torch.float8_e4m3fn, 2, 4, (1, 300), (1, 80), 128, 32),  # GQA 16: two members per tile
 ]
 
 

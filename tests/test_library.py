@@ -62,6 +62,8 @@ def test_workspace_sizes(lib):
         (dict(rows_per_item=48), "rows_per_item"),
         (dict(max_levels=9), "max_levels"),
         (dict(head_dim=96), "head_dim"),
+        (dict(head_dim=512), "head_dim"),
+        (dict(head_dim=256, rows_per_item=64), "head_dim 256"),
         (dict(num_q_heads=30), "num_q_heads"),
     ],
 )
