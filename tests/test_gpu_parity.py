@@ -267,7 +267,7 @@ def test_error_budget_of_fp32_outputs(gpu):
     assert float((lse.cpu().double() - ref_lse).abs().max()) < 1e-5
 
 
-@pytest.mark.parametrize("index,workgroups,chunk", [(2, 8, 512), (2, 4, 1024), (5, 8, 512), (4, 16, 256)])
+@pytest.mark.parametrize("index,workgroups,chunk", [(2, 8, 512), (2, 8, 1024), (5, 8, 512), (4, 16, 256)])
 def test_items_shared_by_pairs_of_waves(gpu, index, workgroups, chunk, monkeypatch):
     """With many items per wave the 32-row kernel sets the largest items aside, one per pair of
     waves, and both waves of a pair attend it from either end until their claims meet.  A
