@@ -107,7 +107,7 @@ class ForestCascadeAttentionBackend:
 
     @staticmethod
     def get_supported_head_sizes():
-        return [64, 128]
+        return [64, 128, 256]
 
     @staticmethod
     def get_kv_cache_shape(num_blocks: int, block_size: int, num_kv_heads: int, head_size: int):

@@ -42,8 +42,14 @@ def _cache_rows(gather, key, value, kv_cache, slot_mapping, k_scale, v_scale) ->
     t, hkv, d = key.shape
     if slot_mapping.dtype != torch.int64 or slot_mapping.shape != (t,) or not slot_mapping.is_contiguous():
         raise ValueError("slot_mapping must be a contiguous int64 tensor of shape [tokens]")
-    if kv_cache.dim() != 4 or kv_cache.shape[0] != 2 or kv_cache.shape[2] != hkv or kv_cache.shape[3] != BLOCK_SIZE * d:
-        raise ValueError("kv_cache must be [2, num_blocks, num_kv_heads, 16 * head_dim]")
+    if (
+        kv_cache.dim() != 4
+        or kv_cache.shape[0] != 2
+        or kv_cache.shape[2] != hkv
+        or kv_cache.shape[3] != BLOCK_SIZE * d
+        or kv_cache.stride(3) != 1
+    ):
+        raise ValueError("kv_cache must be [2, num_blocks, num_kv_heads, 16 * head_dim] with contiguous tiles")
     if kv_cache.dtype == torch.bfloat16:
         code = _lib.FCA_BF16
     elif kv_cache.dtype == torch.float8_e4m3fn:

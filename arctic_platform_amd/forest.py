@@ -196,6 +196,8 @@ def build_forest_metadata(
     num_rows = block_table.shape[0] if row_table is None else row_table.shape[0]
     if block_table.dim() != 2 or block_table.stride(1) != 1 or seq_lens.shape != (num_rows,):
         raise ValueError("block_table must be [num_seqs, max_blocks] with contiguous rows and seq_lens one per query row")
+    if not seq_lens.is_contiguous() or seq_lens.device != block_table.device:
+        raise ValueError("seq_lens must be contiguous and on the device of block_table")
     for name, t in (("row_table", row_table), ("row_group", row_group)):
         if t is not None and (t.dtype != torch.int32 or t.shape != (num_rows,) or not t.is_contiguous() or not t.is_cuda):
             raise ValueError(f"{name} must be a contiguous int32 device tensor with one entry per query row")

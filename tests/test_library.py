@@ -112,6 +112,21 @@ def test_operators_refuse_cpu_tensors():
         )
 
 
+def test_operators_check_layouts_before_the_device():
+    import torch
+
+    from arctic_platform_amd.cache import append_kv
+    from arctic_platform_amd.forest import build_forest_metadata
+
+    table = torch.zeros(2, 4, dtype=torch.int32)
+    with pytest.raises(ValueError, match="contiguous"):  # every other length: a strided view
+        build_forest_metadata(table, torch.ones(4, dtype=torch.int32)[::2], num_q_heads=8, num_kv_heads=2, head_dim=64)
+    kv = torch.zeros(2, 4, 2, 16 * 64 * 2, dtype=torch.bfloat16)[..., ::2]  # tiles not contiguous
+    rows = torch.zeros(3, 2, 64, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="contiguous tiles"):
+        append_kv(rows, rows, kv, torch.zeros(3, dtype=torch.int64))
+
+
 def test_header_is_plain_c_and_links(tmp_path):
     """include/zorro_fca.h compiles as C99 and as C++, and a C program that only sizes a
     workspace links against the library and runs without a GPU."""
