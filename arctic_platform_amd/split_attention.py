@@ -130,6 +130,11 @@ def _check_rows(name, x, tokens):
         raise ValueError(f"the heads of a token of {name} must be contiguous")
 
 
+def _check_heads(q, k, v):
+    if k.shape != v.shape or k.shape[2] != q.shape[2]:
+        raise ValueError(f"k and v must have one shape and the head size of q, got q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
+
+
 def _plan(q, k):
     return _lib.FcaSplitPlan(q.shape[0], q.shape[1], k.shape[1], q.shape[2])
 
@@ -142,11 +147,14 @@ def split_attention_forward(q, k, v, layout: SplitLayout, scale: float, out=None
     _check_rows("q", q, rows)
     for name, x in (("k", k), ("v", v)):
         _check_rows(name, x, t)
+    _check_heads(q, k, v)
     plan = _lib.FcaSplitPlan(t, q.shape[1], k.shape[1], q.shape[2])
     if out is None:
         out = torch.empty((rows, q.shape[1], q.shape[2]), dtype=torch.bfloat16, device=q.device)
     else:
         _check_rows("out", out, rows)
+        if out.shape != q.shape:
+            raise ValueError(f"out must have the shape of q, got {tuple(out.shape)} against {tuple(q.shape)}")
     lse = torch.empty((q.shape[1], 32 * layout.num_tiles), dtype=torch.float32, device=q.device)
     if t == 0:
         return out, lse
@@ -168,6 +176,9 @@ def split_attention_backward(dout, q, k, v, out, lse, layout: SplitLayout, scale
     t = layout.num_tokens
     for name, x in (("q", q), ("k", k), ("v", v), ("out", out), ("dout", dout)):
         _check_rows(name, x, t)
+    _check_heads(q, k, v)
+    if out.shape != q.shape or dout.shape != q.shape:
+        raise ValueError("out and dout must have the shape of q")
     plan = _plan(q, k)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     for name, x in (("dq", dq), ("dk", dk), ("dv", dv)):
