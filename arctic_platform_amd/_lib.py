@@ -142,7 +142,12 @@ def load_library() -> ctypes.CDLL:
             f"{LIB_PATH} is missing: build it with `make -C {CSRC_DIR}` "
             "(or __graft_entry__.build()); there is no non-HIP fallback"
         )
-    lib = ctypes.CDLL(LIB_PATH)
+    _lib = declare_signatures(ctypes.CDLL(LIB_PATH))
+    return _lib
+
+
+def declare_signatures(lib: ctypes.CDLL) -> ctypes.CDLL:
+    """Argument and result types of every entry point of include/zorro_fca.h, set on ``lib``."""
     P, VP, I32, I64 = ctypes.POINTER, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64
     SZ = P(ctypes.c_size_t)
     lib.fca_version.restype = ctypes.c_int
@@ -177,7 +182,6 @@ def load_library() -> ctypes.CDLL:
     for name in EXPORTS:
         if name not in ("fca_version", "fca_last_error"):
             getattr(lib, name).restype = ctypes.c_int
-    _lib = lib
     return lib
 
 

@@ -1,0 +1,261 @@
+"""The HIP kernels on the CPU: the sources of ``csrc/`` are built against ``tests/emu/emu.h`` (a
+workgroup as cooperative fibers, cross-lane operations as rendezvous, MFMA and the other
+GPU-only instructions by their definition) and called through the same C ABI as the real
+library, with host pointers.  Every buffer a kernel is handed ends flush against an inaccessible
+page, so an access past its end stops the test with a segmentation fault, as it would raise a
+memory access fault on the GPU.
+
+This checks the logic of the kernels (work dealing, tile schedules, rings, masks, merges) and their
+addresses against the same oracle as the GPU tests, on small inputs.  It does not replace those
+tests: it runs none of the compiled GPU code and knows nothing of the GPU's memory model."""
+
+import ctypes
+import mmap
+import os
+import random
+import sys
+
+import pytest
+import torch
+
+from arctic_platform_amd import _lib
+from arctic_platform_amd.forest import ForestMetadata, make_plan
+from arctic_platform_amd.workloads import make_forest_workload, two_level_forest
+from oracle.cache import append_kv_reference
+from oracle.forest import canonical_nodes, discover_forest
+from oracle.split_attention import split_attention as oracle_split
+from oracle.split_attention import total_tokens
+from tests.helpers import assert_matches_oracle, oracle_for
+from tests.test_gpu_random_forests import CASES, random_forest
+
+sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "emu"))
+import build as emu_build  # noqa: E402
+
+_libc = ctypes.CDLL(None, use_errno=True)
+_mappings = []
+
+
+def guarded(t: torch.Tensor) -> torch.Tensor:
+    """A copy of ``t`` whose bytes end flush against an inaccessible page and start behind one."""
+    page = mmap.PAGESIZE
+    t = t.contiguous()
+    nbytes = t.numel() * t.element_size()
+    n16 = max(16, (nbytes + 15) // 16 * 16)
+    total = (n16 + page - 1) // page * page + 2 * page
+    m = mmap.mmap(-1, total)
+    base = ctypes.addressof(ctypes.c_char.from_buffer(m))
+    assert _libc.mprotect(ctypes.c_void_p(base), ctypes.c_size_t(page), 0) == 0
+    assert _libc.mprotect(ctypes.c_void_p(base + total - page), ctypes.c_size_t(page), 0) == 0
+    raw = torch.frombuffer(m, dtype=torch.uint8, count=n16, offset=total - page - n16)
+    g = raw[:nbytes].view(t.dtype).view(t.shape)
+    g.copy_(t)
+    _mappings.append(m)
+    return g
+
+
+@pytest.fixture(scope="module")
+def emu():
+    if emu_build.compiler() is None:
+        pytest.skip("no clang++ to build the emulation with")
+    lib = _lib.declare_signatures(ctypes.CDLL(emu_build.build()))
+    lib.emu_set_dma_late.argtypes = [ctypes.c_int]
+    lib.emu_set_dma_late.restype = None
+    os.environ["FCA_ATTEND_WORKGROUPS"] = "8"  # a grid the fibers get through in seconds
+    yield lib
+    os.environ.pop("FCA_ATTEND_WORKGROUPS", None)
+    lib.emu_set_dma_late(0)
+
+
+def _ok(lib, rc):
+    assert rc == 0, lib.fca_last_error().decode()
+
+
+# ---- decode attention: builder, attention kernels, merge ---------------------------------------
+# (seed, Hq, Hkv, D, kv dtype, samples per prompt, prefix range, suffix range, chunk, rows): six prompts,
+# long enough for the waves of eight workgroups to end on items they share
+SHARED_LAST_ITEMS = [
+    (101, 24, 4, 128, torch.float8_e4m3fn, 5, (700, 2500), (40, 700), 512, 32),
+    (102, 16, 4, 128, torch.bfloat16, 5, (700, 2500), (40, 700), 512, 32),
+    (108, 4, 1, 64, torch.bfloat16, 16, (1000, 3000), (1, 1100), 1024, 64),  # 64-row tiles, chunks of 64 blocks
+]
+
+
+def _decode(lib, w, chunk, rows, max_levels=4):
+    S, mb = w.block_table.shape
+    plan = make_plan(S, mb, w.num_q_heads, w.num_kv_heads, w.head_dim, chunk_tokens=chunk, rows_per_item=rows, max_levels=max_levels)
+    layout = _lib.FcaMetaLayout()
+    _ok(lib, lib.fca_meta_describe(ctypes.byref(plan), ctypes.byref(layout)))
+    nm, no, nl = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    _ok(lib, lib.fca_workspace_bytes(ctypes.byref(plan), ctypes.byref(nm), ctypes.byref(no), ctypes.byref(nl)))
+    meta = guarded(torch.zeros(nm.value // 4, dtype=torch.int32))
+    po = guarded(torch.full((no.value // 2,), float("nan"), dtype=torch.float16))
+    pl = guarded(torch.full((nl.value // 4,), float("nan"), dtype=torch.float32))
+    bt, sl = guarded(w.block_table), guarded(w.seq_lens)
+    q = guarded(w.q)
+    kv = guarded(w.kv_cache.view(torch.uint8)).view(w.kv_cache.dtype)
+    ks = None if w.k_scale is None else guarded(w.k_scale)
+    vs = None if w.v_scale is None else guarded(w.v_scale)
+    _ok(lib, lib.fca_build_metadata(ctypes.byref(plan), bt.data_ptr(), bt.stride(0), sl.data_ptr(), meta.data_ptr(), None))
+    md = ForestMetadata(plan=plan, layout=layout, meta=meta, partial_out=po, partial_lse=pl, block_table=bt, seq_lens=sl)
+    md.check()
+    esz = kv.element_size()
+    t = _lib.FcaTensors(
+        q.data_ptr(), q.stride(0), q.stride(1), kv.data_ptr(), kv.data_ptr() + kv.stride(0) * esz, kv.stride(1), kv.stride(2),
+        _lib.FCA_FP8_E4M3 if kv.dtype == torch.float8_e4m3fn else _lib.FCA_BF16, 0, bt.data_ptr(), bt.stride(0),
+        None if ks is None else ks.data_ptr(), None if vs is None else vs.data_ptr(), float(w.scale),
+    )
+    out = guarded(torch.full((S, w.num_q_heads, w.head_dim), float("nan")).bfloat16())
+    lse = guarded(torch.full((S, w.num_q_heads), float("nan"), dtype=torch.float32))
+    _ok(
+        lib,
+        lib.fca_decode_step(
+            ctypes.byref(plan), ctypes.byref(t), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), out.data_ptr(), out.stride(0),
+            out.stride(1), _lib.FCA_BF16, lse.data_ptr(), None,
+        ),
+    )
+    # the launch leaves its work ticket and its claim counters at zero for the next one
+    assert int(meta[layout.header + 3]) == 0
+    assert int(meta[layout.coop_ctr : layout.coop_ctr + 1024].abs().sum()) == 0
+    return md, out, lse
+
+
+def _check_nodes(md, w):
+    nodes, leaves = discover_forest(w.block_table.tolist(), w.seq_lens.tolist(), max_levels=md.plan.max_levels)
+    assert canonical_nodes(md.nodes()) == canonical_nodes(nodes)
+    assert [(l["blk_start"], l["tokens"]) for l in md.leaves()] == [(l["blk_start"], l["tokens"]) for l in leaves]
+    assert md.header()["unique_tokens"] == w.unique_tokens
+
+
+@pytest.mark.parametrize("case", [c for c in CASES if c[0] in (2, 5, 10, 12, 15, 21, 24)], ids=lambda c: f"seed{c[0]}")
+def test_random_forests_decode(emu, case):
+    seed, hq, hkv, d, kv_dtype, depth, fanout, len_range, leaf_range, chunk, rows = case
+    seg_len, paths = random_forest(random.Random(seed), depth, fanout, len_range, leaf_range)
+    w = make_forest_workload(
+        "random", seg_len, paths, torch.Generator().manual_seed(seed), num_q_heads=hq, num_kv_heads=hkv, head_dim=d,
+        kv_dtype=kv_dtype, device="cpu", poison_unused=True,
+    )
+    md, out, lse = _decode(emu, w, chunk, rows)
+    _check_nodes(md, w)
+    assert_matches_oracle(out, lse, *oracle_for(w), what=f"seed {seed}")
+
+
+@pytest.mark.parametrize("case", SHARED_LAST_ITEMS, ids=lambda c: f"seed{c[0]}")
+def test_long_items_shared_by_two_waves(emu, case):
+    seed, hq, hkv, d, kv_dtype, samples, prefix_range, suffix_range, chunk, rows = case
+    gen = torch.Generator().manual_seed(seed)
+    seg_len, paths = two_level_forest(gen, 6, samples, prefix_range, suffix_range)
+    w = make_forest_workload(
+        "two-level", seg_len, paths, gen, num_q_heads=hq, num_kv_heads=hkv, head_dim=d, kv_dtype=kv_dtype, device="cpu",
+        poison_unused=True,
+    )
+    md, out, lse = _decode(emu, w, chunk, rows)
+    # enough items for the 32-row kernel to set the largest ones aside, one per pair of waves
+    if rows == 32:
+        assert md.header()["items"] * hkv >= 16 + 3 * 32
+    _check_nodes(md, w)
+    assert_matches_oracle(out, lse, *oracle_for(w), what=f"seed {seed}")
+
+
+# ---- KV-cache append and the way back -----------------------------------------------------------
+@pytest.mark.parametrize("kv_dtype", [torch.bfloat16, torch.float8_e4m3fn])
+@pytest.mark.parametrize("d", [64, 128])
+def test_cache_append_and_gather(emu, kv_dtype, d):
+    gen = torch.Generator().manual_seed(d)
+    hkv, nblocks = 2, 9
+    # a prefill run that starts off a block boundary, single decode tokens, a padding slot
+    slots = list(range(21, 75)) + [3, 130, -1, 100]
+    tkn = len(slots)
+    key = guarded((torch.randn(tkn, hkv, d, generator=gen) * 3).bfloat16())
+    value = guarded((torch.randn(tkn, hkv, d, generator=gen) * 3).bfloat16())
+    slot_mapping = guarded(torch.tensor(slots, dtype=torch.int64))
+    cache0 = torch.zeros(2, nblocks, hkv, 16 * d, dtype=torch.bfloat16).to(kv_dtype)
+    cache = guarded(cache0.view(torch.uint8)).view(kv_dtype)
+    fp8 = kv_dtype == torch.float8_e4m3fn
+    ks = guarded(torch.tensor([0.5, 2.0])) if fp8 else None
+    vs = guarded(torch.tensor([1.0, 0.25])) if fp8 else None
+    esz = cache.element_size()
+    args = [
+        key.stride(0), key.stride(1), tkn, hkv, d, slot_mapping.data_ptr(), cache.data_ptr(), cache.data_ptr() + cache.stride(0) * esz,
+        cache.stride(1), cache.stride(2), _lib.FCA_FP8_E4M3 if fp8 else _lib.FCA_BF16, None if ks is None else ks.data_ptr(),
+        None if vs is None else vs.data_ptr(), None,
+    ]
+    _ok(emu, emu.fca_append_kv(key.data_ptr(), value.data_ptr(), *args))
+    want = append_kv_reference(cache0, key, value, slot_mapping, ks, vs)
+    assert torch.equal(cache.view(torch.uint8), want.view(torch.uint8))
+    back_k, back_v = guarded(torch.full_like(key, float("nan"))), guarded(torch.full_like(value, float("nan")))
+    _ok(emu, emu.fca_gather_kv(back_k.data_ptr(), back_v.data_ptr(), *args))
+    live = torch.tensor([s >= 0 for s in slots])
+    assert not back_k[~live].any() and not back_v[~live].any()  # a padding slot reads as zeros
+    if not fp8:
+        assert torch.equal(back_k[live], key[live]) and torch.equal(back_v[live], value[live])
+    else:  # what decode attention sees: the stored value times the scale
+        step = torch.tensor([0.5, 2.0]).view(1, 2, 1) * 32 + 1e-3  # spacing of e4m3 below 448, times the scale
+        assert ((back_k.float() - key.float()).abs()[live] <= step).all()
+
+
+# ---- split attention of the trainer --------------------------------------------------------------
+def _close(name, got, ref, scale_tol):
+    got, ref = got.detach().double(), ref.detach().double()
+    bound = scale_tol * ref.abs().max() + 2e-2 * ref.abs() + 1e-5
+    err = (got - ref).abs()
+    assert bool((err <= bound).all()), f"{name}: max |err| {err.max():.4g}, largest reference {ref.abs().max():.4g}"
+
+
+SPLIT_LAYOUTS = [
+    [(40, [20, 3])],
+    [(0, [5]), (33, [0, 64, 1])],
+    [(100, [30, 30, 30, 30])],
+    [(33, [32, 100, 1, 32]), (31, [17, 0, 45])],
+]
+
+
+@pytest.mark.parametrize("late", [False, True], ids=["loads-land-at-once", "loads-land-at-their-wait"])
+@pytest.mark.parametrize("heads", [(8, 2, 128), (4, 1, 64), (6, 2, 64)], ids=lambda h: "Hq%d-Hkv%d-D%d" % h)
+def test_split_attention_forward_and_backward(emu, heads, late):
+    """``late``: a direct-to-LDS load lands only when a wait covers it, the latest the hardware allows
+    (a missing or miscounted wait then shows as stale operands); otherwise at once, the earliest (a
+    buffer refilled while it is still being read then shows)."""
+    from arctic_platform_amd.split_attention import SplitLayout
+
+    hq, hkv, d = heads
+    emu.emu_set_dma_late(1 if late else 0)
+    for ci, layout in enumerate(SPLIT_LAYOUTS):
+        t = total_tokens(layout)
+        g = torch.Generator().manual_seed(ci)
+        q = guarded(torch.randn(t, hq, d, generator=g).bfloat16())
+        k = guarded(torch.randn(t, hkv, d, generator=g).bfloat16())
+        v = guarded(torch.randn(t, hkv, d, generator=g).bfloat16())
+        scale = d**-0.5
+        lay = guarded(torch.from_numpy(SplitLayout(layout, device="cpu").host))
+        nt = (t + 31) // 32
+        plan = _lib.FcaSplitPlan(t, hq, hkv, d)
+        fwd, bwd = ctypes.c_size_t(), ctypes.c_size_t()
+        _ok(emu, emu.fca_split_workspace_bytes(ctypes.byref(plan), ctypes.byref(fwd), ctypes.byref(bwd)))
+        ws_f, ws_b = guarded(torch.zeros(fwd.value, dtype=torch.uint8)), guarded(torch.zeros(bwd.value, dtype=torch.uint8))
+        out = guarded(torch.full((t, hq, d), float("nan")).bfloat16())
+        lse = guarded(torch.full((hq, 32 * nt), float("nan"), dtype=torch.float32))
+        _ok(
+            emu,
+            emu.fca_split_attention_forward(
+                ctypes.byref(plan), q.data_ptr(), hq * d, k.data_ptr(), hkv * d, v.data_ptr(), hkv * d, lay.data_ptr(), scale,
+                ws_f.data_ptr(), out.data_ptr(), hq * d, lse.data_ptr(), None,
+            ),
+        )
+        q64, k64, v64 = (x.double().requires_grad_() for x in (q, k, v))
+        ro, rl = oracle_split(q64, k64, v64, layout, scale)
+        _close("out", out, ro, 2e-2 / max(1.0, float(ro.detach().abs().max())))
+        torch.testing.assert_close(lse[:, :t].T.double(), rl.detach(), rtol=1e-3, atol=1e-3)
+        dout = guarded(torch.randn(t, hq, d, generator=torch.Generator().manual_seed(ci + 1)).bfloat16())
+        ro.backward(dout.double())
+        dq, dk, dv = (guarded(torch.full_like(x, float("nan"))) for x in (q, k, v))
+        _ok(
+            emu,
+            emu.fca_split_attention_backward(
+                ctypes.byref(plan), q.data_ptr(), hq * d, k.data_ptr(), hkv * d, v.data_ptr(), hkv * d, out.data_ptr(), hq * d,
+                dout.data_ptr(), hq * d, lse.data_ptr(), lay.data_ptr(), scale, ws_b.data_ptr(), dq.data_ptr(), hq * d,
+                dk.data_ptr(), hkv * d, dv.data_ptr(), hkv * d, None,
+            ),
+        )
+        _close("dq", dq, q64.grad, 1e-2)
+        _close("dk", dk, k64.grad, 1e-2)
+        _close("dv", dv, v64.grad, 1e-2)
