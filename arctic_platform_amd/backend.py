@@ -158,7 +158,8 @@ class ForestCascadeMetadataBuilder:
         self.rows_multi_token = int(cfg.get("rows_per_item", 32 if head_dim == 256 else 64))
         if head_dim == 256 and (self.rows_per_item != 32 or self.rows_multi_token != 32):
             raise ValueError("head_dim 256 takes rows_per_item 32 only")
-        # the split attention kernels, which serve long prompts, exist for head sizes 64 and 128
+        # long prompts go to the split attention kernels at head sizes 64 and 128 (at 256 those
+        # kernels run one workgroup per CU and the route has not been measured against the query-run path)
         self.prompts_on_split_kernels = head_dim in (64, 128)
         if group > self.rows_per_item:
             raise ValueError(f"{group} query heads per KV head do not fit rows_per_item={self.rows_per_item}")

@@ -416,11 +416,16 @@ namespace {
 int check_split(const fca_split_plan* p) {
   if (!p) return fail(FCA_ERR_INVALID_ARG, "plan is NULL");
   if (p->num_tokens < 0 || p->num_tokens > (1 << 30)) return fail(FCA_ERR_INVALID_ARG, "num_tokens %d is out of range", p->num_tokens);
-  if (p->head_dim != 64 && p->head_dim != 128)
-    return fail(FCA_ERR_UNSUPPORTED, "head_dim %d is not supported (64 or 128)", p->head_dim);
+  if (p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256)
+    return fail(FCA_ERR_UNSUPPORTED, "head_dim %d is not supported (64, 128 or 256)", p->head_dim);
   if (p->num_kv_heads < 1 || p->num_q_heads < p->num_kv_heads || p->num_q_heads % p->num_kv_heads)
     return fail(FCA_ERR_INVALID_ARG, "num_q_heads %d must be a positive multiple of num_kv_heads %d", p->num_q_heads,
                 p->num_kv_heads);
+  if (p->head_dim == 256 && (p->num_q_heads / p->num_kv_heads) % 4)
+    return fail(FCA_ERR_UNSUPPORTED,
+                "head_dim 256 takes a multiple of 4 query heads per KV head (got %d): only the kernels that share "
+                "their operands through LDS have an instance of that size",
+                p->num_q_heads / p->num_kv_heads);
   return FCA_OK;
 }
 int check_rows(const char* name, const void* ptr, int64_t stride, int heads, int head_dim) {

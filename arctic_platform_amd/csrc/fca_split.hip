@@ -210,9 +210,10 @@ __global__ __launch_bounds__(kThreads) void split_images_kernel(const __bf16* x,
 // tile, so they walk the same key tiles: each wave fetches a quarter of a tile's slots one
 // tile ahead, the tile is passed around through LDS (two buffers, one barrier per tile) and
 // the L1 sees a quarter of the operand traffic.  Without it (query heads per KV head not a
-// multiple of four) every wave fetches its own tiles into two register buffers.
+// multiple of four) every wave fetches its own tiles into two register buffers.  Head size
+// 256 runs one workgroup per CU (its accumulators and query rows alone take 192 registers).
 template <int D, bool BWD, bool SHARED>
-__global__ __launch_bounds__(kThreads, SHARED ? 2 : 1) void split_query_kernel(SplitParams p) {
+__global__ __launch_bounds__(kThreads, SHARED && D < 256 ? 2 : 1) void split_query_kernel(SplitParams p) {
   constexpr int KS = D / 16, NDB = D / 32, SLOTS = (BWD ? 3 : 2) * KS, PER = SLOTS / kWaves;
   __shared__ i32x4 lds[SHARED ? 2 : 1][SHARED ? SLOTS : 1][64];
   const SplitLayout L = make_split_layout(p.num_tiles);
@@ -442,7 +443,7 @@ __device__ inline void load_to_lds4(const void* src, unsigned lds_slot) {
 #define FCA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0f70 | ((n) & 15) | (((n) >> 4) << 14))
 
 template <int D, bool DK>
-__global__ __launch_bounds__(kThreads, 2) void split_key_kernel(SplitParams p) {
+__global__ __launch_bounds__(kThreads, D < 256 ? 2 : 1) void split_key_kernel(SplitParams p) {
   constexpr int KS = D / 16, NDB = D / 32, SLOTS = (DK ? 3 : 2) * KS, PER = SLOTS / kWaves;
   __shared__ i32x4 lds[kRing][SLOTS][64];
   __shared__ __attribute__((aligned(16))) float lds_stat[kRing][64];  // lse (in log2 units) of the step's 32 rows, then their delta
@@ -616,6 +617,7 @@ __global__ __launch_bounds__(kThreads) void split_reduce_kernel(const float* par
 template <typename F>
 hipError_t by_head_dim(int head_dim, F&& f) {
   if (head_dim == 128) return f(std::integral_constant<int, 128>{});
+  if (head_dim == 256) return f(std::integral_constant<int, 256>{});
   if (head_dim == 64) return f(std::integral_constant<int, 64>{});
   return hipErrorInvalidValue;
 }
@@ -643,10 +645,15 @@ hipError_t launch_split_forward(const SplitParams& p, int head_dim, hipStream_t 
   return by_head_dim(head_dim, [&](auto d) {
     constexpr int D = decltype(d)::value;
     const unsigned grid = (unsigned)p.num_tiles * ((p.num_q_heads + kWaves - 1) / kWaves);
-    if ((p.num_q_heads / p.num_kv_heads) % kWaves == 0)
+    // (head size 256 has the LDS-shared kernels only: two register buffers of 32 operand slots
+    // each do not fit a wave; such plans are refused when they are checked)
+    if ((p.num_q_heads / p.num_kv_heads) % kWaves == 0) {
       split_query_kernel<D, false, true><<<grid, kThreads, 0, stream>>>(p);
-    else
+    } else if constexpr (D < 256) {
       split_query_kernel<D, false, false><<<grid, kThreads, 0, stream>>>(p);
+    } else {
+      return hipErrorInvalidValue;
+    }
     return hipGetLastError();
   });
 }
@@ -664,10 +671,13 @@ hipError_t launch_split_backward(const SplitParams& p, int head_dim, hipStream_t
   return by_head_dim(head_dim, [&](auto d) {
     constexpr int D = decltype(d)::value;
     const unsigned qgrid = (unsigned)nt * ((p.num_q_heads + kWaves - 1) / kWaves);
-    if ((p.num_q_heads / p.num_kv_heads) % kWaves == 0)
+    if ((p.num_q_heads / p.num_kv_heads) % kWaves == 0) {
       split_query_kernel<D, true, true><<<qgrid, kThreads, 0, stream>>>(p);
-    else
+    } else if constexpr (D < 256) {
       split_query_kernel<D, true, false><<<qgrid, kThreads, 0, stream>>>(p);
+    } else {
+      return hipErrorInvalidValue;
+    }
     if (hipError_t e = hipGetLastError()) return e;
     const int ratio = p.num_q_heads / p.num_kv_heads;
     const unsigned kgrid = (unsigned)((nt + kWaves - 1) / kWaves) * p.num_kv_heads * (p.head_split ? ratio : 1);

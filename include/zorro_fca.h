@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define FCA_VERSION 102
+#define FCA_VERSION 103
 #define FCA_BLOCK_SIZE 16
 #define FCA_MAX_LEVELS 8
 
@@ -280,7 +280,7 @@ typedef struct fca_split_plan {
   int32_t num_tokens; /* T: tokens of the deduplicated batch */
   int32_t num_q_heads;
   int32_t num_kv_heads;
-  int32_t head_dim; /* 64 or 128 */
+  int32_t head_dim; /* 64, 128 or 256 (256: num_q_heads / num_kv_heads a multiple of 4) */
 } fca_split_plan;
 
 /* int32 entries of the layout array of a batch of num_tokens tokens. */

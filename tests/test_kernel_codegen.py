@@ -94,11 +94,11 @@ def test_split_attention_kernels_use_no_scratch_and_keep_their_ring_in_flight(hi
     )
     assert res.returncode == 0, res.stderr[-2000:]
     sizes = re.findall(r"ScratchSize \[bytes/lane\]: (\d+)", res.stderr)
-    assert len(sizes) >= 14 and set(sizes) == {"0"}, sizes
+    assert len(sizes) >= 19 and set(sizes) == {"0"}, sizes
     kernels = {k: v for k, v in _functions(out.read_text()).items() if "split_key_kernel" in k}
-    assert len(kernels) == 4, sorted(kernels)
+    assert len(kernels) == 6, sorted(kernels)
     for name, body in kernels.items():
-        head_dim = 128 if "ILi128E" in name else 64
+        head_dim = 256 if "ILi256E" in name else 128 if "ILi128E" in name else 64
         slots = (3 if "Lb1E" in name else 2) * head_dim // 16
         per_wave = slots // 4
         waits = [int(n) for n in re.findall(r"s_waitcnt[^\n]*vmcnt\((\d+)\)", body)]
