@@ -156,6 +156,196 @@ def test_long_items_shared_by_two_waves(emu, case):
     assert_matches_oracle(out, lse, *oracle_for(w), what=f"seed {seed}")
 
 
+# ---- query runs: rows over table rows, declared groups, causal nodes ------------------------------
+def _decode_rows(lib, table, row_table, row_lens, row_group, q, cache, k_scale, v_scale, *, chunk, rows, levels):
+    """Build with a row table and attend; returns (metadata, out, lse)."""
+    i32 = lambda v: guarded(torch.tensor(v, dtype=torch.int32))
+    hq, d = q.shape[1], q.shape[2]
+    hkv = cache.shape[2]
+    R = len(row_table)
+    plan = make_plan(R, table.shape[1], hq, hkv, d, chunk_tokens=chunk, rows_per_item=rows, max_levels=levels)
+    layout = _lib.FcaMetaLayout()
+    _ok(lib, lib.fca_meta_describe(ctypes.byref(plan), ctypes.byref(layout)))
+    nm, no, nl = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    _ok(lib, lib.fca_workspace_bytes(ctypes.byref(plan), ctypes.byref(nm), ctypes.byref(no), ctypes.byref(nl)))
+    meta = guarded(torch.zeros(nm.value // 4, dtype=torch.int32))
+    po = guarded(torch.full((no.value // 2,), float("nan"), dtype=torch.float16))
+    pl = guarded(torch.full((nl.value // 4,), float("nan"), dtype=torch.float32))
+    bt, rt, rl = guarded(table), i32(row_table), i32(row_lens)
+    rg = None if row_group is None else i32(row_group)
+    _ok(
+        lib,
+        lib.fca_build_metadata_rows(
+            ctypes.byref(plan), bt.data_ptr(), bt.stride(0), bt.shape[0], rt.data_ptr(), None if rg is None else rg.data_ptr(),
+            rl.data_ptr(), meta.data_ptr(), 0, None,
+        ),
+    )
+    md = ForestMetadata(plan=plan, layout=layout, meta=meta, partial_out=po, partial_lse=pl, block_table=bt, seq_lens=rl, row_table=rt, row_group=rg)
+    md.check()
+    qg = guarded(q)
+    kv = guarded(cache.view(torch.uint8)).view(cache.dtype)
+    ks = None if k_scale is None else guarded(k_scale)
+    vs = None if v_scale is None else guarded(v_scale)
+    esz = kv.element_size()
+    t = _lib.FcaTensors(
+        qg.data_ptr(), qg.stride(0), qg.stride(1), kv.data_ptr(), kv.data_ptr() + kv.stride(0) * esz, kv.stride(1), kv.stride(2),
+        _lib.FCA_FP8_E4M3 if kv.dtype == torch.float8_e4m3fn else _lib.FCA_BF16, 1, bt.data_ptr(), bt.stride(0),
+        None if ks is None else ks.data_ptr(), None if vs is None else vs.data_ptr(), float(d**-0.5),
+    )
+    out = guarded(torch.full((R, hq, d), float("nan")).bfloat16())
+    lse = guarded(torch.full((R, hq), float("nan"), dtype=torch.float32))
+    _ok(
+        lib,
+        lib.fca_decode_step(
+            ctypes.byref(plan), ctypes.byref(t), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), out.data_ptr(), out.stride(0),
+            out.stride(1), _lib.FCA_BF16, lse.data_ptr(), None,
+        ),
+    )
+    return md, out, lse
+
+
+def _check_rows(md, out, lse, table, row_table, row_lens, row_group, q, cache, k_scale, v_scale, levels, what):
+    from oracle.attention import flat_decode_attention
+
+    nodes, leaves = discover_forest(table.tolist(), row_lens, max_levels=levels, row_table=row_table, row_group=row_group)
+    assert canonical_nodes(md.nodes()) == canonical_nodes(nodes), what
+    key = lambda ns: sorted((tuple(sorted(n["members"])), n["tokens"], n["causal"]) for n in ns)
+    assert key(md.nodes()) == key(nodes), what
+    assert [l["tokens"] for l in md.leaves()] == [l["tokens"] for l in leaves], what
+    ref_out, ref_lse = flat_decode_attention(
+        q, cache, table[torch.tensor(row_table)], torch.tensor(row_lens), q.shape[2] ** -0.5, k_scale, v_scale
+    )
+    assert_matches_oracle(out, lse, ref_out, ref_lse, what=what)
+
+
+def test_query_runs_and_speculative_verify(emu):
+    from tests.test_query_runs import CASES as RUN_CASES
+    from tests.test_query_runs import _batch_on_gpu, run_rows
+
+    for seed, hq, hkv, d, kv_dtype, rows, chunk, batch, share in RUN_CASES:
+        table, cache, q, k_scale, v_scale, max_blocks = _batch_on_gpu("cpu", seed, batch, hq, hkv, d, kv_dtype, share)
+        row_table, row_lens, row_group = run_rows(batch, max_blocks)
+        for levels in (4, 0):
+            md, out, lse = _decode_rows(emu, table, row_table, row_lens, row_group, q, cache, k_scale, v_scale, chunk=chunk, rows=rows, levels=levels)
+            _check_rows(md, out, lse, table, row_table, row_lens, row_group, q, cache, k_scale, v_scale, levels, f"query runs {seed}, levels {levels}")
+
+
+def test_random_batches_of_query_rows(emu):
+    """Random head sizes, GQA groups (7 among them), tile heights, fp8, chunks, level caps, prefix
+    sharing between sequences, runs tiled per block, no declarations, arbitrary declarations across
+    sequences, rows in shuffled order."""
+    from arctic_platform_amd.kv_layout import kv_cache_shape
+    from tests.test_query_runs import run_rows
+
+    for seed in range(25):
+        rng = random.Random(seed)
+        gen = torch.Generator().manual_seed(seed)
+        d, hkv, g = rng.choice([64, 128]), rng.choice([1, 2, 4]), rng.choice([1, 2, 4, 7, 8, 16])
+        hq, rows_per_item, fp8 = hkv * g, rng.choice([32, 64]), rng.random() < 0.3
+        chunk, levels = rng.choice([32, 64, 128, 1024]), rng.choice([0, 1, 2, 4, 8])
+        nseq, max_blocks = rng.randint(1, 10), rng.randint(2, 14)
+        nblocks = nseq * max_blocks + 2
+        table = torch.randperm(nblocks, generator=gen).to(torch.int32)[: nseq * max_blocks].view(nseq, max_blocks).clone()
+        for s in range(1, nseq):  # a sequence may start with the blocks of an earlier one
+            if rng.random() < 0.6:
+                t, k = rng.randrange(s), rng.randint(1, max_blocks)
+                table[s, :k] = table[t, :k]
+        batch = []
+        for s in range(nseq):
+            ql = min(rng.choice([1, 1, 1, 2, 3, 5, 16, 17, 33]), max_blocks * 16)
+            batch.append((rng.randint(0, max_blocks * 16 - ql), ql))
+        mode = rng.choice(["tiles", "tiles", "none", "odd"])
+        row_table, row_lens, row_group = run_rows(batch, max_blocks)
+        if mode == "odd":  # arbitrary declarations, across sequences too
+            row_group = [rng.randrange(3) for _ in row_group]
+        if rng.random() < 0.3:  # rows in any order: declared tiles then are not runs of adjacent rows
+            perm = list(range(len(row_table)))
+            rng.shuffle(perm)
+            row_table, row_lens, row_group = ([v[i] for i in perm] for v in (row_table, row_lens, row_group))
+        groups = None if mode == "none" else row_group
+        cache = torch.randn(kv_cache_shape(nblocks, 16, hkv, d), generator=gen)
+        k_scale = v_scale = None
+        if fp8:
+            k_scale = torch.rand(hkv, generator=gen) * 0.09 + 0.01
+            v_scale = torch.rand(hkv, generator=gen) * 0.09 + 0.01
+            cache = (cache * 20).clamp(-448, 448).to(torch.float8_e4m3fn)
+        else:
+            cache = cache.to(torch.bfloat16)
+        q = torch.randn(len(row_table), hq, d, generator=gen).to(torch.bfloat16)
+        what = f"seed {seed}: D {d}, Hq {hq} / Hkv {hkv}, rows {rows_per_item}, fp8 {fp8}, chunk {chunk}, levels {levels}, {mode}"
+        md, out, lse = _decode_rows(emu, table, row_table, row_lens, groups, q, cache, k_scale, v_scale, chunk=chunk, rows=rows_per_item, levels=levels)
+        _check_rows(md, out, lse, table, row_table, row_lens, groups, q, cache, k_scale, v_scale, levels, what)
+
+
+def test_row_arrays_from_query_start_loc(emu):
+    from tests.test_query_runs import run_rows
+
+    rng = random.Random(9)
+    for max_blocks in (7, 64):
+        batch = []
+        for _ in range(rng.randint(1, 40)):
+            ql = rng.choice([1, 1, 1, 2, 5, 16, 17, 40])
+            batch.append((rng.randint(0, max_blocks * 16 - ql), ql))
+        want = run_rows(batch, max_blocks)
+        n = len(want[0])
+        starts = guarded(torch.tensor([0] + [q for _, q in batch]).cumsum(0).to(torch.int32))
+        seq_lens = guarded(torch.tensor([c + q for c, q in batch], dtype=torch.int32))
+        got = [guarded(torch.full((n,), -7, dtype=torch.int32)) for _ in range(3)]
+        _ok(emu, emu.fca_rows_from_query_runs(starts.data_ptr(), seq_lens.data_ptr(), len(batch), n, max_blocks, got[0].data_ptr(), got[1].data_ptr(), got[2].data_ptr(), None))
+        for g, w in zip(got, want):
+            assert g.tolist() == w
+
+
+# ---- metadata updates between the steps of a decode loop ------------------------------------------
+def test_update_keeps_the_forest_and_detects_a_changed_batch(emu):
+    from arctic_platform_amd.workloads import make_config
+    from tests.test_metadata_update import _grown, _semantics
+
+    w = make_config(2, device="cpu", shrink=8)
+    S = w.block_table.shape[0]
+    wide = torch.zeros(S, w.block_table.shape[1] + 8, dtype=torch.int32)
+    wide[:, : w.block_table.shape[1]] = w.block_table
+    w.block_table = wide
+    plan = make_plan(S, wide.shape[1], w.num_q_heads, w.num_kv_heads, w.head_dim, chunk_tokens=64, rows_per_item=32, max_levels=4)
+    layout = _lib.FcaMetaLayout()
+    _ok(emu, emu.fca_meta_describe(ctypes.byref(plan), ctypes.byref(layout)))
+    nm = ctypes.c_size_t()
+    _ok(emu, emu.fca_workspace_bytes(ctypes.byref(plan), ctypes.byref(nm), None, None))
+
+    def build(bt, sl, meta=None, update=False):
+        bt, sl = guarded(bt), guarded(sl)
+        if meta is None:
+            meta = guarded(torch.zeros(nm.value // 4, dtype=torch.int32))
+        entry = emu.fca_update_metadata if update else emu.fca_build_metadata
+        _ok(emu, entry(ctypes.byref(plan), bt.data_ptr(), bt.stride(0), sl.data_ptr(), meta.data_ptr(), None))
+        md = ForestMetadata(plan=plan, layout=layout, meta=meta, partial_out=None, partial_lse=None, block_table=bt, seq_lens=sl)
+        md.check()
+        return md
+
+    md = build(w.block_table, w.seq_lens)
+    assert md.header()["updates"] == 0
+    gen = torch.Generator().manual_seed(5)
+    # 1 token (most rows stay inside their block), 17 (every row crosses a block), 70 (chunk counts change)
+    for n, steps in enumerate((1, 17, 70)):
+        bt, sl = _grown(w, steps, gen)
+        md = build(bt, sl, md.meta, update=True)
+        assert md.header()["updates"] == n + 1, "the update fell back to a full build"
+        assert _semantics(md) == _semantics(build(bt, sl))
+        w.block_table, w.seq_lens = bt, sl
+    # sequence 3 leaves its group: one of its shared blocks becomes a private copy
+    bt = w.block_table.clone()
+    bt[3, 2] = int(bt.max()) + 1
+    md = build(bt, w.seq_lens, md.meta, update=True)
+    assert md.header()["updates"] == 0
+    assert _semantics(md) == _semantics(build(bt, w.seq_lens))
+    # a new request in an old slot: shorter than the prefix its row shared
+    sl = w.seq_lens.clone()
+    sl[5] = 20
+    md = build(bt, sl, md.meta, update=True)
+    assert md.header()["updates"] == 0
+    assert _semantics(md) == _semantics(build(bt, sl))
+
+
 # ---- KV-cache append and the way back -----------------------------------------------------------
 @pytest.mark.parametrize("kv_dtype", [torch.bfloat16, torch.float8_e4m3fn])
 @pytest.mark.parametrize("d", [64, 128])
