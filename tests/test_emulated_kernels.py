@@ -156,6 +156,48 @@ def test_long_items_shared_by_two_waves(emu, case):
     assert_matches_oracle(out, lse, *oracle_for(w), what=f"seed {seed}")
 
 
+def test_entry_points_agree(emu):
+    """Shared and private items as launches of their own plus the merge, the decode step on the
+    library's own partial buffers, sharing switched off, fp32 output into a strided tensor: all
+    give the decode step's result (the first three bit for bit)."""
+    seed, hq, hkv, d, kv_dtype, samples, prefix_range, suffix_range, chunk, rows = SHARED_LAST_ITEMS[1]
+    gen = torch.Generator().manual_seed(seed)
+    seg_len, paths = two_level_forest(gen, 3, 4, (200, 900), (10, 300))
+    w = make_forest_workload("two-level", seg_len, paths, gen, num_q_heads=hq, num_kv_heads=hkv, head_dim=d, kv_dtype=kv_dtype, device="cpu", poison_unused=True)
+    md, out, lse = _decode(emu, w, 128, 32)
+    S = w.block_table.shape[0]
+    plan, meta = md.plan, md.meta
+    q, kv, bt = guarded(w.q), guarded(w.kv_cache), md.block_table
+    t = _lib.FcaTensors(
+        q.data_ptr(), q.stride(0), q.stride(1), kv.data_ptr(), kv.data_ptr() + kv.stride(0) * 2, kv.stride(1), kv.stride(2), _lib.FCA_BF16, 0,
+        bt.data_ptr(), bt.stride(0), None, None, float(w.scale),
+    )
+    fresh = lambda: (guarded(torch.full((S, hq, d), float("nan")).bfloat16()), guarded(torch.full((S, hq), float("nan"), dtype=torch.float32)))
+    # 1. two passes and the merge
+    po = guarded(torch.full_like(md.partial_out, float("nan")))
+    pl = guarded(torch.full_like(md.partial_lse, float("nan")))
+    o1, l1 = fresh()
+    _ok(emu, emu.fca_prefix_pass(ctypes.byref(plan), ctypes.byref(t), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), None))
+    _ok(emu, emu.fca_suffix_pass(ctypes.byref(plan), ctypes.byref(t), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), None))
+    _ok(emu, emu.fca_merge(ctypes.byref(plan), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), o1.data_ptr(), o1.stride(0), o1.stride(1), _lib.FCA_BF16, l1.data_ptr(), None))
+    assert torch.equal(o1.view(torch.int16), out.view(torch.int16)) and torch.equal(l1, lse)
+    # 2. the library's own partial buffers
+    o2, l2 = fresh()
+    _ok(emu, emu.fca_decode_step_static(ctypes.byref(plan), ctypes.byref(t), meta.data_ptr(), o2.data_ptr(), o2.stride(0), o2.stride(1), _lib.FCA_BF16, l2.data_ptr(), None))
+    assert torch.equal(o2.view(torch.int16), out.view(torch.int16)) and torch.equal(l2, lse)
+    # 3. fp32 output into every second row of a wider tensor
+    wide = guarded(torch.full((S, 2, hq, d), float("nan"), dtype=torch.float32))
+    o3 = wide[:, 1]
+    _ok(emu, emu.fca_decode_step(ctypes.byref(plan), ctypes.byref(t), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1), _lib.FCA_F32, None, None))
+    assert torch.isnan(wide[:, 0]).all()
+    torch.testing.assert_close(o3.bfloat16().float(), out.float(), rtol=1e-2, atol=1e-2)
+    # 4. sharing off: the same kernels as a plain paged decode attention
+    md0, out0, lse0 = _decode(emu, w, 128, 32, max_levels=0)
+    assert md0.header()["shared_items"] == 0
+    assert_matches_oracle(out0, lse0, *oracle_for(w), what="sharing off")
+    torch.testing.assert_close(lse0, lse, rtol=0, atol=1e-4)
+
+
 # ---- query runs: rows over table rows, declared groups, causal nodes ------------------------------
 def _decode_rows(lib, table, row_table, row_lens, row_group, q, cache, k_scale, v_scale, *, chunk, rows, levels):
     """Build with a row table and attend; returns (metadata, out, lse)."""
