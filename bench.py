@@ -44,6 +44,7 @@ def parse_args():
     ap.add_argument("--kv-copies", type=int, default=4, help="distinct KV caches cycled over the layers")
     ap.add_argument("--chunk", type=int, default=0, help="split-K chunk in tokens (0 = default of the configuration)")
     ap.add_argument("--rows", type=int, default=0, help="query rows per work item, 32 or 64 (0 = default)")
+    ap.add_argument("--kv-reread", action="store_true", help="keep the KV loads cacheable instead of streaming them (worth a try where a shared node fills more than one row tile, e.g. --config 3 --rows 32: its row tiles then read the same blocks at nearly the same time)")
     ap.add_argument("--time-every", type=int, default=0, help="time the attention launch of every n-th step with events (0 = every second step of a short run, about 24 launches of a long one; -1 = none, for runs under a profiler)")
     ap.add_argument("--cpu-seqs", type=int, default=512, help="sequences in the CPU baseline sample (0 = skip)")
     ap.add_argument("--skip-noncascade", action="store_true")
@@ -516,6 +517,8 @@ def main():
     chunk = args.chunk or 1024
     rows = args.rows or (64 if args.config == 3 else 32)
     kw = dict(num_q_heads=w.num_q_heads, num_kv_heads=w.num_kv_heads, head_dim=w.head_dim, chunk_tokens=chunk, rows_per_item=rows)
+    if args.kv_reread:
+        kw["kv_reread"] = True
     out = torch.empty_like(w.q)
 
     md = build_forest_metadata(w.block_table, w.seq_lens, **kw)
