@@ -165,3 +165,90 @@ def test_header_is_plain_c_and_links(tmp_path):
     assert int(out[0]) >= 1 and int(out[2]) == (512 * (320 * 16 // 1024 + 6) * 32 + 32 * 1024) * 128 * 2
     # lim of every key: a prompt token is seen up to the end of its group, a response token up to its own end
     assert [int(x) for x in out[4:16]] == [6, 6, 6, 5, 5, 6, 12, 12, 12, 12, 12, 12]
+
+
+def test_attention_and_cache_entry_points_refuse_bad_tensors(lib):
+    """Every check that stands between a caller's mistake and a kernel launch: the calls below
+    must come back with an error code and a message, never reach a launch (there is no GPU here:
+    a call that got that far would report a HIP error instead)."""
+    plan = make_plan(4, 8, 32, 8, 128)
+    ok = 1 << 20  # an address that is 16-byte aligned and never dereferenced
+
+    def tensors(**kw):
+        t = _lib.FcaTensors(ok, 32 * 128, 128, ok, ok + (1 << 16), 8 * 16 * 128, 16 * 128, _lib.FCA_BF16, 0, ok, 8, None, None, 0.1)
+        for k, v in kw.items():
+            setattr(t, k, v)
+        return t
+
+    def decode(t, meta=ok, po=ok, pl=ok, out=ok, out_dtype=_lib.FCA_BF16):
+        return lib.fca_decode_step(ctypes.byref(plan), ctypes.byref(t), meta, po, pl, out, 32 * 128, 128, out_dtype, None, None)
+
+    cases = [
+        (tensors(q_dev=ok + 2), "q must be 16-byte aligned"),
+        (tensors(q_head_stride=100), "strides that are multiples of 8"),
+        (tensors(k_cache_dev=ok + 8), "KV cache planes must be 16-byte aligned"),
+        (tensors(kv_dtype=7), "kv_dtype 7"),
+        (tensors(kv_head_stride=16 * 64), "smaller than one tile"),
+        (tensors(block_table_stride=4), "block_table_stride 4 is smaller than max_blocks 8"),
+        (tensors(block_table_dev=None), "must be non-NULL"),
+    ]
+    for t, fragment in cases:
+        assert decode(t) < 0
+        assert fragment in lib.fca_last_error().decode(), (fragment, lib.fca_last_error())
+    assert decode(tensors(), po=ok + 4) == -1 and "partial workspaces must be 16-byte aligned" in lib.fca_last_error().decode()
+    assert decode(tensors(), meta=None) == -1
+    # the merge: output type and pointers
+    assert lib.fca_merge(ctypes.byref(plan), ok, ok, ok, ok, 32 * 128, 128, 5, None, None) == -2
+    assert lib.fca_merge(ctypes.byref(plan), ok, ok, ok, None, 32 * 128, 128, _lib.FCA_BF16, None, None) == -1
+    # the static entry point refuses plans whose partial rows do not fit its array
+    big = make_plan(4096, 512, 32, 8, 128, chunk_tokens=32)
+    assert lib.fca_decode_step_static(ctypes.byref(big), ctypes.byref(tensors(block_table_stride=512)), ok, ok, 32 * 128, 128, _lib.FCA_BF16, None, None) == -2
+    assert "static scratch" in lib.fca_last_error().decode()
+    # cache writer and reader
+    def append(fn=lib.fca_append_kv, key=ok, tstride=8 * 128, hstride=128, tokens=3, heads=8, d=128, slots=ok, kc=ok, bstride=8 * 16 * 128, hs=16 * 128, dt=_lib.FCA_BF16):
+        return fn(key, ok, tstride, hstride, tokens, heads, d, slots, kc, ok + (1 << 16), bstride, hs, dt, None, None, None)
+
+    assert append(tokens=0) == 0  # nothing to do
+    for kw, fragment in [
+        (dict(tokens=-1), "num_tokens must be >= 0"),
+        (dict(d=96), "head_dim 96"),
+        (dict(dt=3), "kv_dtype 3"),
+        (dict(key=ok + 8), "key and value must be 16-byte aligned"),
+        (dict(tstride=100), "multiples of 8"),
+        (dict(slots=None), "must be non-NULL"),
+        (dict(hs=16 * 64), "at least one tile"),
+    ]:
+        for fn in (lib.fca_append_kv, lib.fca_gather_kv):
+            assert append(fn=fn, **kw) < 0
+            assert fragment in lib.fca_last_error().decode(), (fragment, lib.fca_last_error())
+    # the measurement hook takes its events as a pair
+    assert lib.fca_time_next_attention(ok, None) == -1
+    assert lib.fca_time_next_attention(None, None) == 0
+    assert lib.fca_calibration_copy(ok, ok + 4, 64, None) == -1
+
+
+def test_split_entry_points_refuse_bad_tensors(lib):
+    ok = 1 << 20
+    plan = _lib.FcaSplitPlan(100, 8, 2, 128)
+
+    def forward(q=ok, qs=8 * 128, ks=2 * 128, layout=ok, scale=0.1, ws=ok, out_stride=8 * 128, lse=ok):
+        return lib.fca_split_attention_forward(ctypes.byref(plan), q, qs, ok, ks, ok, 2 * 128, layout, scale, ws, ok, out_stride, lse, None)
+
+    for kw, fragment in [
+        (dict(scale=0.0), "scale must be positive"),
+        (dict(q=ok + 2), "q must be 16-byte aligned"),
+        (dict(qs=7 * 128), "at least heads * head_dim"),
+        (dict(ks=100), "k must be"),
+        (dict(out_stride=4), "out must be"),
+        (dict(layout=None), "layout, workspace and lse"),
+        (dict(lse=ok + 4), "layout, workspace and lse"),
+    ]:
+        assert forward(**kw) < 0
+        assert fragment in lib.fca_last_error().decode(), (fragment, lib.fca_last_error())
+    empty = _lib.FcaSplitPlan(0, 8, 2, 128)
+    assert lib.fca_split_attention_forward(ctypes.byref(empty), None, 0, None, 0, None, 0, None, 0.1, None, None, 0, None, None) == 0
+    bad = _lib.FcaSplitPlan(-1, 8, 2, 128)
+    assert lib.fca_split_workspace_bytes(ctypes.byref(bad), None, None) == -1
+    args = [ok, 8 * 128, ok, 2 * 128, ok, 2 * 128, ok, 8 * 128, ok, 8 * 128, ok, ok, 0.1, ok, ok, 8 * 128, ok, 2 * 128, ok, 2 * 128, None]
+    args[16] = 100  # dk stride (every call in this file must fail a check: with a GPU present a call that passed them all would launch on made-up addresses)
+    assert lib.fca_split_attention_backward(ctypes.byref(plan), *args) == -1 and "dk must be" in lib.fca_last_error().decode()
