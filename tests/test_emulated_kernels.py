@@ -442,7 +442,9 @@ SPLIT_LAYOUTS = [
 
 
 @pytest.mark.parametrize("late", [False, True], ids=["loads-land-at-once", "loads-land-at-their-wait"])
-@pytest.mark.parametrize("heads", [(8, 2, 128), (4, 1, 64), (6, 2, 64), (8, 2, 256)], ids=lambda h: "Hq%d-Hkv%d-D%d" % h)
+# (with as many KV heads as query heads dK and dV are stored straight from the accumulators; a small batch
+# with fewer KV heads forms them per query head and sums the slices)
+@pytest.mark.parametrize("heads", [(8, 2, 128), (4, 1, 64), (6, 2, 64), (8, 2, 256), (2, 2, 64)], ids=lambda h: "Hq%d-Hkv%d-D%d" % h)
 def test_split_attention_forward_and_backward(emu, heads, late):
     """``late``: a direct-to-LDS load lands only when a wait covers it, the latest the hardware allows
     (a missing or miscounted wait then shows as stale operands); otherwise at once, the earliest (a
