@@ -84,6 +84,8 @@ class FcaTensors(ctypes.Structure):
         ("k_scale_dev", ctypes.c_void_p),
         ("v_scale_dev", ctypes.c_void_p),
         ("softmax_scale", ctypes.c_float),
+        ("reproducible", ctypes.c_int32),
+        ("max_workgroups", ctypes.c_int32),
     ]
 
 

@@ -76,11 +76,13 @@ def parse_forest_cascade_configs(value) -> dict:
     or a dict.  Known keys: chunk_tokens, rows_per_item, max_levels, enable, rebuild_every,
     kv_reread (true: keep KV loads cacheable, for batches whose shared prompts carry more
     query rows than one row tile holds, e.g. more than rows_per_item / (Hq / Hkv) samples per
-    prompt; false: stream; absent: decided per step from the query lengths)."""
+    prompt; false: stream; absent: decided per step from the query lengths), reproducible
+    (true: no work item is cut between two waves at a point that depends on timing, so equal
+    inputs give equal bits, at a few per cent of the speed)."""
     if value is None or value == "":
         return {}
     cfg = json.loads(value) if isinstance(value, str) else dict(value)
-    unknown = set(cfg) - {"chunk_tokens", "rows_per_item", "max_levels", "enable", "rebuild_every", "kv_reread"}
+    unknown = set(cfg) - {"chunk_tokens", "rows_per_item", "max_levels", "enable", "rebuild_every", "kv_reread", "reproducible"}
     if unknown:
         raise ValueError(f"unknown forest_cascade_attn_configs keys: {sorted(unknown)}")
     return cfg
@@ -150,6 +152,8 @@ class ForestCascadeMetadataBuilder:
         self.max_levels = int(cfg.get("max_levels", 4))
         self.rebuild_every = max(1, int(cfg.get("rebuild_every", 32)))
         self.kv_reread = None if cfg.get("kv_reread") is None else bool(cfg["kv_reread"])
+        # the same bits from every launch on the same inputs (no item attended by two waves together)
+        self.reproducible = bool(cfg.get("reproducible", False))
         group = num_q_heads // num_kv_heads
         self.rows_per_item = int(cfg.get("rows_per_item", 64 if group > 32 else 32))
         # several query tokens per sequence multiply the rows of every shared node: unless the
@@ -260,7 +264,14 @@ class ForestCascadeMetadataBuilder:
             # one row per query token: the row of its sequence, cut off behind the token itself;
             # the tokens of a run that fall into one cache block form a tile
             starts = m.query_start_loc[: m.num_reqs + 1]
-            num_tokens = m.num_actual_tokens if m.num_actual_tokens is not None else int(starts[-1])
+            # (the count comes from the host side: reading it off the device tensor would stall
+            # the scheduler step on a device -> host copy and cannot be captured in a graph)
+            if m.num_actual_tokens is not None:
+                num_tokens = int(m.num_actual_tokens)
+            elif m.query_start_loc_cpu is not None:
+                num_tokens = int(m.query_start_loc_cpu[m.num_reqs])
+            else:
+                raise ValueError("a step with query runs needs num_actual_tokens or query_start_loc_cpu (the number of query tokens)")
             rows_key = (num_tokens, "rows")
             if rows_key not in self._workspaces:
                 self._keep(rows_key, tuple(torch.empty(num_tokens, dtype=torch.int32, device=bt.device) for _ in range(3)))
@@ -294,6 +305,8 @@ class ForestCascadeMetadataBuilder:
             # plain decode, and stream.
             kv_reread=m.max_query_len > 2 if self.kv_reread is None else self.kv_reread,
         )
+        if forest is not None:  # (a test double of the builder returns none)
+            forest.reproducible = self.reproducible
         self._keep(key, forest)
         return ForestCascadeMetadata(forest=forest, slot_mapping=m.slot_mapping[:num_tokens], num_decode_tokens=num_tokens)
 

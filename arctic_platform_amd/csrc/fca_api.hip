@@ -1,6 +1,7 @@
 // C ABI of libzorro_fca.so (declared in include/zorro_fca.h): argument checks and launches.
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 
@@ -69,6 +70,7 @@ int check_tensors(const fca_plan* p, const fca_tensors* t) {
   if (t->block_table_stride < p->max_blocks)
     return fail(FCA_ERR_INVALID_ARG, "block_table_stride %lld is smaller than max_blocks %d",
                 (long long)t->block_table_stride, p->max_blocks);
+  if (t->max_workgroups < 0) return fail(FCA_ERR_INVALID_ARG, "max_workgroups must be >= 0, got %d", t->max_workgroups);
   return FCA_OK;
 }
 
@@ -100,9 +102,15 @@ fca::AttendParams attend_params(const fca_plan* p, const fca_tensors* t, void* m
   a.max_partials = (int32_t)L.max_partials;
   a.select = select;
   a.kv_reread = t->kv_reread;
-  a.coop_ctr = a.meta + L.coop_ctr;
+  // items attended by two waves together: not when the caller wants the same bits from every launch
+  a.coop_ctr = t->reproducible ? nullptr : a.meta + L.coop_ctr;
   a.coop_pairs = (int32_t)fca::coop_pairs_for(*p, L);
-  a.coop_row0 = (int64_t)p->num_seqs * L.max_partials * p->num_q_heads;
+  // a launch over the private items alone takes the second set of back rows (and tags that
+  // say so), so that the two passes in front of one merge do not write the same rows
+  const int region = select == 2 ? 1 : 0;
+  a.coop_tag0 = region * 32 * a.coop_pairs;
+  a.coop_row0 = (int64_t)p->num_seqs * L.max_partials * p->num_q_heads + a.coop_tag0;
+  a.max_workgroups = t->max_workgroups;
   return a;
 }
 
@@ -140,6 +148,7 @@ int run_merge(const fca_plan* p, const void* meta, const void* po, const float* 
   m.head_dim = p->head_dim;
   m.max_partials = (int32_t)L.max_partials;
   m.coop_row0 = (int64_t)p->num_seqs * L.max_partials * p->num_q_heads;
+  m.coop_rows = 32 * fca::kCoopRegions * fca::coop_pairs_for(*p, L);
   m.out_dtype = out_dtype;
   // whole 16-byte stores when every 8-channel group of out is 16-byte aligned
   const int64_t esz = out_dtype == FCA_F32 ? 4 : 2;
@@ -159,8 +168,9 @@ const char* fca_last_error(void) { return g_error; }
 int fca_workspace_bytes(const fca_plan* plan, size_t* meta_bytes, size_t* partial_out_bytes, size_t* partial_lse_bytes) {
   if (int rc = check_plan(plan)) return rc;
   const fca::MetaLayout L = fca::make_layout(*plan);
-  // one row per (partial slot, query head), then 32 rows per pair of waves that may share an item
-  const size_t rows = (size_t)plan->num_seqs * (size_t)L.max_partials * plan->num_q_heads + 32 * (size_t)fca::coop_pairs_for(*plan, L);
+  // one row per (partial slot, query head), then two sets of 32 rows per pair of waves that may share an item
+  const size_t rows = (size_t)plan->num_seqs * (size_t)L.max_partials * plan->num_q_heads +
+                      32 * (size_t)fca::kCoopRegions * (size_t)fca::coop_pairs_for(*plan, L);
   if (meta_bytes) *meta_bytes = (size_t)L.total * sizeof(int32_t);
   if (partial_out_bytes) *partial_out_bytes = rows * plan->head_dim * 2;  // half
   if (partial_lse_bytes) *partial_lse_bytes = rows * 2 * sizeof(float);    // {lse, scale}
@@ -398,6 +408,16 @@ int fca_gather_kv(void* key_dev, void* value_dev, int64_t token_stride, int64_t 
 int fca_time_next_attention(void* start_event, void* stop_event) {
   if ((start_event == nullptr) != (stop_event == nullptr))
     return fail(FCA_ERR_INVALID_ARG, "start and stop events come as a pair (both or neither)");
+  // A profiler that intercepts dispatches (rocprofv3 announces its tool library in the
+  // environment of the program it starts) holds every dispatch's completion signal itself:
+  // a launch that also carries events is refused there, not tried.
+  static const bool profiled = [] {
+    const char* tool = getenv("ROCP_TOOL_LIBRARIES");
+    return tool != nullptr && tool[0] != 0;
+  }();
+  if (profiled && start_event)
+    return fail(FCA_ERR_UNSUPPORTED, "launches are not timed with events under a profiler (ROCP_TOOL_LIBRARIES is set): "
+                                     "take the kernel durations from its trace");
   fca::set_attend_timing(static_cast<hipEvent_t>(start_event), static_cast<hipEvent_t>(stop_event));
   return FCA_OK;
 }

@@ -461,12 +461,9 @@ hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dty
                               ((int64_t)plan.max_blocks * kBlock / plan.chunk_tokens + plan.max_levels + 2) *
                               plan.num_kv_heads;
   int grid = cached_cu_count() * workgroups_per_cu(plan.head_dim, fp8, plan.rows_per_item);
-  // FCA_ATTEND_WORKGROUPS caps the grid (tests use it to reach the many-items-per-wave
-  // schedules of a large batch with a small one)
-  if (const char* cap = getenv("FCA_ATTEND_WORKGROUPS")) {
-    const int n = atoi(cap);
-    if (n > 0 && n < grid) grid = n;
-  }
+  // the caller's cap: leaves CUs to other streams (and brings the many-items-per-wave
+  // schedules of a large batch to a small one)
+  if (p.max_workgroups > 0 && p.max_workgroups < grid) grid = p.max_workgroups;
   if ((int64_t)grid * kWaves > max_tickets) grid = (int)((max_tickets + kWaves - 1) / kWaves);
   if (grid < 1) grid = 1;
   if (nrt == 1 && plan.head_dim != 256) return launch_attend32(p, plan, kv_dtype, grid, stream);

@@ -18,7 +18,11 @@ constexpr int kHeaderInts = 16;
 // Items that two waves of the 32-row attention kernel attend together (one from either end):
 // at most this many pairs of waves, one claim counter each in the metadata workspace, and 32
 // partial rows each behind the ordinary partial rows for the wave that comes from the back.
+// There are kCoopRegions such sets of rows: a launch over the private items only writes the
+// second one, so that it leaves the rows of a launch over the shared items alone when both
+// precede one merge.
 constexpr int kCoopMaxPairs = 1024;
+constexpr int kCoopRegions = 2;
 constexpr int kCoopMinPairs = 4;  // pairs of 32-token tiles an item needs to be shared
 
 enum HeaderSlot {
@@ -181,7 +185,9 @@ struct AttendParams {
   // buffers have rows for, and the first of those rows
   int32_t* coop_ctr;
   int32_t coop_pairs;
-  int64_t coop_row0;
+  int32_t max_workgroups;  // > 0: cap of the grid
+  int32_t coop_tag0;  // added to the tags of this launch: 32 * coop_pairs * (set of back rows it writes)
+  int64_t coop_row0;  // first back row of this launch
 };
 
 struct MergeParams {
@@ -195,6 +201,7 @@ struct MergeParams {
   int32_t num_seqs, num_q_heads, head_dim, max_partials, out_dtype;
   int32_t vector_out;  // out rows allow 16-byte stores
   int64_t coop_row0;   // first of the partial rows written by waves that took a shared item from the back
+  int64_t coop_rows;   // how many such rows the partial buffers hold: a tag that points past them is not followed
 };
 
 struct AppendParams {

@@ -37,6 +37,7 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
   // One online pass (running maximum, rescaled sum): the loads of successive partials do
   // not depend on each other, so unrolling keeps several of them in flight.
   float m = -INFINITY, wsum = 0.f;
+  int stray = 0;  // a row scale pointed outside the rows set aside for second partials
   float acc[V];
 #pragma unroll
   for (int e = 0; e < V; ++e) acc[e] = 0.f;
@@ -65,10 +66,18 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
     const unsigned tag = sbits & 0x007fffffu;
     take(ls.x, __uint_as_float(sbits & 0xff800000u), o);
     if (tag) {
-      const int64_t br = p.coop_row0 + (int64_t)(tag - 32);  // tag = (pair + 1) * 32 + row of the tile
-      const float2 bls = lse_scale[br];
-      const f16x8 bo = *reinterpret_cast<const f16x8*>(rows + br * D + sub * V);
-      take(bls.x, bls.y, bo);
+      // tag = 32 * (pair + 1) + row of the tile, counted over the sets of back rows.  Only a
+      // buffer no attention launch has written (or one written for another plan) holds a tag
+      // that points anywhere else: it is not followed, and the output row leaves as NaN.
+      const int64_t rel = (int64_t)tag - 32;
+      if (rel >= 0 && rel < p.coop_rows) {
+        const int64_t br = p.coop_row0 + rel;
+        const float2 bls = lse_scale[br];
+        const f16x8 bo = *reinterpret_cast<const f16x8*>(rows + br * D + sub * V);
+        take(bls.x, __uint_as_float(__float_as_uint(bls.y) & 0xff800000u), bo);
+      } else {
+        stray = 1;
+      }
     }
   }
   // combine the shares: the same update with a whole running result in place of one partial
@@ -82,12 +91,13 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
 #pragma unroll
     for (int e = 0; e < V; ++e) acc[e] = acc[e] * keep + __shfl_xor(acc[e], off) * take;
     m = m_new;
+    stray |= __shfl_xor(stray, off);
   }
   if (!live_row || share != 0) return;
   // The builder records input it had to clamp (a length beyond the block table, a row-table
   // entry out of range, overflowing lists) in the header and carries on; results made from
   // such metadata leave as NaN so that they cannot pass for attention over a cut-off sequence.
-  const bool flagged = p.header[H_ERROR] != 0;
+  const bool flagged = p.header[H_ERROR] != 0 || stray != 0;
   const float inv = flagged ? __builtin_nanf("") : (wsum > 0.f ? 1.f / wsum : 0.f);
   const int64_t o = (int64_t)s * p.out_seq_stride + (int64_t)hq * p.out_head_stride + sub * V;
   if (p.out_dtype == FCA_F32) {

@@ -41,6 +41,11 @@ class ForestMetadata:
     # The tiles of a long query run read the same blocks one after the other: the attention
     # calls then keep their KV loads cacheable (fca_tensors.kv_reread).
     kv_reread: bool = False
+    # Attention launches never let two waves attend one item together (fca_tensors.reproducible):
+    # the same bits from every launch on the same inputs, at a few per cent of the speed.
+    reproducible: bool = False
+    # Cap of the attention grid in workgroups, 0 = the whole GPU (fca_tensors.max_workgroups).
+    max_workgroups: int = 0
 
     # ---- inspection (synchronises; not for the decode loop) -------------------------
     def header(self) -> dict:
@@ -229,7 +234,9 @@ def build_forest_metadata(
             layout=layout,
             meta=torch.zeros(nm.value // 4, dtype=torch.int32, device=dev),
             partial_out=torch.empty(no.value // 2, dtype=torch.float16, device=dev),
-            partial_lse=torch.empty(nl.value // 4, dtype=torch.float32, device=dev),
+            # (zeros: a merge that runs before any attention pass has written the buffers then
+            # finds plain empty rows, not row scales that point somewhere)
+            partial_lse=torch.zeros(nl.value // 4, dtype=torch.float32, device=dev),
             block_table=block_table,
             seq_lens=seq_lens,
             row_table=row_table,

@@ -64,6 +64,8 @@ def _tensors(q, kv_cache, meta: ForestMetadata, scale, k_scale, v_scale) -> _lib
         k_scale.data_ptr() if k_scale is not None else None,
         v_scale.data_ptr() if v_scale is not None else None,
         float(scale),
+        1 if meta.reproducible else 0,
+        int(meta.max_workgroups),
     )
 
 

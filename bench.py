@@ -45,7 +45,7 @@ def parse_args():
     ap.add_argument("--chunk", type=int, default=0, help="split-K chunk in tokens (0 = default of the configuration)")
     ap.add_argument("--rows", type=int, default=0, help="query rows per work item, 32 or 64 (0 = default)")
     ap.add_argument("--kv-reread", action="store_true", help="keep the KV loads cacheable instead of streaming them (worth a try where a shared node fills more than one row tile, e.g. --config 3 --rows 32: its row tiles then read the same blocks at nearly the same time)")
-    ap.add_argument("--time-every", type=int, default=0, help="time the attention launch of every n-th step with events (0 = every second step of a short run, about 24 launches of a long one; -1 = none, for runs under a profiler)")
+    ap.add_argument("--time-every", type=int, default=0, help="time the attention launch of every n-th step with events (0 = every second step of a short run, about 24 launches of a long one; -1 = none; under rocprofv3 no launch is timed whatever this says)")
     ap.add_argument("--cpu-seqs", type=int, default=512, help="sequences in the CPU baseline sample (0 = skip)")
     ap.add_argument("--skip-noncascade", action="store_true")
     ap.add_argument("--split-passes", action="store_true", help="also time the shared-prefix pass and the suffix pass as launches of their own (and leave them in the trace for the profiler)")
@@ -85,16 +85,22 @@ def run_steps(torch, ops, build, w, caches, md, out, lse, steps, layers, timed_e
     return used
 
 
+def under_profiler():
+    """rocprofv3 names its tool library in the environment of the program it starts."""
+    return bool(os.environ.get("ROCP_TOOL_LIBRARIES"))
+
+
 def time_steps(torch, ops, build, w, caches, md, out, lse, steps, warmup, layers, time_every=0):
     """Wall time of ``steps`` steps after ``warmup`` untimed ones, and the durations of the
     attention launches inside the timed region.  A launch that records events costs the step
     about 5 us (measured: 305.3 against 300.5 us per step with every launch timed), so by
     default (``time_every`` = 0) every second step of a short run is timed and about 24
     launches, evenly spread, of a long one."""
+    if under_profiler():
+        time_every = -1  # the profiler has its own hold on every dispatch: its trace has the durations
     if time_every == 0:
         time_every = max(2, steps // 24)
-    # (negative: no launch is timed; runs under rocprofv3 take that, the profiler has its own
-    # hold on every dispatch)
+    # (negative: no launch is timed)
     pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range((steps + time_every - 1) // time_every if time_every > 0 else 0)]
     for a, b in pairs:  # a first record creates the underlying HIP events
         a.record()
@@ -552,6 +558,8 @@ def main():
 
     build_us = ev_time(build)
     update_us = ev_time(refresh)
+    # the merge reads what an attention pass wrote: one whole step first, then the merge on its own
+    ops.forest_cascade_decode(w.q, w.kv_cache, md, w.scale, w.k_scale, w.v_scale, out=out, return_lse=False)
     merge_us = ev_time(lambda: ops.merge_partials(md, w.q, out=out, return_lse=False))
 
     split = None
@@ -658,7 +666,7 @@ def main():
             "unit": "GB/s",
             "frac": round(unique_bytes / (kern * 1e-6) / 1e9 / HBM_PEAK_GBS, 4) if kern else None,
             "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, chunk, rows)),
-            "launches_timed": len(kern_us),
+            "launches_timed": len(kern_us),  # 0 under rocprofv3: the trace has the durations
             "launch_us_mean": round(kern, 2) if kern else None,
             "launch_us_min": round(min(kern_us), 2) if kern_us else None,
             "launch_us_max": round(max(kern_us), 2) if kern_us else None,

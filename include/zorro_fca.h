@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define FCA_VERSION 103
+#define FCA_VERSION 104
 #define FCA_BLOCK_SIZE 16
 #define FCA_MAX_LEVELS 8
 
@@ -89,6 +89,11 @@ typedef struct fca_tensors {
   const float* k_scale_dev;    /* [Hkv] dequant scales for fp8 caches, or NULL (= 1) */
   const float* v_scale_dev;
   float softmax_scale;         /* usually head_dim ** -0.5 */
+  int32_t reproducible;        /* non-zero: no work item is attended by two waves together, so where an
+                                  item is cut, and with it the last bit of a few outputs, never depends
+                                  on timing: two launches on the same inputs give the same bits */
+  int32_t max_workgroups;      /* > 0: the attention launch uses at most this many workgroups (of four
+                                  waves), leaving the rest of the GPU to work on other streams; 0: all */
 } fca_tensors;
 
 /* Offsets (in int32 units) of the arrays inside a built metadata workspace, for
@@ -131,10 +136,12 @@ const char* fca_last_error(void);
 /* Workspace sizes for a plan: metadata (int32 arrays) and the two partial buffers.  A
  * partial output row is D half-precision values times one power-of-two scale per row:
  * partial_out is half [rows, D], partial_lse is fp32 [rows, 2] = {natural-log lse, scale},
- * rows = S * max_partials * Hq plus 32 for each pair of waves that may attend an item
+ * rows = S * max_partials * Hq plus 2 x 32 for each pair of waves that may attend an item
  * together (at most 1024 pairs; the second wave of a pair writes there, and the scale of
- * the first wave's row carries the place in its mantissa bits).  Both are opaque to the
- * caller: written by the passes, read by the merge. */
+ * the first wave's row carries the place in its mantissa bits; fca_suffix_pass writes the
+ * second set of 32, every other pass the first, so a prefix and a suffix pass in front of one
+ * merge do not meet).  Both are opaque to the caller: written by the passes, read by the
+ * merge. */
 int fca_workspace_bytes(const fca_plan* plan, size_t* meta_bytes, size_t* partial_out_bytes, size_t* partial_lse_bytes);
 int fca_meta_describe(const fca_plan* plan, fca_meta_layout* layout);
 
@@ -221,7 +228,13 @@ int fca_forest_pass(const fca_plan* plan, const fca_tensors* t, void* meta_dev,
                     void* partial_out_dev, float* partial_lse_dev, void* stream);
 /* Log-sum-exp merge of each sequence's partials (online max / rescaled sum as in
  * arctic_platform/model/implementations/qwen35/models/layers/lm_head.py:190-202).
- * out: [S, Hq, D] bf16 or f32; lse: fp32 [S, Hq], natural log, may be NULL. */
+ * out: [S, Hq, D] bf16 or f32; lse: fp32 [S, Hq], natural log, may be NULL.
+ * Precondition: since the metadata was last built or updated, fca_forest_pass, or both
+ * fca_prefix_pass and fca_suffix_pass, have run on these partial buffers, so that every slot
+ * the metadata counts for a row has been written.  On buffers that hold anything else the
+ * merge stays inside the buffers (a row scale whose mantissa bits point past the rows set
+ * aside for second partials is not followed, and that output row becomes NaN) but its
+ * results mean nothing. */
 int fca_merge(const fca_plan* plan, const void* meta_dev, const void* partial_out_dev,
               const float* partial_lse_dev, void* out_dev, int64_t out_seq_stride, int64_t out_head_stride,
               int32_t out_dtype, float* lse_dev, void* stream);
@@ -325,8 +338,10 @@ int fca_calibration_copy(const void* src_dev, void* dst_dev, size_t bytes, void*
  * by the caller with timing enabled), taken from the kernel's dispatch itself, so that
  * hipEventElapsedTime(start, stop) is the kernel's duration and the launch is not fenced in
  * by event records on the stream (those cost about 3 us each here).  One launch consumes the
- * pair; NULL, NULL withdraws it.  Not for use under a profiler that intercepts dispatches
- * (rocprofv3): it keeps its own hold on every dispatch's completion signal. */
+ * pair; NULL, NULL withdraws it.  Not for use under a profiler that intercepts dispatches:
+ * it keeps its own hold on every dispatch's completion signal.  Under rocprofv3 (recognised
+ * by ROCP_TOOL_LIBRARIES in the environment) a non-NULL pair is refused with
+ * FCA_ERR_UNSUPPORTED and the next launch is an ordinary one. */
 int fca_time_next_attention(void* start_event, void* stop_event);
 
 #ifdef __cplusplus

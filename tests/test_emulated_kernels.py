@@ -31,6 +31,7 @@ from tests.test_gpu_random_forests import CASES, random_forest
 sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "emu"))
 import build as emu_build  # noqa: E402
 
+EMU_WORKGROUPS = 8  # fca_tensors.max_workgroups: a grid the fibers get through in seconds
 _libc = ctypes.CDLL(None, use_errno=True)
 _mappings = []
 
@@ -60,9 +61,7 @@ def emu():
     lib = _lib.declare_signatures(ctypes.CDLL(emu_build.build()))
     lib.emu_set_dma_late.argtypes = [ctypes.c_int]
     lib.emu_set_dma_late.restype = None
-    os.environ["FCA_ATTEND_WORKGROUPS"] = "8"  # a grid the fibers get through in seconds
     yield lib
-    os.environ.pop("FCA_ATTEND_WORKGROUPS", None)
     lib.emu_set_dma_late(0)
 
 
@@ -102,7 +101,7 @@ def _decode(lib, w, chunk, rows, max_levels=4):
     t = _lib.FcaTensors(
         q.data_ptr(), q.stride(0), q.stride(1), kv.data_ptr(), kv.data_ptr() + kv.stride(0) * esz, kv.stride(1), kv.stride(2),
         _lib.FCA_FP8_E4M3 if kv.dtype == torch.float8_e4m3fn else _lib.FCA_BF16, 0, bt.data_ptr(), bt.stride(0),
-        None if ks is None else ks.data_ptr(), None if vs is None else vs.data_ptr(), float(w.scale),
+        None if ks is None else ks.data_ptr(), None if vs is None else vs.data_ptr(), float(w.scale), 0, EMU_WORKGROUPS,
     )
     out = guarded(torch.full((S, w.num_q_heads, w.head_dim), float("nan")).bfloat16())
     lse = guarded(torch.full((S, w.num_q_heads), float("nan"), dtype=torch.float32))
@@ -170,7 +169,7 @@ def test_entry_points_agree(emu):
     q, kv, bt = guarded(w.q), guarded(w.kv_cache), md.block_table
     t = _lib.FcaTensors(
         q.data_ptr(), q.stride(0), q.stride(1), kv.data_ptr(), kv.data_ptr() + kv.stride(0) * 2, kv.stride(1), kv.stride(2), _lib.FCA_BF16, 0,
-        bt.data_ptr(), bt.stride(0), None, None, float(w.scale),
+        bt.data_ptr(), bt.stride(0), None, None, float(w.scale), 0, EMU_WORKGROUPS,
     )
     fresh = lambda: (guarded(torch.full((S, hq, d), float("nan")).bfloat16()), guarded(torch.full((S, hq), float("nan"), dtype=torch.float32)))
     # 1. two passes and the merge
@@ -196,6 +195,109 @@ def test_entry_points_agree(emu):
     assert md0.header()["shared_items"] == 0
     assert_matches_oracle(out0, lse0, *oracle_for(w), what="sharing off")
     torch.testing.assert_close(lse0, lse, rtol=0, atol=1e-4)
+
+
+def test_separate_passes_with_shared_items_equal_the_fused_step(emu):
+    """Shared and private items as launches of their own, on a batch where both launches end on
+    items that pairs of waves attend together: each launch has rows of its own for the second
+    partials, so the suffix launch leaves the prefix launch's alone and the merge finds both."""
+    hq, hkv, d, chunk = 16, 4, 128, 512
+    gen = torch.Generator().manual_seed(311)
+    seg_len, paths = two_level_forest(gen, 12, 5, (700, 2500), (230, 900))
+    w = make_forest_workload("two-level", seg_len, paths, gen, num_q_heads=hq, num_kv_heads=hkv, head_dim=d, device="cpu", poison_unused=True)
+    md, out, lse = _decode(emu, w, chunk, 32)
+    waves = 4 * EMU_WORKGROUPS
+    items = md.items()
+    for shared in (True, False):
+        own = [it for it in items if it["shared"] == shared]
+        assert len(own) * hkv >= waves // 2 + 3 * waves, "too few items for the launch to set some aside"
+        assert max(it["tok_len"] for it in own[: waves // 2 // hkv + 1]) >= 7 * 32 - 31, "no item long enough to be shared"
+    S = w.block_table.shape[0]
+    plan, meta, bt = md.plan, md.meta, md.block_table
+    q, kv = guarded(w.q), guarded(w.kv_cache)
+    t = _lib.FcaTensors(
+        q.data_ptr(), q.stride(0), q.stride(1), kv.data_ptr(), kv.data_ptr() + kv.stride(0) * 2, kv.stride(1), kv.stride(2), _lib.FCA_BF16, 0,
+        bt.data_ptr(), bt.stride(0), None, None, float(w.scale), 0, EMU_WORKGROUPS,
+    )
+    po = guarded(torch.full_like(md.partial_out, float("nan")))
+    pl = guarded(torch.full_like(md.partial_lse, float("nan")))
+    o1 = guarded(torch.full((S, hq, d), float("nan")).bfloat16())
+    l1 = guarded(torch.full((S, hq), float("nan"), dtype=torch.float32))
+    _ok(emu, emu.fca_prefix_pass(ctypes.byref(plan), ctypes.byref(t), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), None))
+    _ok(emu, emu.fca_suffix_pass(ctypes.byref(plan), ctypes.byref(t), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), None))
+    # both launches left second partials, each in its own set of rows
+    S_rows = S * md.layout.max_partials * hq
+    back = pl.view(-1, 2)[S_rows:, 0]
+    half = back.shape[0] // 2
+    assert bool((~torch.isnan(back[:half])).any()) and bool((~torch.isnan(back[half:])).any())
+    _ok(emu, emu.fca_merge(ctypes.byref(plan), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), o1.data_ptr(), o1.stride(0), o1.stride(1), _lib.FCA_BF16, l1.data_ptr(), None))
+    ref_out, ref_lse = oracle_for(w)
+    assert_matches_oracle(o1, l1, ref_out, ref_lse, what="prefix + suffix + merge")
+    assert_matches_oracle(out, lse, ref_out, ref_lse, what="fused step")
+    # where the waves of a pair meet is the one thing the launches may differ in
+    torch.testing.assert_close(l1, lse, rtol=0, atol=2e-3)
+    # reproducible: no item is shared, nothing is written behind the ordinary rows, and the step equals itself
+    t.reproducible = 1
+    res = []
+    for _ in range(2):
+        po.fill_(float("nan")), pl.fill_(float("nan"))
+        o2 = guarded(torch.full((S, hq, d), float("nan")).bfloat16())
+        l2 = guarded(torch.full((S, hq), float("nan"), dtype=torch.float32))
+        _ok(emu, emu.fca_decode_step(ctypes.byref(plan), ctypes.byref(t), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), o2.data_ptr(), o2.stride(0), o2.stride(1), _lib.FCA_BF16, l2.data_ptr(), None))
+        assert bool(torch.isnan(pl.view(-1, 2)[S_rows:]).all())
+        res.append((o2, l2))
+    assert torch.equal(res[0][0].view(torch.int16), res[1][0].view(torch.int16)) and torch.equal(res[0][1], res[1][1])
+    assert_matches_oracle(res[0][0], res[0][1], ref_out, ref_lse, what="reproducible step")
+
+
+@pytest.mark.parametrize("rows,d", [(32, 128), (64, 128), (32, 64), (32, 256)])
+def test_merge_stays_inside_buffers_of_random_bits(emu, rows, d):
+    """fca_merge on partial buffers nothing has written: whatever bits they hold, every load stays
+    inside them (the buffers end against inaccessible pages), and a row whose scale points
+    outside the rows set aside for second partials comes out as NaN."""
+    hq, hkv = 8, 2
+    gen = torch.Generator().manual_seed(rows + d)
+    seg_len, paths = two_level_forest(gen, 3, 4, (2000, 2600), (10, 300))
+    w = make_forest_workload("two-level", seg_len, paths, gen, num_q_heads=hq, num_kv_heads=hkv, head_dim=d, device="cpu")
+    S, mb = w.block_table.shape
+    plan = make_plan(S, mb, hq, hkv, d, chunk_tokens=128, rows_per_item=rows, max_levels=4)
+    layout = _lib.FcaMetaLayout()
+    _ok(emu, emu.fca_meta_describe(ctypes.byref(plan), ctypes.byref(layout)))
+    assert layout.max_partials >= 16  # the merge with several lane groups per row
+    nm, no, nl = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    _ok(emu, emu.fca_workspace_bytes(ctypes.byref(plan), ctypes.byref(nm), ctypes.byref(no), ctypes.byref(nl)))
+    meta = guarded(torch.zeros(nm.value // 4, dtype=torch.int32))
+    bt, sl = guarded(w.block_table), guarded(w.seq_lens)
+    _ok(emu, emu.fca_build_metadata(ctypes.byref(plan), bt.data_ptr(), bt.stride(0), sl.data_ptr(), meta.data_ptr(), None))
+    npart = meta[layout.seq_npart : layout.seq_npart + S]
+    assert int(npart.min()) >= 16
+    out = guarded(torch.zeros(S, hq, d).bfloat16())
+    lse = guarded(torch.zeros(S, hq, dtype=torch.float32))
+    merge = lambda po, pl: _ok(emu, emu.fca_merge(ctypes.byref(plan), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), out.data_ptr(), out.stride(0), out.stride(1), _lib.FCA_BF16, lse.data_ptr(), None))
+    # 1. random bits everywhere
+    po = guarded(torch.randint(-(2**15), 2**15, (no.value // 2,), generator=gen, dtype=torch.int16))
+    pl = guarded(torch.randint(-(2**31), 2**31, (nl.value // 4,), generator=gen, dtype=torch.int64).to(torch.int32))
+    merge(po, pl)
+    # 2. plausible values: finite log-sum-exps, and scales whose mantissa bits point anywhere in their 23 bits
+    plf = pl.view(torch.float32).view(-1, 2)
+    plf[:, 0] = torch.randn(plf.shape[0], generator=gen)
+    scale_bits = torch.randint(0, 2**23, (plf.shape[0],), generator=gen, dtype=torch.int32) | 0x3F800000
+    plf[:, 1] = scale_bits.view(torch.float32)
+    po.view(torch.float16).copy_(torch.randn(po.shape[0], generator=gen).half())
+    merge(po, pl)
+    stray = (scale_bits & 0x7FFFFF) - 32
+    back_rows = plf.shape[0] - S * layout.max_partials * hq
+    assert back_rows == 2 * 32 * min(1024, (layout.max_items * hkv + 3) // 2)
+    bad = ((stray < 0) & (scale_bits & 0x7FFFFF != 0)) | (stray >= back_rows)
+    for s in range(S):
+        for h in range(hq):
+            first = (s * layout.max_partials) * hq + h
+            rows_of = [first + i * hq for i in range(int(npart[s]))]
+            assert bool(torch.isnan(lse[s, h])) == bool(bad[rows_of].any()), (s, h)
+    # 3. a buffer of zeros (what the Python side allocates): empty rows, no NaN
+    po.zero_(), pl.zero_()
+    merge(po, pl)
+    assert not bool(torch.isnan(out.float()).any())
 
 
 # ---- query runs: rows over table rows, declared groups, causal nodes ------------------------------
@@ -232,7 +334,7 @@ def _decode_rows(lib, table, row_table, row_lens, row_group, q, cache, k_scale, 
     t = _lib.FcaTensors(
         qg.data_ptr(), qg.stride(0), qg.stride(1), kv.data_ptr(), kv.data_ptr() + kv.stride(0) * esz, kv.stride(1), kv.stride(2),
         _lib.FCA_FP8_E4M3 if kv.dtype == torch.float8_e4m3fn else _lib.FCA_BF16, 1, bt.data_ptr(), bt.stride(0),
-        None if ks is None else ks.data_ptr(), None if vs is None else vs.data_ptr(), float(d**-0.5),
+        None if ks is None else ks.data_ptr(), None if vs is None else vs.data_ptr(), float(d**-0.5), 0, EMU_WORKGROUPS,
     )
     out = guarded(torch.full((R, hq, d), float("nan")).bfloat16())
     lse = guarded(torch.full((R, hq), float("nan"), dtype=torch.float32))

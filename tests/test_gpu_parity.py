@@ -10,13 +10,14 @@ from tests.helpers import assert_matches_oracle, oracle_for
 pytestmark = pytest.mark.gpu
 
 
-def _run(w, **kw):
+def _run(w, max_workgroups=0, reproducible=False, **kw):
     from arctic_platform_amd.forest import build_forest_metadata
     from arctic_platform_amd.ops import forest_cascade_decode
 
     md = build_forest_metadata(
         w.block_table, w.seq_lens, num_q_heads=w.num_q_heads, num_kv_heads=w.num_kv_heads, head_dim=w.head_dim, **kw
     )
+    md.max_workgroups, md.reproducible = max_workgroups, reproducible
     out, lse = forest_cascade_decode(w.q, w.kv_cache, md, w.scale, w.k_scale, w.v_scale)
     torch.cuda.synchronize()
     md.check()
@@ -268,7 +269,7 @@ def test_error_budget_of_fp32_outputs(gpu):
 
 
 @pytest.mark.parametrize("index,workgroups,chunk", [(2, 8, 512), (2, 8, 1024), (5, 8, 512), (4, 16, 256)])
-def test_items_shared_by_pairs_of_waves(gpu, index, workgroups, chunk, monkeypatch):
+def test_items_shared_by_pairs_of_waves(gpu, index, workgroups, chunk):
     """With many items per wave the 32-row kernel sets the largest items aside, one per pair of
     waves, and both waves of a pair attend it from either end until their claims meet.  A
     small grid brings that schedule to a small batch.  Items long enough (four pairs of tiles)
@@ -276,9 +277,8 @@ def test_items_shared_by_pairs_of_waves(gpu, index, workgroups, chunk, monkeypat
     the claim counters are zero again after every launch, and a second launch agrees."""
     from arctic_platform_amd.ops import forest_cascade_decode
 
-    monkeypatch.setenv("FCA_ATTEND_WORKGROUPS", str(workgroups))
     w = make_config(index, device=gpu, shrink=4, poison_unused=True)
-    md, out, lse = _run(w, chunk_tokens=chunk)
+    md, out, lse = _run(w, max_workgroups=workgroups, chunk_tokens=chunk)
     items = md.items()
     waves = 4 * workgroups
     tickets = len(items) * w.num_kv_heads

@@ -26,13 +26,13 @@ def test_exports_every_declared_symbol(lib):
     assert declared == set(_lib.EXPORTS)
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.fca_version() == 103
+    assert lib.fca_version() == 104
 
 
 def test_struct_sizes_match_header():
     assert ctypes.sizeof(_lib.FcaPlan) == 9 * 4
     assert ctypes.sizeof(_lib.FcaMetaLayout) == 18 * 8
-    assert ctypes.sizeof(_lib.FcaTensors) == 104
+    assert ctypes.sizeof(_lib.FcaTensors) == 112
 
 
 def test_workspace_sizes(lib):
@@ -44,14 +44,14 @@ def test_workspace_sizes(lib):
     nm, no, nl = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
     assert lib.fca_workspace_bytes(ctypes.byref(plan), ctypes.byref(nm), ctypes.byref(no), ctypes.byref(nl)) == 0
     assert nm.value == layout.total_int32 * 4
-    # one row per (partial slot, query head), then 32 rows for each of up to 1024 pairs of waves
-    # that attend an item together
-    rows = 512 * layout.max_partials * 32 + 32 * 1024
+    # one row per (partial slot, query head), then two sets of 32 rows for each of up to 1024
+    # pairs of waves that attend an item together
+    rows = 512 * layout.max_partials * 32 + 2 * 32 * 1024
     assert no.value == rows * 128 * 2  # half-precision rows
     assert nl.value == rows * 2 * 4  # {lse, scale}
     tiny = make_plan(2, 4, 8, 2, 64, chunk_tokens=32, max_levels=1)  # at most 2 * 5 * 2 tickets: 11 pairs of waves
     assert lib.fca_workspace_bytes(ctypes.byref(tiny), None, ctypes.byref(no), ctypes.byref(nl)) == 0
-    assert no.value == (2 * 5 * 8 + 32 * 11) * 64 * 2 and nl.value == (2 * 5 * 8 + 32 * 11) * 8
+    assert no.value == (2 * 5 * 8 + 2 * 32 * 11) * 64 * 2 and nl.value == (2 * 5 * 8 + 2 * 32 * 11) * 8
 
 
 @pytest.mark.parametrize(
@@ -162,7 +162,7 @@ def test_header_is_plain_c_and_links(tmp_path):
     exe = tmp_path / "probe"
     subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", f"-I{inc}", str(src), f"-L{libdir}", "-lzorro_fca", f"-Wl,-rpath,{libdir}", "-o", str(exe)], check=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
-    assert int(out[0]) >= 1 and int(out[2]) == (512 * (320 * 16 // 1024 + 6) * 32 + 32 * 1024) * 128 * 2
+    assert int(out[0]) >= 1 and int(out[2]) == (512 * (320 * 16 // 1024 + 6) * 32 + 2 * 32 * 1024) * 128 * 2
     # lim of every key: a prompt token is seen up to the end of its group, a response token up to its own end
     assert [int(x) for x in out[4:16]] == [6, 6, 6, 5, 5, 6, 12, 12, 12, 12, 12, 12]
 
