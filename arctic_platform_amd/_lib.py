@@ -51,6 +51,7 @@ class FcaSplitPlan(ctypes.Structure):
         ("num_q_heads", ctypes.c_int32),
         ("num_kv_heads", ctypes.c_int32),
         ("head_dim", ctypes.c_int32),
+        ("window", ctypes.c_int32),
     ]
 
 
@@ -175,7 +176,7 @@ def declare_signatures(lib: ctypes.CDLL) -> ctypes.CDLL:
     lib.fca_time_next_attention.argtypes = [VP, VP]
     F32 = ctypes.c_float
     lib.fca_split_layout_ints.argtypes = [I32, P(I64)]
-    lib.fca_split_layout_build.argtypes = [I32, VP, VP, VP, I32, I32, VP]
+    lib.fca_split_layout_build.argtypes = [I32, VP, VP, VP, I32, I32, I32, VP]
     lib.fca_split_workspace_bytes.argtypes = [P(FcaSplitPlan), SZ, SZ]
     lib.fca_split_attention_forward.argtypes = [P(FcaSplitPlan), VP, I64, VP, I64, VP, I64, VP, F32, VP, VP, I64, VP, VP]
     lib.fca_split_attention_backward.argtypes = (

@@ -102,15 +102,12 @@ fca::AttendParams attend_params(const fca_plan* p, const fca_tensors* t, void* m
   a.max_partials = (int32_t)L.max_partials;
   a.select = select;
   a.kv_reread = t->kv_reread;
-  // items attended by two waves together: not when the caller wants the same bits from every launch
-  a.coop_ctr = t->reproducible ? nullptr : a.meta + L.coop_ctr;
+  // Items attended by two waves together: not when the caller wants the same bits from every
+  // launch, and not in a launch over the private items alone, whose second partials would land
+  // in the rows the launch over the shared items has just written for the same merge.
+  a.coop_ctr = t->reproducible || select == 2 ? nullptr : a.meta + L.coop_ctr;
   a.coop_pairs = (int32_t)fca::coop_pairs_for(*p, L);
-  // a launch over the private items alone takes the second set of back rows (and tags that
-  // say so), so that the two passes in front of one merge do not write the same rows
-  const int region = select == 2 ? 1 : 0;
-  a.coop_tag0 = region * 32 * a.coop_pairs;
-  a.coop_row0 = (int64_t)p->num_seqs * L.max_partials * p->num_q_heads + a.coop_tag0;
-  a.max_workgroups = t->max_workgroups;
+  a.coop_row0 = (int64_t)p->num_seqs * L.max_partials * p->num_q_heads;
   return a;
 }
 
@@ -121,7 +118,7 @@ int run_attend(const fca_plan* p, const fca_tensors* t, void* meta, void* po, fl
   if ((reinterpret_cast<uintptr_t>(po) & 15) || (reinterpret_cast<uintptr_t>(pl) & 15))
     return fail(FCA_ERR_INVALID_ARG, "partial workspaces must be 16-byte aligned");
   const fca::AttendParams a = attend_params(p, t, meta, po, pl, select);
-  hipError_t e = fca::launch_attend(a, *p, t->kv_dtype, static_cast<hipStream_t>(stream));
+  hipError_t e = fca::launch_attend(a, *p, t->kv_dtype, t->max_workgroups, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? FCA_OK : hip_fail(e, "attention pass launch");
 }
 
@@ -148,7 +145,7 @@ int run_merge(const fca_plan* p, const void* meta, const void* po, const float* 
   m.head_dim = p->head_dim;
   m.max_partials = (int32_t)L.max_partials;
   m.coop_row0 = (int64_t)p->num_seqs * L.max_partials * p->num_q_heads;
-  m.coop_rows = 32 * fca::kCoopRegions * fca::coop_pairs_for(*p, L);
+  m.coop_rows = 32 * fca::coop_pairs_for(*p, L);
   m.out_dtype = out_dtype;
   // whole 16-byte stores when every 8-channel group of out is 16-byte aligned
   const int64_t esz = out_dtype == FCA_F32 ? 4 : 2;
@@ -168,9 +165,8 @@ const char* fca_last_error(void) { return g_error; }
 int fca_workspace_bytes(const fca_plan* plan, size_t* meta_bytes, size_t* partial_out_bytes, size_t* partial_lse_bytes) {
   if (int rc = check_plan(plan)) return rc;
   const fca::MetaLayout L = fca::make_layout(*plan);
-  // one row per (partial slot, query head), then two sets of 32 rows per pair of waves that may share an item
-  const size_t rows = (size_t)plan->num_seqs * (size_t)L.max_partials * plan->num_q_heads +
-                      32 * (size_t)fca::kCoopRegions * (size_t)fca::coop_pairs_for(*plan, L);
+  // one row per (partial slot, query head), then 32 rows per pair of waves that may share an item
+  const size_t rows = (size_t)plan->num_seqs * (size_t)L.max_partials * plan->num_q_heads + 32 * (size_t)fca::coop_pairs_for(*plan, L);
   if (meta_bytes) *meta_bytes = (size_t)L.total * sizeof(int32_t);
   if (partial_out_bytes) *partial_out_bytes = rows * plan->head_dim * 2;  // half
   if (partial_lse_bytes) *partial_lse_bytes = rows * 2 * sizeof(float);    // {lse, scale}
@@ -446,6 +442,7 @@ int check_split(const fca_split_plan* p) {
                 "head_dim 256 takes a multiple of 4 query heads per KV head (got %d): only the kernels that share "
                 "their operands through LDS have an instance of that size",
                 p->num_q_heads / p->num_kv_heads);
+  if (p->window < 0) return fail(FCA_ERR_INVALID_ARG, "window must be >= 0 (0 = none), got %d", p->window);
   return FCA_OK;
 }
 int check_rows(const char* name, const void* ptr, int64_t stride, int heads, int head_dim) {
@@ -476,8 +473,10 @@ int fca_split_layout_ints(int32_t num_tokens, int64_t* num_ints) {
 }
 
 int fca_split_layout_build(int32_t num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,
-                           const int32_t* response_tokens, int32_t num_tokens, int32_t responses_only, int32_t* layout_host) {
+                           const int32_t* response_tokens, int32_t num_tokens, int32_t responses_only, int32_t window,
+                           int32_t* layout_host) {
   if (num_groups < 0 || num_tokens < 0) return fail(FCA_ERR_INVALID_ARG, "num_groups and num_tokens must be >= 0");
+  if (window < 0) return fail(FCA_ERR_INVALID_ARG, "window must be >= 0 (0 = none), got %d", window);
   if (num_groups > 0 && (!prompt_tokens || !group_sizes)) return fail(FCA_ERR_INVALID_ARG, "prompt_tokens and group_sizes must be non-NULL");
   int64_t total = 0, samples = 0;
   for (int g = 0; g < num_groups; ++g) {
@@ -495,7 +494,7 @@ int fca_split_layout_build(int32_t num_groups, const int32_t* prompt_tokens, con
   if (num_tokens == 0) return FCA_OK;
   if (!layout_host) return fail(FCA_ERR_INVALID_ARG, "layout_host is NULL");
   fca::build_split_layout(num_groups, prompt_tokens, group_sizes, response_tokens, (num_tokens + 31) / 32, responses_only != 0,
-                          layout_host);
+                          window, layout_host);
   return FCA_OK;
 }
 
@@ -534,6 +533,7 @@ int fca_split_attention_forward(const fca_split_plan* plan, const void* q_dev, i
   p.num_q_heads = plan->num_q_heads;
   p.num_kv_heads = plan->num_kv_heads;
   p.scale = scale;
+  p.window = plan->window;
   hipError_t e = fca::launch_split_forward(p, plan->head_dim, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? FCA_OK : hip_fail(e, "split attention forward launch");
 }
@@ -585,6 +585,7 @@ int fca_split_attention_backward(const fca_split_plan* plan, const void* q_dev, 
   p.num_q_heads = hq;
   p.num_kv_heads = hkv;
   p.scale = scale;
+  p.window = plan->window;
   hipError_t e = fca::launch_split_backward(p, d, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? FCA_OK : hip_fail(e, "split attention backward launch");
 }

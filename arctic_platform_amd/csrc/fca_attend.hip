@@ -450,7 +450,7 @@ static int cached_cu_count() {
   return cus;
 }
 
-hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, hipStream_t stream) {
+hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, int max_workgroups, hipStream_t stream) {
   const bool fp8 = kv_dtype == FCA_FP8_E4M3;
   const int nrt = plan.rows_per_item / 32;
   // Four independent waves per workgroup.  At head size 128 a wave uses the whole register
@@ -463,7 +463,7 @@ hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dty
   int grid = cached_cu_count() * workgroups_per_cu(plan.head_dim, fp8, plan.rows_per_item);
   // the caller's cap: leaves CUs to other streams (and brings the many-items-per-wave
   // schedules of a large batch to a small one)
-  if (p.max_workgroups > 0 && p.max_workgroups < grid) grid = p.max_workgroups;
+  if (max_workgroups > 0 && max_workgroups < grid) grid = max_workgroups;
   if ((int64_t)grid * kWaves > max_tickets) grid = (int)((max_tickets + kWaves - 1) / kWaves);
   if (grid < 1) grid = 1;
   if (nrt == 1 && plan.head_dim != 256) return launch_attend32(p, plan, kv_dtype, grid, stream);

@@ -491,7 +491,7 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
       const int64_t back_row = p.coop_row0 + (int64_t)pair_id * 32 + m;
       const int64_t prow = row_member < mcnt ? (from_back ? back_row : front_row) : -1;
       // the front partial says where the back partial of the same query row is
-      const int tag = shared_item && !coop_back ? p.coop_tag0 + (((pair_id + 1) << 5) | m) : 0;
+      const int tag = shared_item && !coop_back ? ((pair_id + 1) << 5) | m : 0;
       const int inc = shared_item ? (coop_back ? 1 << 10 : 1) : 0;
       int* ctr = p.coop_ctr + pair_id;
       int added = 0, claim_v = 0;

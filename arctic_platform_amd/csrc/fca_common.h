@@ -18,11 +18,9 @@ constexpr int kHeaderInts = 16;
 // Items that two waves of the 32-row attention kernel attend together (one from either end):
 // at most this many pairs of waves, one claim counter each in the metadata workspace, and 32
 // partial rows each behind the ordinary partial rows for the wave that comes from the back.
-// There are kCoopRegions such sets of rows: a launch over the private items only writes the
-// second one, so that it leaves the rows of a launch over the shared items alone when both
-// precede one merge.
+// A launch over the private items alone (fca_suffix_pass) shares no item: it would write the
+// same 32 rows per pair as the launch over the shared items that precedes the same merge.
 constexpr int kCoopMaxPairs = 1024;
-constexpr int kCoopRegions = 2;
 constexpr int kCoopMinPairs = 4;  // pairs of 32-token tiles an item needs to be shared
 
 enum HeaderSlot {
@@ -185,9 +183,7 @@ struct AttendParams {
   // buffers have rows for, and the first of those rows
   int32_t* coop_ctr;
   int32_t coop_pairs;
-  int32_t max_workgroups;  // > 0: cap of the grid
-  int32_t coop_tag0;  // added to the tags of this launch: 32 * coop_pairs * (set of back rows it writes)
-  int64_t coop_row0;  // first back row of this launch
+  int64_t coop_row0;
 };
 
 struct MergeParams {
@@ -237,6 +233,9 @@ struct SplitParams {
   // small batches: dk and dv are formed per query head (fp32 slices [Hq / Hkv][T][Hkv][D]) and summed afterwards
   int32_t head_split;
   float *dk_part, *dv_part;
+  // > 0: a row sees only the keys fewer than `window` positions before it in its own sequence
+  // (prompt followed by the sample's response); the kernels then have instances of their own
+  int32_t window;
 };
 // A batch with few key tiles leaves most of the chip idle behind its longest walks (a prompt's
 // key tiles are seen by the whole group): then every query head of a KV head gets a workgroup
@@ -246,7 +245,7 @@ inline bool split_by_head(int64_t tiles, int num_q_heads, int num_kv_heads) {
 }
 // Offsets into the int32 layout array of a batch of `tiles` 32-token tiles.
 struct SplitLayout {
-  int64_t kv_lim, q_tiles, kv_qend, q_order, kv_limmin, kv_order, q_index, total;
+  int64_t kv_lim, q_tiles, kv_qend, q_order, kv_limmin, kv_order, q_index, pos, total;
 };
 __host__ __device__ inline SplitLayout make_split_layout(int64_t tiles) {
   SplitLayout L;
@@ -257,11 +256,12 @@ __host__ __device__ inline SplitLayout make_split_layout(int64_t tiles) {
   L.kv_limmin = L.q_order + tiles;
   L.kv_order = L.kv_limmin + tiles;  // ceil(tiles / 4) entries used
   L.q_index = L.kv_order + tiles;  // row of q and out that belongs to a packed token, -1 = none
-  L.total = L.q_index + 32 * tiles;
+  L.pos = L.q_index + 32 * tiles;  // position of a packed token in its sample's sequence (prompt, then response)
+  L.total = L.pos + 32 * tiles;
   return L;
 }
 void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,
-                        const int32_t* response_tokens, int64_t tiles, bool responses_only, int32_t* out);
+                        const int32_t* response_tokens, int64_t tiles, bool responses_only, int32_t window, int32_t* out);
 hipError_t launch_split_forward(const SplitParams& p, int head_dim, hipStream_t stream);
 hipError_t launch_split_backward(const SplitParams& p, int head_dim, hipStream_t stream);
 
@@ -270,7 +270,8 @@ hipError_t launch_rows(const int32_t* query_start_loc, const int32_t* seq_lens, 
                        int32_t* row_table, int32_t* row_lens, int32_t* row_group, hipStream_t stream);
 hipError_t launch_append(const AppendParams& p, int kv_dtype, hipStream_t stream);
 hipError_t launch_gather(const AppendParams& p, int kv_dtype, hipStream_t stream);  // key / value are written
-hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, hipStream_t stream);
+// max_workgroups > 0 caps the grid
+hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, int max_workgroups, hipStream_t stream);
 // Events the next attention launch of this thread records its begin and end in (NULL: none).
 void set_attend_timing(hipEvent_t start, hipEvent_t stop);
 void take_attend_timing(hipEvent_t* start, hipEvent_t* stop);

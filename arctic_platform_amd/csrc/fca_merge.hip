@@ -66,7 +66,7 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
     const unsigned tag = sbits & 0x007fffffu;
     take(ls.x, __uint_as_float(sbits & 0xff800000u), o);
     if (tag) {
-      // tag = 32 * (pair + 1) + row of the tile, counted over the sets of back rows.  Only a
+      // tag = 32 * (pair + 1) + row of the tile.  Only a
       // buffer no attention launch has written (or one written for another plan) holds a tag
       // that points anywhere else: it is not followed, and the output row leaves as NaN.
       const int64_t rel = (int64_t)tag - 32;

@@ -31,6 +31,7 @@
 // The first product feeds its rows in the order that makes its output registers the B
 // operand of the second, so probabilities never leave registers.
 #include <algorithm>
+#include <cstdint>
 #include <numeric>
 #include <type_traits>
 #include <vector>
@@ -40,12 +41,18 @@
 namespace fca {
 
 // ---- host: the layout array ------------------------------------------------------------
+// With a window (> 0) row r sees key t only if pos(r) - pos(t) < window as well, pos = place of
+// a token in its sample's own sequence (the prompt's tokens, then the response's): the walks
+// of the query tiles start at the first tile any of their rows still sees, and a key tile's
+// walk ends at the last query tile that still sees any of its keys.
 void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,
-                        const int32_t* response_tokens, int64_t tiles, bool responses_only, int32_t* out) {
+                        const int32_t* response_tokens, int64_t tiles, bool responses_only, int32_t window, int32_t* out) {
   const SplitLayout L = make_split_layout(tiles);
   const int64_t padded = 32 * tiles;
   std::vector<int32_t> own(padded, 0), pstart(padded, 0), pend(padded, 0), group_of(padded, 0);
+  std::vector<int64_t> seen_end(padded, 0);  // one past the last row that sees key x
   int32_t* lim = out + L.kv_lim;
+  int32_t* pos = out + L.pos;
   int64_t t = 0;
   int64_t ri = 0;
   int group = 0;
@@ -60,6 +67,8 @@ void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int3
       own[x] = (int32_t)from;
       pstart[x] = (int32_t)p0;
       pend[x] = (int32_t)p1;
+      pos[x] = (int32_t)(in_prompt ? x - p0 : (p1 - p0) + (x - from));
+      seen_end[x] = window > 0 ? std::min<int64_t>(to, x + window) : limit;
     }
   };
   for (int g = 0; g < num_groups; ++g) {
@@ -71,31 +80,61 @@ void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int3
     fill(p0, p1, gend, p0, p1);
     in_prompt = false;
     t = p1;
+    int64_t last_start = -1, last_len = 0;  // the group's last response that has tokens
     for (int s = 0; s < group_sizes[g]; ++s) {
       const int64_t s1 = t + response_tokens[ri + s];
       fill(t, s1, s1, p0, p1);
+      if (s1 > t) last_start = t, last_len = s1 - t;
       t = s1;
+    }
+    if (window > 0 && last_start >= 0) {
+      // a prompt key at position pt is seen by the first pt + window - (prompt length) rows of every response
+      for (int64_t x = p0; x < p1; ++x) {
+        const int64_t rows = (x - p0) + window - (p1 - p0);
+        if (rows > 0) seen_end[x] = std::max(seen_end[x], last_start + std::min(last_len, rows));
+      }
     }
     ri += group_sizes[g];
   }
-  for (int64_t x = t; x < padded; ++x) lim[x] = 0, q_index[x] = -1;
+  for (int64_t x = t; x < padded; ++x) lim[x] = 0, q_index[x] = -1, pos[x] = 0;
+  const int64_t num_tokens = t;
   std::vector<int64_t> qcost(tiles);
   for (int64_t i = 0; i < tiles; ++i) {
     // The needs of a tile's first row cover those of the rows behind it: they belong to
     // later segments, whose own tokens and (if the group changes inside the tile) prompt
     // lie between the first row and themselves.
     const int64_t r0 = 32 * i;
-    const int32_t b0 = own[r0] / 32;
-    const int32_t a0 = pstart[r0] / 32;
+    int32_t b0 = own[r0] / 32;
+    int32_t a0 = pstart[r0] / 32;
     int32_t a1 = pend[r0] > pstart[r0] ? (pend[r0] + 31) / 32 : a0;
     a1 = std::max(a0, std::min(a1, b0));
+    if (window > 0) {
+      // the keys each row still sees, a range in its own segment and one in its prompt; the
+      // part of a range inside the tiles [a0, a1) bounds that walk from the left, the rest
+      // (a prompt's last tile may be the first of the other walk) the other one
+      int64_t need_a = INT64_MAX, need_b = INT64_MAX;
+      auto need = [&](int64_t lo, int64_t hi) {  // keys lo .. hi - 1
+        if (lo / 32 >= a0 && lo / 32 < a1) need_a = std::min(need_a, lo);
+        else need_b = std::min(need_b, lo);
+        if (lo / 32 < a1 && (hi - 1) / 32 >= a1) need_b = std::min<int64_t>(need_b, 32 * (int64_t)a1);
+      };
+      for (int64_t r = r0; r < std::min<int64_t>(r0 + 32, num_tokens); ++r) {
+        need(std::max<int64_t>(own[r], r - window + 1), r + 1);
+        if (own[r] >= pend[r] && pend[r] > pstart[r]) {  // a response row behind a prompt
+          const int64_t first = pstart[r] + std::max<int64_t>(0, (int64_t)pos[r] - window + 1);
+          if (first < pend[r]) need(first, pend[r]);
+        }
+      }
+      a0 = need_a == INT64_MAX ? a1 : std::max<int32_t>(a0, (int32_t)(need_a / 32));
+      if (need_b != INT64_MAX) b0 = std::max<int32_t>(b0, (int32_t)(need_b / 32));
+    }
     int32_t* rec = out + L.q_tiles + 4 * i;
     rec[0] = a0, rec[1] = a1, rec[2] = b0, rec[3] = 0;
     for (int x = 0; x < 32; ++x) rec[3] |= q_index[r0 + x] >= 0;  // any row of the tile that has a query
     qcost[i] = (a1 - a0) + (i - b0 + 1);
-    int32_t mx = 0;
-    for (int x = 0; x < 32; ++x) mx = std::max(mx, lim[r0 + x]);
-    out[L.kv_qend + i] = (mx + 31) / 32;
+    int64_t mx = 0;
+    for (int x = 0; x < 32; ++x) mx = std::max(mx, seen_end[r0 + x]);
+    out[L.kv_qend + i] = (int32_t)((mx + 31) / 32);
     int32_t mn = lim[r0];
     for (int x = 1; x < 32; ++x) mn = std::min(mn, lim[r0 + x]);
     out[L.kv_limmin + i] = mn;
@@ -116,7 +155,6 @@ void build_split_layout(int num_groups, const int32_t* prompt_tokens, const int3
   int32_t* ko = out + L.kv_order;
   std::iota(ko, ko + tiles, 0);
   std::stable_sort(ko, ko + quads, [&](int32_t a, int32_t b) { return kcost[a] > kcost[b]; });
-
 }
 
 namespace {
@@ -212,7 +250,9 @@ __global__ __launch_bounds__(kThreads) void split_images_kernel(const __bf16* x,
 // the L1 sees a quarter of the operand traffic.  Without it (query heads per KV head not a
 // multiple of four) every wave fetches its own tiles into two register buffers.  Head size
 // 256 runs one workgroup per CU (its accumulators and query rows alone take 192 registers).
-template <int D, bool BWD, bool SHARED>
+// WIN: the instances for a sliding window (p.window > 0).  Every pair of tiles is tested element
+// by element there, with the positions of row and key in their own sequence beside the limits.
+template <int D, bool BWD, bool SHARED, bool WIN>
 __global__ __launch_bounds__(kThreads, SHARED && D < 256 ? 2 : 1) void split_query_kernel(SplitParams p) {
   constexpr int KS = D / 16, NDB = D / 32, SLOTS = (BWD ? 3 : 2) * KS, PER = SLOTS / kWaves;
   __shared__ i32x4 lds[SHARED ? 2 : 1][SHARED ? SLOTS : 1][64];
@@ -239,6 +279,9 @@ __global__ __launch_bounds__(kThreads, SHARED && D < 256 ? 2 : 1) void split_que
   const int r = 32 * i + n;
   const int qi = p.layout[L.q_index + r];  // this lane's row of q and out, -1 = none
   const int64_t rc = max(qi, 0);
+  // the first position this lane's row still sees: keys at positions pos_lo .. its own
+  int pos_lo = 0;
+  if constexpr (WIN) pos_lo = p.layout[L.pos + r] - p.window + 1;
 
   bf16x8 qreg[KS], doreg[BWD ? KS : 1];
 #pragma unroll
@@ -281,22 +324,43 @@ __global__ __launch_bounds__(kThreads, SHARED && D < 256 ? 2 : 1) void split_que
     bool ok[16];
 #pragma unroll
     for (int x = 0; x < 16; ++x) ok[x] = true;
-    const bool masked = !(j < i && limmin >= 32 * i + 32);
-    if (masked) {
+    const bool masked = WIN || !(j < i && limmin >= 32 * i + 32);
+    if constexpr (WIN) {
+      // (four keys at a time, applied at once: sixteen tests kept side by side cost registers)
       const int tok0 = 32 * j + 8 * h;
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
           const i32x4 lim = *reinterpret_cast<const i32x4*>(p.layout + L.kv_lim + tok0 + 16 * blk + 4 * half);
+          const i32x4 kpos = *reinterpret_cast<const i32x4*>(p.layout + L.pos + tok0 + 16 * blk + 4 * half);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) ok[8 * blk + 4 * half + e] = tok0 + 16 * blk + 4 * half + e <= r && lim[e] > r;
+          for (int e = 0; e < 4; ++e) {
+            const int x = 8 * blk + 4 * half + e;
+            const bool sees = tok0 + 16 * blk + 4 * half + e <= r && lim[e] > r && kpos[e] >= pos_lo;
+            sr[x] = sees ? sr[x] : -INFINITY;
+          }
+          // (keeps the loads of the next four keys behind these tests: hoisted together, the
+          // eight loads of a tile push the dq instance of head size 128 into scratch)
+          __builtin_amdgcn_sched_barrier(0);
         }
-    }
-    // a hidden score becomes -inf, whose exponential is 0 (no branch around the exponentials)
-    if (masked) {
+    } else {
+      if (masked) {
+        const int tok0 = 32 * j + 8 * h;
 #pragma unroll
-      for (int x = 0; x < 16; ++x) sr[x] = ok[x] ? sr[x] : -INFINITY;
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            const i32x4 lim = *reinterpret_cast<const i32x4*>(p.layout + L.kv_lim + tok0 + 16 * blk + 4 * half);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ok[8 * blk + 4 * half + e] = tok0 + 16 * blk + 4 * half + e <= r && lim[e] > r;
+          }
+      }
+      // a hidden score becomes -inf, whose exponential is 0 (no branch around the exponentials)
+      if (masked) {
+#pragma unroll
+        for (int x = 0; x < 16; ++x) sr[x] = ok[x] ? sr[x] : -INFINITY;
+      }
     }
     bf16x8 pb[2];
     if constexpr (!BWD) {
@@ -442,11 +506,14 @@ __device__ inline void load_to_lds4(const void* src, unsigned lds_slot) {
 // s_waitcnt that constrains only the vector-memory counter (gfx9 encoding)
 #define FCA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0f70 | ((n) & 15) | (((n) >> 4) << 14))
 
-template <int D, bool DK>
+// WIN: the instances for a sliding window; the positions of a step's 32 rows ride through the
+// ring beside their log-sum-exp (requested by wave 1), and every step is tested element by element.
+template <int D, bool DK, bool WIN>
 __global__ __launch_bounds__(kThreads, D < 256 ? 2 : 1) void split_key_kernel(SplitParams p) {
   constexpr int KS = D / 16, NDB = D / 32, SLOTS = (DK ? 3 : 2) * KS, PER = SLOTS / kWaves;
   __shared__ i32x4 lds[kRing][SLOTS][64];
   __shared__ __attribute__((aligned(16))) float lds_stat[kRing][64];  // lse (in log2 units) of the step's 32 rows, then their delta
+  __shared__ __attribute__((aligned(16))) int lds_pos[WIN ? kRing : 1][64];  // positions of the step's 32 rows (twice)
   const SplitLayout L = make_split_layout(p.num_tiles);
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, h = lane >> 5;
@@ -469,6 +536,9 @@ __global__ __launch_bounds__(kThreads, D < 256 ? 2 : 1) void split_key_kernel(Sp
   const int t = 32 * j + n;
   const int64_t tc = min(t, T - 1);
   const int lim_t = p.layout[L.kv_lim + t];
+  // the last position that still sees this lane's key
+  int pos_hi = 0;
+  if constexpr (WIN) pos_hi = p.layout[L.pos + t] + p.window - 1;
   const float sc = p.scale * kLog2e;
 
   bf16x8 kreg[KS], vreg[DK ? KS : 1];
@@ -502,12 +572,17 @@ __global__ __launch_bounds__(kThreads, D < 256 ? 2 : 1) void split_key_kernel(Sp
   const float* stat_src = (DK && h == 1 ? p.delta : p.lse2) + n;
   const unsigned slot_lds = lds_address(&lds[0][0][0]) + wave * PER * 1024;
   const unsigned stat_lds = lds_address(&lds_stat[0][0]);
+  const int32_t* pos_src = p.layout + L.pos + n;
+  const unsigned pos_lds = lds_address(&lds_pos[0][0]);
   auto request = [&]() {
     const int hq = hq0 + req_g;
     const int64_t at = ((int64_t)hq * nt + req_i) * KS * 512;
 #pragma unroll
     for (int x = 0; x < PER; ++x) load_to_lds16(slot_src[x] + at, slot_lds + (req_buf * SLOTS + x) * 1024);
     if (wave == 0) load_to_lds4(stat_src + hq * padded + 32 * req_i, stat_lds + req_buf * 256);
+    if constexpr (WIN) {
+      if (wave == 1) load_to_lds4(pos_src + 32 * req_i, pos_lds + req_buf * 256);
+    }
     req_buf = req_buf + 1 == kRing ? 0 : req_buf + 1;
     // past the last step the last one is requested again
     if (req_g + 1 < group)
@@ -525,7 +600,7 @@ __global__ __launch_bounds__(kThreads, D < 256 ? 2 : 1) void split_key_kernel(Sp
     for (int step = 0; step < steps; ++step) {
       // this wave's requests of `step` have landed; after the barrier so have everyone's, and
       // everyone has finished with the stage of the step before, which the next request refills
-      if (wave == 0)
+      if (wave == 0 || (WIN && wave == 1))
         FCA_WAIT_VMCNT((kRing - 2) * (PER + 1));
       else
         FCA_WAIT_VMCNT((kRing - 2) * PER);
@@ -543,11 +618,13 @@ __global__ __launch_bounds__(kThreads, D < 256 ? 2 : 1) void split_key_kernel(Sp
         bf16x8 pb[2];
         const int row0 = 32 * i + 8 * h;
         // a hidden score becomes -inf, whose exponential is 0 (no branch around the exponentials)
-        if (!(i > j && limmin >= 32 * i + 32)) {
+        if (WIN || !(i > j && limmin >= 32 * i + 32)) {
 #pragma unroll
           for (int x = 0; x < 16; ++x) {
             const int qrow = row0 + 16 * (x >> 3) + (x & 7);
-            sr[x] = (t <= qrow && qrow < lim_t) ? sr[x] : -INFINITY;
+            bool sees = t <= qrow && qrow < lim_t;
+            if constexpr (WIN) sees = sees && lds_pos[buf][8 * h + 16 * (x >> 3) + (x & 7)] <= pos_hi;
+            sr[x] = sees ? sr[x] : -INFINITY;
           }
         }
 #pragma unroll
@@ -647,12 +724,20 @@ hipError_t launch_split_forward(const SplitParams& p, int head_dim, hipStream_t 
     const unsigned grid = (unsigned)p.num_tiles * ((p.num_q_heads + kWaves - 1) / kWaves);
     // (head size 256 has the LDS-shared kernels only: two register buffers of 32 operand slots
     // each do not fit a wave; such plans are refused when they are checked)
-    if ((p.num_q_heads / p.num_kv_heads) % kWaves == 0) {
-      split_query_kernel<D, false, true><<<grid, kThreads, 0, stream>>>(p);
-    } else if constexpr (D < 256) {
-      split_query_kernel<D, false, false><<<grid, kThreads, 0, stream>>>(p);
+    const bool shared = (p.num_q_heads / p.num_kv_heads) % kWaves == 0;
+    if (!shared && D == 256) return hipErrorInvalidValue;
+    if (p.window > 0) {
+      if (shared) {
+        split_query_kernel<D, false, true, true><<<grid, kThreads, 0, stream>>>(p);
+      } else if constexpr (D < 256) {
+        split_query_kernel<D, false, false, true><<<grid, kThreads, 0, stream>>>(p);
+      }
     } else {
-      return hipErrorInvalidValue;
+      if (shared) {
+        split_query_kernel<D, false, true, false><<<grid, kThreads, 0, stream>>>(p);
+      } else if constexpr (D < 256) {
+        split_query_kernel<D, false, false, false><<<grid, kThreads, 0, stream>>>(p);
+      }
     }
     return hipGetLastError();
   });
@@ -671,19 +756,31 @@ hipError_t launch_split_backward(const SplitParams& p, int head_dim, hipStream_t
   return by_head_dim(head_dim, [&](auto d) {
     constexpr int D = decltype(d)::value;
     const unsigned qgrid = (unsigned)nt * ((p.num_q_heads + kWaves - 1) / kWaves);
-    if ((p.num_q_heads / p.num_kv_heads) % kWaves == 0) {
-      split_query_kernel<D, true, true><<<qgrid, kThreads, 0, stream>>>(p);
-    } else if constexpr (D < 256) {
-      split_query_kernel<D, true, false><<<qgrid, kThreads, 0, stream>>>(p);
-    } else {
-      return hipErrorInvalidValue;
-    }
-    if (hipError_t e = hipGetLastError()) return e;
+    const bool shared = (p.num_q_heads / p.num_kv_heads) % kWaves == 0;
+    if (!shared && D == 256) return hipErrorInvalidValue;
     const int ratio = p.num_q_heads / p.num_kv_heads;
     const unsigned kgrid = (unsigned)((nt + kWaves - 1) / kWaves) * p.num_kv_heads * (p.head_split ? ratio : 1);
-    split_key_kernel<D, false><<<kgrid, kThreads, 0, stream>>>(p);
-    if (hipError_t e = hipGetLastError()) return e;
-    split_key_kernel<D, true><<<kgrid, kThreads, 0, stream>>>(p);
+    if (p.window > 0) {
+      if (shared) {
+        split_query_kernel<D, true, true, true><<<qgrid, kThreads, 0, stream>>>(p);
+      } else if constexpr (D < 256) {
+        split_query_kernel<D, true, false, true><<<qgrid, kThreads, 0, stream>>>(p);
+      }
+      if (hipError_t e = hipGetLastError()) return e;
+      split_key_kernel<D, false, true><<<kgrid, kThreads, 0, stream>>>(p);
+      if (hipError_t e = hipGetLastError()) return e;
+      split_key_kernel<D, true, true><<<kgrid, kThreads, 0, stream>>>(p);
+    } else {
+      if (shared) {
+        split_query_kernel<D, true, true, false><<<qgrid, kThreads, 0, stream>>>(p);
+      } else if constexpr (D < 256) {
+        split_query_kernel<D, true, false, false><<<qgrid, kThreads, 0, stream>>>(p);
+      }
+      if (hipError_t e = hipGetLastError()) return e;
+      split_key_kernel<D, false, false><<<kgrid, kThreads, 0, stream>>>(p);
+      if (hipError_t e = hipGetLastError()) return e;
+      split_key_kernel<D, true, false><<<kgrid, kThreads, 0, stream>>>(p);
+    }
     if (hipError_t e = hipGetLastError()) return e;
     if (p.head_split) {
       const int row = p.num_kv_heads * D;

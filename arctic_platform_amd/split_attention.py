@@ -31,14 +31,20 @@ def _stream_ptr(device) -> int:
 class SplitLayout:
     """Token layout of one deduplicated batch: ``[(prompt_tokens, [response_tokens, ...]), ...]``."""
 
-    def __init__(self, groups, device="cuda", responses_only=False, scratch_pool=None):
+    def __init__(self, groups, device="cuda", responses_only=False, scratch_pool=None, sliding_window=None):
         """``scratch_pool``: a dict shared by layouts whose calls run one after the other on one
         stream (the adapter makes a layout per step), so that they share their scratch buffers.
         ``responses_only`` (forward only): ``k`` and ``v`` hold every token, ``q`` and ``out`` only
         the response rows, in packed order, and the prompts' own attention is not computed (a
-        prefill chunk behind a cached context, with the context as the prompt)."""
+        prefill chunk behind a cached context, with the context as the prompt).
+        ``sliding_window`` (the argument of the trainer's attention calls,
+        qwen_attention_patcher.py:1206, :1226; None = no window): a row sees only the keys fewer
+        than that many positions before it in its own sample's sequence, itself included."""
         self.groups = [(int(p), [int(n) for n in rs]) for p, rs in groups]
         self.responses_only = bool(responses_only)
+        if sliding_window is not None and int(sliding_window) < 1:
+            raise ValueError(f"sliding_window must be a positive number of tokens or None, got {sliding_window}")
+        self.window = 0 if sliding_window is None else int(sliding_window)
         prompt = np.asarray([p for p, _ in self.groups], dtype=np.int32)
         sizes = np.asarray([len(rs) for _, rs in self.groups], dtype=np.int32)
         resp = np.asarray([n for _, rs in self.groups for n in rs], dtype=np.int32)
@@ -52,7 +58,7 @@ class SplitLayout:
         _lib.check(
             lib.fca_split_layout_build(
                 len(self.groups), prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, self.num_tokens,
-                1 if self.responses_only else 0, self.host.ctypes.data,
+                1 if self.responses_only else 0, self.window, self.host.ctypes.data,
             )
         )
         self.device = torch.device(device)
@@ -60,11 +66,11 @@ class SplitLayout:
         self._scratch = {} if scratch_pool is None else scratch_pool
 
     @classmethod
-    def from_group_token_layout(cls, layout, device="cuda"):
-        return cls([(g["prompt_tokens"], g["response_tokens"]) for g in layout], device=device)
+    def from_group_token_layout(cls, layout, device="cuda", sliding_window=None):
+        return cls([(g["prompt_tokens"], g["response_tokens"]) for g in layout], device=device, sliding_window=sliding_window)
 
     @classmethod
-    def from_reconstruction_info(cls, reconstruction_info, device="cuda"):
+    def from_reconstruction_info(cls, reconstruction_info, device="cuda", sliding_window=None):
         """From the trainer's ``reconstruction_info`` itself: ``prompt_groups`` (lists of sample
         indices) and ``segment_info`` (dicts with ``group_idx``, ``type`` "prompt" / "response",
         ``original_idx`` and ``num_valid_tokens``, or ``start`` / ``end`` before unpadding), read the
@@ -79,7 +85,7 @@ class SplitLayout:
         for g, members in enumerate(reconstruction_info["prompt_groups"]):
             prompt = valid(segs[(g, "prompt", members[0])])
             groups.append((prompt, [valid(segs[(g, "response", m)]) for m in members]))
-        return cls(groups, device=device)
+        return cls(groups, device=device, sliding_window=sliding_window)
 
     # views of the layout array (tests, inspection)
     def kv_lim(self):
@@ -109,6 +115,10 @@ class SplitLayout:
         o = 40 * self.num_tiles
         return self.host[o : o + 32 * self.num_tiles]
 
+    def pos(self):
+        o = 72 * self.num_tiles
+        return self.host[o : o + 32 * self.num_tiles]
+
     def scratch(self, plan, backward: bool) -> torch.Tensor:
         """Scratch of a call, kept with the layout: layers run one after the other on a stream."""
         fwd, bwd = ctypes.c_size_t(), ctypes.c_size_t()
@@ -135,8 +145,8 @@ def _check_heads(q, k, v):
         raise ValueError(f"k and v must have one shape and the head size of q, got q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
 
 
-def _plan(q, k):
-    return _lib.FcaSplitPlan(q.shape[0], q.shape[1], k.shape[1], q.shape[2])
+def _plan(q, k, layout):
+    return _lib.FcaSplitPlan(layout.num_tokens, q.shape[1], k.shape[1], q.shape[2], layout.window)
 
 
 def split_attention_forward(q, k, v, layout: SplitLayout, scale: float, out=None):
@@ -148,7 +158,7 @@ def split_attention_forward(q, k, v, layout: SplitLayout, scale: float, out=None
     for name, x in (("k", k), ("v", v)):
         _check_rows(name, x, t)
     _check_heads(q, k, v)
-    plan = _lib.FcaSplitPlan(t, q.shape[1], k.shape[1], q.shape[2])
+    plan = _plan(q, k, layout)
     if out is None:
         out = torch.empty((rows, q.shape[1], q.shape[2]), dtype=torch.bfloat16, device=q.device)
     else:
@@ -179,7 +189,7 @@ def split_attention_backward(dout, q, k, v, out, lse, layout: SplitLayout, scale
     _check_heads(q, k, v)
     if out.shape != q.shape or dout.shape != q.shape:
         raise ValueError("out and dout must have the shape of q")
-    plan = _plan(q, k)
+    plan = _plan(q, k, layout)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     for name, x in (("dq", dq), ("dk", dk), ("dv", dv)):
         _check_rows(name, x, t)
@@ -213,22 +223,27 @@ class _SplitAttention(torch.autograd.Function):
         return dq, dk, dv, None, None
 
 
-def _refuse_unsupported(dropout, sliding_window):
+def _check_call_arguments(dropout, sliding_window, layout):
     """The trainer hands both to its attention calls on every step
-    (qwen_attention_patcher.py:1204-1206, :1224-1226); Qwen3 has no dropout in attention and
-    no window, and these kernels implement neither, so anything else is refused rather than
-    silently ignored."""
+    (qwen_attention_patcher.py:1204-1206, :1224-1226).  The window is a property of the layout
+    (its walks are cut to it), so the call's value must be the one the layout was made for.
+    Attention dropout is 0 outside training and in every recipe of the reference; the kernels
+    have none, and another value is refused rather than silently ignored."""
     if dropout is not None and float(dropout) != 0.0:
         raise NotImplementedError(f"attention dropout {dropout} is not supported by the split attention kernels (only 0.0)")
-    if sliding_window is not None:
-        raise NotImplementedError(f"sliding_window={sliding_window} is not supported by the split attention kernels (only None)")
+    want = 0 if sliding_window is None else int(sliding_window)
+    if want != layout.window:
+        raise ValueError(
+            f"sliding_window={sliding_window} but the layout was made for "
+            f"{layout.window or None}: pass sliding_window to SplitLayout as well"
+        )
 
 
 def split_attention(q, k, v, layout: SplitLayout, scale: float, dropout: float = 0.0, sliding_window=None):
     """Differentiable split attention: ``out [T, Hq, D]`` in deduplicated order.  ``dropout``
-    and ``sliding_window`` are the arguments of the trainer's attention calls; only 0.0 and
-    None are accepted."""
-    _refuse_unsupported(dropout, sliding_window)
+    and ``sliding_window`` are the arguments of the trainer's attention calls: dropout must be
+    0.0, the window the one ``layout`` was made for."""
+    _check_call_arguments(dropout, sliding_window, layout)
     return _SplitAttention.apply(q, k, v, layout, scale)
 
 
@@ -239,9 +254,9 @@ def split_attention_padded(q, k, v, valid, layout: SplitLayout, scale: float, dr
     ``[T_padded]`` (the deduplicated attention mask, zorro_train.py:359-372), ``layout`` counts
     the valid tokens.  The valid rows are gathered, attended, and scattered back; padding rows
     of the result are zero and receive no gradient.  Differentiable."""
-    _refuse_unsupported(dropout, sliding_window)
+    _check_call_arguments(dropout, sliding_window, layout)
     index = torch.nonzero(valid, as_tuple=False).squeeze(-1)
     if index.numel() != layout.num_tokens:
         raise ValueError(f"{index.numel()} valid tokens, the layout counts {layout.num_tokens}")
-    out = split_attention(q.index_select(0, index), k.index_select(0, index), v.index_select(0, index), layout, scale)
+    out = split_attention(q.index_select(0, index), k.index_select(0, index), v.index_select(0, index), layout, scale, dropout, sliding_window)
     return torch.zeros_like(q).index_copy(0, index, out)

@@ -136,12 +136,11 @@ const char* fca_last_error(void);
 /* Workspace sizes for a plan: metadata (int32 arrays) and the two partial buffers.  A
  * partial output row is D half-precision values times one power-of-two scale per row:
  * partial_out is half [rows, D], partial_lse is fp32 [rows, 2] = {natural-log lse, scale},
- * rows = S * max_partials * Hq plus 2 x 32 for each pair of waves that may attend an item
+ * rows = S * max_partials * Hq plus 32 for each pair of waves that may attend an item
  * together (at most 1024 pairs; the second wave of a pair writes there, and the scale of
- * the first wave's row carries the place in its mantissa bits; fca_suffix_pass writes the
- * second set of 32, every other pass the first, so a prefix and a suffix pass in front of one
- * merge do not meet).  Both are opaque to the caller: written by the passes, read by the
- * merge. */
+ * the first wave's row carries the place in its mantissa bits; fca_suffix_pass shares no
+ * item, so that it leaves alone what fca_prefix_pass wrote there for the same merge).  Both
+ * are opaque to the caller: written by the passes, read by the merge. */
 int fca_workspace_bytes(const fca_plan* plan, size_t* meta_bytes, size_t* partial_out_bytes, size_t* partial_lse_bytes);
 int fca_meta_describe(const fca_plan* plan, fca_meta_layout* layout);
 
@@ -288,12 +287,20 @@ int fca_gather_kv(void* key_dev, void* value_dev, int64_t token_stride, int64_t 
  * them (arctic_platform/rl/zorro_train/qwen_attention_patcher.py:1186-1231): prompt rows
  * attend causally to their prompt, response rows to their group's whole prompt and causally
  * to their own response.  Row strides are in elements; the heads of a token are contiguous
- * ([H, D]); every pointer 16-byte aligned, strides multiples of 8. */
+ * ([H, D]); every pointer 16-byte aligned, strides multiples of 8.
+ * window > 0 is the sliding_window both reference calls receive (:1206, :1226): a row also
+ * sees only the keys fewer than `window` positions before it, its own included, positions
+ * counted in the sample's own sequence (the prompt's tokens, then the response's), i.e.
+ * key position > row position - window.  The layout must have been built for a window at
+ * least as wide (or for none): its walks leave out the tiles no row sees any more.
+ * Attention dropout, the other argument of those calls, has no counterpart here (it is 0
+ * outside training and in every recipe of the reference). */
 typedef struct fca_split_plan {
   int32_t num_tokens; /* T: tokens of the deduplicated batch */
   int32_t num_q_heads;
   int32_t num_kv_heads;
   int32_t head_dim; /* 64, 128 or 256 (256: num_q_heads / num_kv_heads a multiple of 4) */
+  int32_t window;   /* 0 = none */
 } fca_split_plan;
 
 /* int32 entries of the layout array of a batch of num_tokens tokens. */
@@ -306,9 +313,11 @@ int fca_split_layout_ints(int32_t num_tokens, int64_t* num_ints);
  * responses_only != 0 (forward only, no counterpart in the reference): k and v still hold
  * all num_tokens rows, but q and out hold the response rows only, in packed order, and the
  * prompts' own attention is not computed -- a prefill chunk behind a cached context, with
- * the context as the prompt. */
+ * the context as the prompt.
+ * window > 0: the walks of the layout skip what a sliding window of that width hides from
+ * every row of a tile; such a layout serves plans with 0 < plan->window <= window only. */
 int fca_split_layout_build(int32_t num_groups, const int32_t* prompt_tokens, const int32_t* group_sizes,
-                           const int32_t* response_tokens, int32_t num_tokens, int32_t responses_only,
+                           const int32_t* response_tokens, int32_t num_tokens, int32_t responses_only, int32_t window,
                            int32_t* layout_host);
 /* Bytes of device scratch a forward / a backward call needs: operand tiles in MFMA order,
  * per-row sums, and for small batches fp32 slices of dk and dv per query head of a KV head. */

@@ -19,9 +19,18 @@ against.  ``full_attention_of_samples`` is the computation the split replaces, e
 sample's whole sequence attended causally on its own, which is what the reference's own
 test compares the patched model with (tests/zorro_train/test_once_patcher.py:189-206).
 
+Both calls also receive ``sliding_window`` (:1206, :1226), which the attention interface
+turns into "key index > query index - sliding_window" on top of the causal mask, indices
+counted in the call's own key sequence (transformers ``sliding_window_overlay``,
+masking_utils.py:92-101; the flash path's ``window_size = (sliding_window - 1, ...)``,
+modeling_flash_attention_utils.py:650-655).  ``window`` below is that argument.
+
 Pins (tests/test_split_attention.py): split == full on the rows both produce, for outputs
 and for gradients (prompt rows of a group receive the sum over its samples), a closed form
-(constant V), and the row sums of the probabilities implied by the log-sum-exp.
+(constant V), and the row sums of the probabilities implied by the log-sum-exp; with a
+window: the same against ``scaled_dot_product_attention`` under an explicit boolean mask
+built with plain loops, a window of 1 (every row returns its own V row), and a window at
+least as long as the longest sample (equal to no window).
 """
 
 from __future__ import annotations
@@ -47,10 +56,10 @@ def total_tokens(layout) -> int:
     return sum(int(p) + sum(int(n) for n in rs) for p, rs in layout)
 
 
-def _attend(q, k, v, scale, first_key_offset):
+def _attend(q, k, v, scale, first_key_offset, window=None):
     """q [Lq, Hq, D], k/v [Lk, Hkv, D]; query i sees keys 0 .. first_key_offset + i
-    (bottom-right aligned causal mask when first_key_offset = Lk - Lq).  Returns out and
-    the natural-log log-sum-exp [Lq, Hq]."""
+    (bottom-right aligned causal mask when first_key_offset = Lk - Lq), with ``window`` only
+    the last ``window`` of them.  Returns out and the natural-log log-sum-exp [Lq, Hq]."""
     lq, hq, _ = q.shape
     lk, hkv, _ = k.shape
     rep = hq // hkv
@@ -60,12 +69,14 @@ def _attend(q, k, v, scale, first_key_offset):
     keys = torch.arange(lk)[None, :]
     rows = torch.arange(lq)[:, None]
     s = s.masked_fill(keys > rows + first_key_offset, -math.inf)
+    if window is not None:
+        s = s.masked_fill(keys <= rows + first_key_offset - int(window), -math.inf)
     lse = torch.logsumexp(s, dim=-1)
     p = torch.exp(s - lse[..., None])
     return torch.einsum("hqk,khd->qhd", p, vv), lse.transpose(0, 1)
 
 
-def split_attention(q, k, v, layout, scale, dtype=torch.float64):
+def split_attention(q, k, v, layout, scale, dtype=torch.float64, window=None):
     """q [T, Hq, D], k/v [T, Hkv, D] in deduplicated order.  Returns (out [T, Hq, D],
     lse [T, Hq]) in ``dtype``.  Differentiable."""
     q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
@@ -74,12 +85,12 @@ def split_attention(q, k, v, layout, scale, dtype=torch.float64):
     for g, kind, start, n in segments(layout):
         if kind == "p":
             prompt_of[g] = (start, n)
-            o, l = _attend(q[start : start + n], k[start : start + n], v[start : start + n], scale, 0)
+            o, l = _attend(q[start : start + n], k[start : start + n], v[start : start + n], scale, 0, window)
         else:
             ps, pn = prompt_of[g]
             kk = torch.cat([k[ps : ps + pn], k[start : start + n]])
             vv = torch.cat([v[ps : ps + pn], v[start : start + n]])
-            o, l = _attend(q[start : start + n], kk, vv, scale, pn)
+            o, l = _attend(q[start : start + n], kk, vv, scale, pn, window)
         outs.append(o)
         lses.append(l)
     return torch.cat(outs), torch.cat(lses)
@@ -98,18 +109,19 @@ def reconstruct(x, layout):
     return samples
 
 
-def full_attention_of_samples(q, k, v, layout, scale, dtype=torch.float64):
+def full_attention_of_samples(q, k, v, layout, scale, dtype=torch.float64, window=None):
     """Every sample's whole sequence attended causally on its own, from the deduplicated
     tensors; returns per sample (out, lse) of prompt + response rows."""
     q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
     return [
-        _attend(qs, ks, vs, scale, 0)
+        _attend(qs, ks, vs, scale, 0, window)
         for qs, ks, vs in zip(reconstruct(q, layout), reconstruct(k, layout), reconstruct(v, layout))
     ]
 
 
-def visible(layout):
-    """Brute force: boolean [T, T], entry (r, t) true when query row r attends to key t."""
+def visible(layout, window=None):
+    """Brute force: boolean [T, T], entry (r, t) true when query row r attends to key t.
+    With ``window``, positions count along the sample's own sequence (prompt, then response)."""
     n = total_tokens(layout)
     vis = torch.zeros(n, n, dtype=torch.bool)
     prompt_of = {}
@@ -118,8 +130,14 @@ def visible(layout):
             prompt_of[g] = (start, length)
         for i in range(length):
             r = start + i
-            vis[r, start : r + 1] = True
+            row_pos = i if kind == "p" else prompt_of[g][1] + i
+            for j in range(i + 1):  # the row's own segment
+                key_pos = j if kind == "p" else prompt_of[g][1] + j
+                if window is None or row_pos - key_pos < window:
+                    vis[r, start + j] = True
             if kind == "r":
                 ps, pn = prompt_of[g]
-                vis[r, ps : ps + pn] = True
+                for j in range(pn):
+                    if window is None or row_pos - j < window:
+                        vis[r, ps + j] = True
     return vis

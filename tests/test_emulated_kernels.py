@@ -198,9 +198,10 @@ def test_entry_points_agree(emu):
 
 
 def test_separate_passes_with_shared_items_equal_the_fused_step(emu):
-    """Shared and private items as launches of their own, on a batch where both launches end on
-    items that pairs of waves attend together: each launch has rows of its own for the second
-    partials, so the suffix launch leaves the prefix launch's alone and the merge finds both."""
+    """Shared and private items as launches of their own, on a batch where either launch has
+    enough long items for pairs of waves to attend some together: the launch over the private
+    items shares none, so the second partials that the launch over the shared items left are
+    still there when the merge follows them."""
     hq, hkv, d, chunk = 16, 4, 128, 512
     gen = torch.Generator().manual_seed(311)
     seg_len, paths = two_level_forest(gen, 12, 5, (700, 2500), (230, 900))
@@ -224,12 +225,11 @@ def test_separate_passes_with_shared_items_equal_the_fused_step(emu):
     o1 = guarded(torch.full((S, hq, d), float("nan")).bfloat16())
     l1 = guarded(torch.full((S, hq), float("nan"), dtype=torch.float32))
     _ok(emu, emu.fca_prefix_pass(ctypes.byref(plan), ctypes.byref(t), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), None))
-    _ok(emu, emu.fca_suffix_pass(ctypes.byref(plan), ctypes.byref(t), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), None))
-    # both launches left second partials, each in its own set of rows
     S_rows = S * md.layout.max_partials * hq
-    back = pl.view(-1, 2)[S_rows:, 0]
-    half = back.shape[0] // 2
-    assert bool((~torch.isnan(back[:half])).any()) and bool((~torch.isnan(back[half:])).any())
+    back = pl.view(-1, 2)[S_rows:].clone()
+    assert bool((~torch.isnan(back[:, 0])).any()), "the launch over the shared items left no second partial"
+    _ok(emu, emu.fca_suffix_pass(ctypes.byref(plan), ctypes.byref(t), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), None))
+    assert torch.equal(pl.view(-1, 2)[S_rows:].view(torch.int32), back.view(torch.int32)), "the suffix launch wrote second partials"
     _ok(emu, emu.fca_merge(ctypes.byref(plan), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), o1.data_ptr(), o1.stride(0), o1.stride(1), _lib.FCA_BF16, l1.data_ptr(), None))
     ref_out, ref_lse = oracle_for(w)
     assert_matches_oracle(o1, l1, ref_out, ref_lse, what="prefix + suffix + merge")
@@ -287,7 +287,7 @@ def test_merge_stays_inside_buffers_of_random_bits(emu, rows, d):
     merge(po, pl)
     stray = (scale_bits & 0x7FFFFF) - 32
     back_rows = plf.shape[0] - S * layout.max_partials * hq
-    assert back_rows == 2 * 32 * min(1024, (layout.max_items * hkv + 3) // 2)
+    assert back_rows == 32 * min(1024, (layout.max_items * hkv + 3) // 2)
     bad = ((stray < 0) & (scale_bits & 0x7FFFFF != 0)) | (stray >= back_rows)
     for s in range(S):
         for h in range(hq):
@@ -551,6 +551,23 @@ def test_split_attention_forward_and_backward(emu, heads, late):
     """``late``: a direct-to-LDS load lands only when a wait covers it, the latest the hardware allows
     (a missing or miscounted wait then shows as stale operands); otherwise at once, the earliest (a
     buffer refilled while it is still being read then shows)."""
+    _split_cases(emu, heads, late, None)
+
+
+@pytest.mark.parametrize("late", [False, True], ids=["loads-land-at-once", "loads-land-at-their-wait"])
+@pytest.mark.parametrize(
+    "heads,window",
+    [((8, 2, 128), 1), ((8, 2, 128), 45), ((8, 2, 128), 200), ((6, 2, 64), 7), ((6, 2, 64), 32), ((4, 1, 256), 45)],
+    ids=lambda x: "Hq%d-Hkv%d-D%d" % x if isinstance(x, tuple) else f"w{x}",
+)
+def test_split_attention_with_a_sliding_window(emu, heads, window, late):
+    """The instances for a sliding window: a row sees the last ``window`` positions of its own
+    sample's sequence (the prompt's tokens, then the response's), itself included.  Windows
+    shorter than a tile, of exactly a tile, across tiles, and longer than every sample."""
+    _split_cases(emu, heads, late, window)
+
+
+def _split_cases(emu, heads, late, window):
     from arctic_platform_amd.split_attention import SplitLayout
 
     hq, hkv, d = heads
@@ -562,9 +579,9 @@ def test_split_attention_forward_and_backward(emu, heads, late):
         k = guarded(torch.randn(t, hkv, d, generator=g).bfloat16())
         v = guarded(torch.randn(t, hkv, d, generator=g).bfloat16())
         scale = d**-0.5
-        lay = guarded(torch.from_numpy(SplitLayout(layout, device="cpu").host))
+        lay = guarded(torch.from_numpy(SplitLayout(layout, device="cpu", sliding_window=window).host))
         nt = (t + 31) // 32
-        plan = _lib.FcaSplitPlan(t, hq, hkv, d)
+        plan = _lib.FcaSplitPlan(t, hq, hkv, d, window or 0)
         fwd, bwd = ctypes.c_size_t(), ctypes.c_size_t()
         _ok(emu, emu.fca_split_workspace_bytes(ctypes.byref(plan), ctypes.byref(fwd), ctypes.byref(bwd)))
         ws_f, ws_b = guarded(torch.zeros(fwd.value, dtype=torch.uint8)), guarded(torch.zeros(bwd.value, dtype=torch.uint8))
@@ -578,7 +595,7 @@ def test_split_attention_forward_and_backward(emu, heads, late):
             ),
         )
         q64, k64, v64 = (x.double().requires_grad_() for x in (q, k, v))
-        ro, rl = oracle_split(q64, k64, v64, layout, scale)
+        ro, rl = oracle_split(q64, k64, v64, layout, scale, window=window)
         _close("out", out, ro, 2e-2 / max(1.0, float(ro.detach().abs().max())))
         torch.testing.assert_close(lse[:, :t].T.double(), rl.detach(), rtol=1e-3, atol=1e-3)
         dout = guarded(torch.randn(t, hq, d, generator=torch.Generator().manual_seed(ci + 1)).bfloat16())

@@ -44,14 +44,14 @@ def test_workspace_sizes(lib):
     nm, no, nl = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
     assert lib.fca_workspace_bytes(ctypes.byref(plan), ctypes.byref(nm), ctypes.byref(no), ctypes.byref(nl)) == 0
     assert nm.value == layout.total_int32 * 4
-    # one row per (partial slot, query head), then two sets of 32 rows for each of up to 1024
-    # pairs of waves that attend an item together
-    rows = 512 * layout.max_partials * 32 + 2 * 32 * 1024
+    # one row per (partial slot, query head), then 32 rows for each of up to 1024 pairs of waves
+    # that attend an item together
+    rows = 512 * layout.max_partials * 32 + 32 * 1024
     assert no.value == rows * 128 * 2  # half-precision rows
     assert nl.value == rows * 2 * 4  # {lse, scale}
     tiny = make_plan(2, 4, 8, 2, 64, chunk_tokens=32, max_levels=1)  # at most 2 * 5 * 2 tickets: 11 pairs of waves
     assert lib.fca_workspace_bytes(ctypes.byref(tiny), None, ctypes.byref(no), ctypes.byref(nl)) == 0
-    assert no.value == (2 * 5 * 8 + 2 * 32 * 11) * 64 * 2 and nl.value == (2 * 5 * 8 + 2 * 32 * 11) * 8
+    assert no.value == (2 * 5 * 8 + 32 * 11) * 64 * 2 and nl.value == (2 * 5 * 8 + 32 * 11) * 8
 
 
 @pytest.mark.parametrize(
@@ -150,7 +150,7 @@ def test_header_is_plain_c_and_links(tmp_path):
         "  int64_t n = 0;\n"
         "  int32_t layout[512];\n"
         "  if (fca_split_layout_ints(12, &n) != 0 || n > 512) return 2;\n"
-        "  if (fca_split_layout_build(2, prompts, sizes, responses, 12, 0, layout) != 0) { puts(fca_last_error()); return 3; }\n"
+        "  if (fca_split_layout_build(2, prompts, sizes, responses, 12, 0, 0, layout) != 0) { puts(fca_last_error()); return 3; }\n"
         '  for (int i = 0; i < 12; ++i) printf("%d ", layout[i]);\n'
         "  p.head_dim = 96;\n"
         "  return fca_workspace_bytes(&p, &m, &o, &l) == 0;  /* must be refused */\n"
@@ -162,7 +162,7 @@ def test_header_is_plain_c_and_links(tmp_path):
     exe = tmp_path / "probe"
     subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", f"-I{inc}", str(src), f"-L{libdir}", "-lzorro_fca", f"-Wl,-rpath,{libdir}", "-o", str(exe)], check=True)
     out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
-    assert int(out[0]) >= 1 and int(out[2]) == (512 * (320 * 16 // 1024 + 6) * 32 + 2 * 32 * 1024) * 128 * 2
+    assert int(out[0]) >= 1 and int(out[2]) == (512 * (320 * 16 // 1024 + 6) * 32 + 32 * 1024) * 128 * 2
     # lim of every key: a prompt token is seen up to the end of its group, a response token up to its own end
     assert [int(x) for x in out[4:16]] == [6, 6, 6, 5, 5, 6, 12, 12, 12, 12, 12, 12]
 

@@ -108,20 +108,66 @@ def test_oracle_against_the_brute_force_mask_and_closed_forms():
     torch.testing.assert_close(lz, vis.sum(1).double().log()[:, None].expand(-1, 4), rtol=1e-12, atol=1e-12)
 
 
+@pytest.mark.parametrize("window", [1, 5, 40, 1000])
+def test_oracle_with_a_sliding_window(window):
+    """The window of the two reference calls (qwen_attention_patcher.py:1206, :1226), pinned
+    three ways: against scaled_dot_product_attention under a boolean mask written with plain
+    loops over positions; split == every sample's whole sequence under the same window; and the
+    special cases that need no arithmetic."""
+    layout = LAYOUTS[1]
+    q, k, v = _inputs(layout, 4, 2, 8, 13)
+    out, lse = oracle_split(q, k, v, layout, 0.3, window=window)
+    vis = visible(layout, window)
+    kk, vv = k.repeat_interleave(2, 1), v.repeat_interleave(2, 1)
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.transpose(0, 1), kk.transpose(0, 1), vv.transpose(0, 1), attn_mask=vis[None], scale=0.3
+    ).transpose(0, 1)
+    torch.testing.assert_close(out, ref, rtol=1e-10, atol=1e-10)
+    s = (torch.einsum("qhd,khd->hqk", q, kk) * 0.3).masked_fill(~vis[None], -math.inf)
+    torch.testing.assert_close(lse, torch.logsumexp(s, -1).T, rtol=1e-12, atol=1e-12)
+    # every sample on its own, its whole sequence under the same window
+    full = full_attention_of_samples(q, k, v, layout, 0.3, window=window)
+    for (fo, fl), so, sl in zip(full, reconstruct(out, layout), reconstruct(lse, layout)):
+        torch.testing.assert_close(so, fo, rtol=1e-12, atol=1e-12)
+        torch.testing.assert_close(sl, fl, rtol=1e-12, atol=1e-12)
+    # the number of keys a row sees: min(window, its position + 1)
+    seen = []
+    for g, kind, start, n in segments(layout):
+        base = 0 if kind == "p" else layout[g][0]
+        seen += [min(window, base + i + 1) for i in range(n)]
+    assert vis.sum(1).tolist() == seen
+    if window == 1:  # a row sees itself only: its own V row, and lse = its own score
+        torch.testing.assert_close(out, vv, rtol=1e-12, atol=1e-12)
+        torch.testing.assert_close(lse, torch.einsum("qhd,qhd->qh", q, kk) * 0.3, rtol=1e-12, atol=1e-12)
+    if window == 1000:  # longer than every sample: no window at all
+        o2, l2 = oracle_split(q, k, v, layout, 0.3)
+        assert torch.equal(out, o2) and torch.equal(lse, l2)
+        assert torch.equal(vis, visible(layout))
+
+
 # ---- the layout array (host code of the library) -------------------------------------------------
-def test_layout_array_against_brute_force():
+@pytest.mark.parametrize("window", [None, 1, 9, 32, 50, 200])
+def test_layout_array_against_brute_force(window):
     rng = random.Random(7)
-    layouts = LAYOUTS + [_random_layout(rng) for _ in range(120)]
+    layouts = LAYOUTS + [_random_layout(rng) for _ in range(120 if window is None else 40)]
     for layout in layouts:
         if total_tokens(layout) == 0:
             continue
-        L = SplitLayout(layout, device="cpu")
+        L = SplitLayout(layout, device="cpu", sliding_window=window)
         t, nt = L.num_tokens, L.num_tiles
-        vis = visible(layout).numpy()
+        vis = visible(layout, window).numpy()
         lim = L.kv_lim()
         r, c = np.arange(t)[:, None], np.arange(t)[None, :]
-        assert (((c <= r) & (r < lim[:t][None, :])) == vis).all(), layout
-        assert (lim[t:] == 0).all()
+        pos = L.pos()
+        seen = (c <= r) & (r < lim[:t][None, :])
+        if window is not None:  # what the kernels test element by element
+            seen &= pos[:t][:, None] - pos[:t][None, :] < window
+        assert (seen == vis).all(), layout
+        assert (lim[t:] == 0).all() and (pos[t:] == 0).all()
+        want_pos = []
+        for g, kind, start, n in segments(layout):
+            want_pos += [(0 if kind == "p" else layout[g][0]) + i for i in range(n)]
+        assert pos[:t].tolist() == want_pos
         padded = np.zeros((32 * nt, 32 * nt), bool)
         padded[:t, :t] = vis
         tiles = padded.reshape(nt, 32, nt, 32).any(axis=(1, 3))  # [query tile, key tile]
@@ -131,7 +177,7 @@ def test_layout_array_against_brute_force():
             assert set(np.nonzero(tiles[i])[0].tolist()) <= covered, (layout, i)
         for j, qend in enumerate(L.kv_qend()):
             need = np.nonzero(tiles[:, j])[0]
-            assert need.min() >= j and need.max() < qend, (layout, j)
+            assert need.min() >= j and need.max() == qend - 1, (layout, j)
         assert sorted(L.q_order().tolist()) == list(range(nt))
         assert (L.kv_limmin() == lim.reshape(nt, 32).min(axis=1)).all()
         assert sorted(L.kv_order().tolist()) == list(range((nt + 3) // 4))
@@ -196,18 +242,43 @@ def test_layout_for_response_rows_only():
     assert (full.kv_lim() == L.kv_lim()).all()
 
 
-def test_dropout_and_sliding_window_are_refused():
-    """The trainer passes both on every call (qwen_attention_patcher.py:1204-1206): the values
-    Qwen3 uses go through, anything else raises before a tensor is looked at."""
+def test_dropout_is_refused_and_the_window_must_be_the_layouts():
+    """The trainer passes both on every call (qwen_attention_patcher.py:1204-1206).  Dropout
+    other than 0 raises before a tensor is looked at; so does a window that is not the one the
+    layout was made for (its walks are cut to it)."""
     from arctic_platform_amd.split_attention import split_attention, split_attention_padded
 
-    for fn, args in ((split_attention, (None, None, None, None, 1.0)), (split_attention_padded, (None, None, None, None, None, 1.0))):
+    plain = SplitLayout([(4, [3])], device="cpu")
+    windowed = SplitLayout([(4, [3])], device="cpu", sliding_window=128)
+    for fn, args in ((split_attention, (None, None, None)), (split_attention_padded, (None, None, None, None))):
         with pytest.raises(NotImplementedError, match="dropout"):
-            fn(*args, dropout=0.1)
-        with pytest.raises(NotImplementedError, match="sliding_window"):
-            fn(*args, sliding_window=4096)
-        with pytest.raises(NotImplementedError, match="sliding_window"):
-            fn(*args, dropout=0.0, sliding_window=128)
+            fn(*args, plain, 1.0, dropout=0.1)
+        with pytest.raises(ValueError, match="sliding_window"):
+            fn(*args, plain, 1.0, sliding_window=4096)
+        with pytest.raises(ValueError, match="sliding_window"):
+            fn(*args, windowed, 1.0, dropout=0.0, sliding_window=64)
+        with pytest.raises(ValueError, match="sliding_window"):
+            fn(*args, windowed, 1.0)
+    with pytest.raises(ValueError, match="positive"):
+        SplitLayout([(4, [3])], device="cpu", sliding_window=0)
+
+
+def test_layout_with_a_window_walks_only_what_the_window_leaves():
+    """One prompt of 1024 tokens, eight responses of 512, window 256: a query tile deep inside a
+    response walks eight key tiles of its own response and nothing of the prompt; the first tile
+    of a response walks the prompt's last eight tiles; a prompt key tile is walked by the query
+    tiles up to the start of the last response and no further."""
+    L = SplitLayout([(1024, [512] * 8)], device="cpu", sliding_window=256)
+    last = L.num_tiles - 1
+    a0, a1, b0, _ = L.q_tiles()[last]
+    assert a0 == a1 and b0 == last - 8
+    first_of_last = (1024 + 7 * 512) // 32
+    a0, a1, b0, _ = L.q_tiles()[first_of_last]
+    assert (a0, a1) == (32 - 8, 32) and b0 == first_of_last
+    # the prompt's last key tile: seen by the first 255 rows of every response, the last of which starts at tile first_of_last
+    assert L.kv_qend()[31] == first_of_last + 8
+    # the prompt's first key tile: positions 0..31 are seen by prompt rows up to position 286 only
+    assert L.kv_qend()[0] == (31 + 256 - 1) // 32 + 1
 
 
 def test_layout_arguments_are_checked():
@@ -216,11 +287,11 @@ def test_layout_arguments_are_checked():
     sizes = np.asarray([2], dtype=np.int32)
     resp = np.asarray([3, 2], dtype=np.int32)
     out = np.zeros(128, dtype=np.int32)
-    assert lib.fca_split_layout_build(1, prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, 9, 0, out.ctypes.data) == 0
-    assert lib.fca_split_layout_build(1, prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, 10, 0, out.ctypes.data) < 0
+    assert lib.fca_split_layout_build(1, prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, 9, 0, 0, out.ctypes.data) == 0
+    assert lib.fca_split_layout_build(1, prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, 10, 0, 0, out.ctypes.data) < 0
     assert b"holds 9 tokens" in lib.fca_last_error()
     resp[1] = -1
-    assert lib.fca_split_layout_build(1, prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, 6, 0, out.ctypes.data) < 0
+    assert lib.fca_split_layout_build(1, prompt.ctypes.data, sizes.ctypes.data, resp.ctypes.data, 6, 0, 0, out.ctypes.data) < 0
     plan = _lib.FcaSplitPlan(100, 6, 4, 128)
     assert lib.fca_split_workspace_bytes(ctypes.byref(plan), None, None) < 0
     plan = _lib.FcaSplitPlan(100, 8, 2, 128)
@@ -249,12 +320,12 @@ def _close(name, got, ref, scale_tol):
     assert bool((err <= bound).all()), f"{name}: max |err| {err.max():.4g}, largest reference {ref.abs().max():.4g}"
 
 
-def _run_case(layout, hq, hkv, d, seed, strided=False, q_gain=1.0):
+def _run_case(layout, hq, hkv, d, seed, strided=False, q_gain=1.0, window=None):
     q, k, v = _inputs(layout, hq, hkv, d, seed, torch.bfloat16)
     q = (q.float() * q_gain).bfloat16()
     t = q.shape[0]
     scale = d**-0.5
-    L = SplitLayout(layout)
+    L = SplitLayout(layout, sliding_window=window)
     if strided:
         # slices of one projection output [T, (Hq + 2 Hkv) * D], the way a fused QKV arrives
         fused = torch.cat([q.reshape(t, -1), k.reshape(t, -1), v.reshape(t, -1)], dim=1).cuda()
@@ -266,7 +337,7 @@ def _run_case(layout, hq, hkv, d, seed, strided=False, q_gain=1.0):
         qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
     out, lse = split_attention_forward(qd, kd, vd, L, scale)
     q64, k64, v64 = (x.double().requires_grad_() for x in (q, k, v))
-    ro, rl = oracle_split(q64, k64, v64, layout, scale)
+    ro, rl = oracle_split(q64, k64, v64, layout, scale, window=window)
     _close("out", out, ro, 2e-2 / max(1.0, float(ro.detach().abs().max())))
     torch.testing.assert_close(lse[:, :t].T.cpu().double(), rl.detach(), rtol=1e-3, atol=1e-3)
     dout = torch.randn(t, hq, d, generator=torch.Generator().manual_seed(seed + 1)).bfloat16()
@@ -282,6 +353,36 @@ def _run_case(layout, hq, hkv, d, seed, strided=False, q_gain=1.0):
 @pytest.mark.parametrize("heads", [(4, 2, 128), (8, 1, 64), (2, 2, 128)])
 def test_forward_and_backward_match_the_oracle(layout, heads):
     _run_case(layout, *heads, seed=21)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("window", [1, 20, 32, 100, 4096])
+@pytest.mark.parametrize("heads", [(8, 2, 128), (6, 2, 64), (4, 4, 128)])
+def test_sliding_window_matches_the_oracle(heads, window):
+    """The window of the trainer's attention calls (qwen_attention_patcher.py:1206, :1226):
+    shorter than a tile, a tile, across tiles, longer than every sample; the kernels that share
+    their operands through LDS and the per-wave ones."""
+    for layout in LAYOUTS:
+        _run_case(layout, *heads, seed=51, window=window)
+
+
+@pytest.mark.gpu
+def test_sliding_window_through_autograd_and_on_long_responses():
+    """Long responses over a long prompt with a window much shorter than either (most tiles of
+    the walks are left out), through the autograd function with the window passed on the call."""
+    layout = [(700, [400, 260]), (300, [500])]
+    hq, hkv, d, window = 8, 2, 128, 128
+    q, k, v = (x.cuda().requires_grad_() for x in _inputs(layout, hq, hkv, d, 61, torch.bfloat16))
+    L = SplitLayout(layout, sliding_window=window)
+    out = split_attention(q, k, v, L, d**-0.5, dropout=0.0, sliding_window=window)
+    w = torch.randn(out.shape, generator=torch.Generator().manual_seed(62)).bfloat16()
+    (out.float() * w.cuda().float()).sum().backward()
+    q64, k64, v64 = (x.detach().cpu().double().requires_grad_() for x in (q, k, v))
+    ro, _ = oracle_split(q64, k64, v64, layout, d**-0.5, window=window)
+    (ro * w.double()).sum().backward()
+    _close("out", out, ro, 2e-2 / max(1.0, float(ro.detach().abs().max())))
+    for name, got, ref in (("dq", q.grad, q64.grad), ("dk", k.grad, k64.grad), ("dv", v.grad, v64.grad)):
+        _close(name, got, ref, 1e-2)
 
 
 @pytest.mark.gpu
