@@ -22,6 +22,7 @@ EXPORTS = (
     "fca_version",
     "fca_last_error",
     "fca_workspace_bytes",
+    "fca_workspace_bytes_dtype",
     "fca_meta_describe",
     "fca_build_metadata",
     "fca_update_metadata",
@@ -158,6 +159,7 @@ def declare_signatures(lib: ctypes.CDLL) -> ctypes.CDLL:
     lib.fca_last_error.restype = ctypes.c_char_p
     lib.fca_last_error.argtypes = []
     lib.fca_workspace_bytes.argtypes = [P(FcaPlan), SZ, SZ, SZ]
+    lib.fca_workspace_bytes_dtype.argtypes = [P(FcaPlan), I32, SZ, SZ, SZ]
     lib.fca_meta_describe.argtypes = [P(FcaPlan), P(FcaMetaLayout)]
     lib.fca_build_metadata.argtypes = [P(FcaPlan), VP, I64, VP, VP, VP]
     lib.fca_update_metadata.argtypes = [P(FcaPlan), VP, I64, VP, VP, VP]

@@ -52,13 +52,24 @@ int check_plan(const fca_plan* p) {
   return FCA_OK;
 }
 
-int check_tensors(const fca_plan* p, const fca_tensors* t) {
+int kv_elem_bytes(int kv_dtype) { return kv_dtype == FCA_FP8_E4M3 ? 1 : kv_dtype == FCA_F32 ? 4 : 2; }
+
+// f32_ok: the entry point has an fp32 path (fca_decode_step and fca_decode_step_static)
+int check_tensors(const fca_plan* p, const fca_tensors* t, bool f32_ok = false) {
   if (!t) return fail(FCA_ERR_INVALID_ARG, "tensors is NULL");
   if (!t->q_dev || !t->k_cache_dev || !t->v_cache_dev || !t->block_table_dev)
     return fail(FCA_ERR_INVALID_ARG, "q, k_cache, v_cache and block_table must be non-NULL");
-  if (t->kv_dtype != FCA_BF16 && t->kv_dtype != FCA_FP8_E4M3)
-    return fail(FCA_ERR_UNSUPPORTED, "kv_dtype %d is not supported (bf16 or fp8 e4m3)", t->kv_dtype);
-  const int esz = t->kv_dtype == FCA_FP8_E4M3 ? 1 : 2;
+  if (t->kv_dtype == FCA_F32) {
+    if (!f32_ok)
+      return fail(FCA_ERR_UNSUPPORTED, "fp32 tensors (kv_dtype FCA_F32) run through fca_decode_step and fca_decode_step_static only");
+    if (p->head_dim != 64 && p->head_dim != 128)
+      return fail(FCA_ERR_UNSUPPORTED, "the fp32 path takes head_dim 64 or 128, got %d", p->head_dim);
+    if (p->rows_per_item != 32)
+      return fail(FCA_ERR_UNSUPPORTED, "the fp32 path takes rows_per_item 32, got %d", p->rows_per_item);
+  } else if (t->kv_dtype != FCA_BF16 && t->kv_dtype != FCA_FP8_E4M3) {
+    return fail(FCA_ERR_UNSUPPORTED, "kv_dtype %d is not supported (bf16, fp8 e4m3, or fp32 with an fp32 q)", t->kv_dtype);
+  }
+  const int esz = kv_elem_bytes(t->kv_dtype);
   if ((reinterpret_cast<uintptr_t>(t->q_dev) & 15) || (t->q_seq_stride % 8) || (t->q_head_stride % 8))
     return fail(FCA_ERR_INVALID_ARG, "q must be 16-byte aligned with strides that are multiples of 8 elements");
   if ((reinterpret_cast<uintptr_t>(t->k_cache_dev) & 15) || (reinterpret_cast<uintptr_t>(t->v_cache_dev) & 15) ||
@@ -76,7 +87,7 @@ int check_tensors(const fca_plan* p, const fca_tensors* t) {
 
 fca::AttendParams attend_params(const fca_plan* p, const fca_tensors* t, void* meta, void* po, float* pl, int select) {
   const fca::MetaLayout L = fca::make_layout(*p);
-  const int esz = t->kv_dtype == FCA_FP8_E4M3 ? 1 : 2;
+  const int esz = kv_elem_bytes(t->kv_dtype);
   fca::AttendParams a{};
   a.q = t->q_dev;
   a.q_seq_stride = t->q_seq_stride;
@@ -111,19 +122,22 @@ fca::AttendParams attend_params(const fca_plan* p, const fca_tensors* t, void* m
   return a;
 }
 
-int run_attend(const fca_plan* p, const fca_tensors* t, void* meta, void* po, float* pl, int select, void* stream) {
+int run_attend(const fca_plan* p, const fca_tensors* t, void* meta, void* po, float* pl, int select, void* stream,
+               bool f32_ok = false) {
   if (int rc = check_plan(p)) return rc;
-  if (int rc = check_tensors(p, t)) return rc;
+  if (int rc = check_tensors(p, t, f32_ok)) return rc;
   if (!meta || !po || !pl) return fail(FCA_ERR_INVALID_ARG, "metadata and partial workspaces must be non-NULL");
   if ((reinterpret_cast<uintptr_t>(po) & 15) || (reinterpret_cast<uintptr_t>(pl) & 15))
     return fail(FCA_ERR_INVALID_ARG, "partial workspaces must be 16-byte aligned");
   const fca::AttendParams a = attend_params(p, t, meta, po, pl, select);
-  hipError_t e = fca::launch_attend(a, *p, t->kv_dtype, t->max_workgroups, static_cast<hipStream_t>(stream));
+  hipError_t e = t->kv_dtype == FCA_F32
+                     ? fca::launch_attend_f32(a, *p, t->max_workgroups, static_cast<hipStream_t>(stream))
+                     : fca::launch_attend(a, *p, t->kv_dtype, t->max_workgroups, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? FCA_OK : hip_fail(e, "attention pass launch");
 }
 
 int run_merge(const fca_plan* p, const void* meta, const void* po, const float* pl, void* out, int64_t oss, int64_t ohs,
-              int32_t out_dtype, float* lse, void* stream) {
+              int32_t out_dtype, float* lse, void* stream, bool partial_f32 = false) {
   if (int rc = check_plan(p)) return rc;
   if (!meta || !po || !pl || !out) return fail(FCA_ERR_INVALID_ARG, "metadata, partials and out must be non-NULL");
   if (out_dtype != FCA_BF16 && out_dtype != FCA_F32)
@@ -146,6 +160,7 @@ int run_merge(const fca_plan* p, const void* meta, const void* po, const float* 
   m.max_partials = (int32_t)L.max_partials;
   m.coop_row0 = (int64_t)p->num_seqs * L.max_partials * p->num_q_heads;
   m.coop_rows = 32 * fca::coop_pairs_for(*p, L);
+  m.partial_f32 = partial_f32;
   m.out_dtype = out_dtype;
   // whole 16-byte stores when every 8-channel group of out is 16-byte aligned
   const int64_t esz = out_dtype == FCA_F32 ? 4 : 2;
@@ -163,12 +178,19 @@ int fca_version(void) { return FCA_VERSION; }
 const char* fca_last_error(void) { return g_error; }
 
 int fca_workspace_bytes(const fca_plan* plan, size_t* meta_bytes, size_t* partial_out_bytes, size_t* partial_lse_bytes) {
+  return fca_workspace_bytes_dtype(plan, FCA_BF16, meta_bytes, partial_out_bytes, partial_lse_bytes);
+}
+
+int fca_workspace_bytes_dtype(const fca_plan* plan, int32_t kv_dtype, size_t* meta_bytes, size_t* partial_out_bytes,
+                              size_t* partial_lse_bytes) {
   if (int rc = check_plan(plan)) return rc;
+  if (kv_dtype != FCA_BF16 && kv_dtype != FCA_FP8_E4M3 && kv_dtype != FCA_F32)
+    return fail(FCA_ERR_UNSUPPORTED, "kv_dtype %d is not supported (bf16, fp8 e4m3 or fp32)", kv_dtype);
   const fca::MetaLayout L = fca::make_layout(*plan);
   // one row per (partial slot, query head), then 32 rows per pair of waves that may share an item
   const size_t rows = (size_t)plan->num_seqs * (size_t)L.max_partials * plan->num_q_heads + 32 * (size_t)fca::coop_pairs_for(*plan, L);
   if (meta_bytes) *meta_bytes = (size_t)L.total * sizeof(int32_t);
-  if (partial_out_bytes) *partial_out_bytes = rows * plan->head_dim * 2;  // half
+  if (partial_out_bytes) *partial_out_bytes = rows * plan->head_dim * (kv_dtype == FCA_F32 ? 4 : 2);  // fp32 or half
   if (partial_lse_bytes) *partial_lse_bytes = rows * 2 * sizeof(float);    // {lse, scale}
   return FCA_OK;
 }
@@ -284,9 +306,9 @@ int fca_merge(const fca_plan* plan, const void* meta_dev, const void* partial_ou
 int fca_decode_step(const fca_plan* plan, const fca_tensors* t, void* meta_dev, void* partial_out_dev,
                     float* partial_lse_dev, void* out_dev, int64_t out_seq_stride, int64_t out_head_stride,
                     int32_t out_dtype, float* lse_dev, void* stream) {
-  if (int rc = run_attend(plan, t, meta_dev, partial_out_dev, partial_lse_dev, 0, stream)) return rc;
+  if (int rc = run_attend(plan, t, meta_dev, partial_out_dev, partial_lse_dev, 0, stream, true)) return rc;
   return run_merge(plan, meta_dev, partial_out_dev, partial_lse_dev, out_dev, out_seq_stride, out_head_stride, out_dtype,
-                   lse_dev, stream);
+                   lse_dev, stream, t->kv_dtype == FCA_F32);
 }
 
 }  // extern "C"
@@ -327,7 +349,8 @@ int fca_decode_step_static(const fca_plan* plan, const fca_tensors* t, void* met
                            int64_t out_seq_stride, int64_t out_head_stride, int32_t out_dtype, float* lse_dev,
                            void* stream) {
   size_t po = 0, pl = 0;
-  if (int rc = fca_workspace_bytes(plan, nullptr, &po, &pl)) return rc;
+  if (!t) return fail(FCA_ERR_INVALID_ARG, "tensors is NULL");
+  if (int rc = fca_workspace_bytes_dtype(plan, t->kv_dtype, nullptr, &po, &pl)) return rc;
   const size_t lse_at = (po + 255) / 256 * 256;
   if (lse_at + pl > (size_t)FCA_STATIC_SCRATCH_BYTES)
     return fail(FCA_ERR_UNSUPPORTED,
@@ -340,9 +363,9 @@ int fca_decode_step_static(const fca_plan* plan, const fca_tensors* t, void* met
   // the attention launch of the same call, so nothing of the last call's contents is read.
   void* partial_out = base;
   float* partial_lse = reinterpret_cast<float*>(base + lse_at);
-  if (int rc = run_attend(plan, t, meta_dev, partial_out, partial_lse, 0, stream)) return rc;
+  if (int rc = run_attend(plan, t, meta_dev, partial_out, partial_lse, 0, stream, true)) return rc;
   return run_merge(plan, meta_dev, partial_out, partial_lse, out_dev, out_seq_stride, out_head_stride, out_dtype, lse_dev,
-                   stream);
+                   stream, t->kv_dtype == FCA_F32);
 }
 
 static int cache_rows(bool gather, const void* key_dev, const void* value_dev, int64_t token_stride, int64_t head_stride,

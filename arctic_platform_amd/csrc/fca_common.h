@@ -198,6 +198,7 @@ struct MergeParams {
   int32_t vector_out;  // out rows allow 16-byte stores
   int64_t coop_row0;   // first of the partial rows written by waves that took a shared item from the back
   int64_t coop_rows;   // how many such rows the partial buffers hold: a tag that points past them is not followed
+  int32_t partial_f32; // the partial rows are fp32 (written by the fp32 attention pass), not scaled halves
 };
 
 struct AppendParams {
@@ -275,6 +276,7 @@ hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dty
 // Events the next attention launch of this thread records its begin and end in (NULL: none).
 void set_attend_timing(hipEvent_t start, hipEvent_t stop);
 void take_attend_timing(hipEvent_t* start, hipEvent_t* stop);
+hipError_t launch_attend_f32(const AttendParams& p, const fca_plan& plan, int max_workgroups, hipStream_t stream);
 hipError_t launch_attend32(const AttendParams& p, const fca_plan& plan, int kv_dtype, int grid, hipStream_t stream);
 hipError_t launch_merge(const MergeParams& p, hipStream_t stream);
 hipError_t launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);

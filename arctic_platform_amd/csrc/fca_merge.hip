@@ -3,6 +3,8 @@
 // arctic_platform/model/implementations/qwen35/models/layers/lm_head.py:190-202.
 #include <hip/hip_bf16.h>
 
+#include <type_traits>
+
 #include "fca_common.h"
 
 namespace fca {
@@ -10,15 +12,19 @@ namespace fca {
 constexpr int kMergeThreads = 256;
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
 
 // D / 8 lanes per (sequence, query head) row and share; each lane owns 8 adjacent channels
 // (16 bytes of a half-precision partial row).  A partial row is its stored halves times the
 // row's scale; {lse, scale} sit side by side.  With SPLIT > 1 (plans with many partials per
 // row: long contexts cut into many chunks) SPLIT such lane groups take every SPLIT-th
 // partial of the row each and combine their running results at the end, which puts SPLIT
-// times the loads in flight.
-template <int D, int SPLIT>
+// times the loads in flight.  F32: the partial rows are fp32 (the fp32 attention pass), 32 bytes
+// per lane, with scale 1.
+template <int D, int SPLIT, bool F32 = false>
 __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p) {
+  using RowElem = std::conditional_t<F32, float, _Float16>;
+  using Row8 = std::conditional_t<F32, f32x8, f16x8>;
   constexpr int V = 8;
   constexpr int kLanesPerShare = D / V;
   constexpr int kLanesPerRow = kLanesPerShare * SPLIT;
@@ -31,7 +37,7 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
   const int s = live_row ? row / p.num_q_heads : 0, hq = live_row ? row - s * p.num_q_heads : 0;
   const int np = live_row ? p.seq_npart[s] : 0;
   const int64_t base = (int64_t)s * p.max_partials;
-  const _Float16* rows = static_cast<const _Float16*>(p.partial_out);
+  const RowElem* rows = static_cast<const RowElem*>(p.partial_out);
   const float2* lse_scale = reinterpret_cast<const float2*>(p.partial_lse);
 
   // One online pass (running maximum, rescaled sum): the loads of successive partials do
@@ -41,7 +47,7 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
   float acc[V];
 #pragma unroll
   for (int e = 0; e < V; ++e) acc[e] = 0.f;
-  auto take = [&](float l, float scale, const f16x8& o) {
+  auto take = [&](float l, float scale, const Row8& o) {
     if (!(l > -INFINITY)) return;  // empty partial: weight 0, whatever its output holds
     const float m_new = fmaxf(m, l);
     const float keep = __expf(m - m_new);  // exp(-inf) = 0 on the first live partial
@@ -59,7 +65,7 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
     typedef float f2v __attribute__((ext_vector_type(2)));
     const f2v lsv = __builtin_nontemporal_load(reinterpret_cast<const f2v*>(lse_scale + pr));
     const float2 ls = make_float2(lsv[0], lsv[1]);
-    const f16x8 o = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(rows + pr * D + sub * V));
+    const Row8 o = __builtin_nontemporal_load(reinterpret_cast<const Row8*>(rows + pr * D + sub * V));
     // the scale is a power of two; its mantissa bits say where a second partial of the same
     // chunk is (an item attended by two waves of the attention kernel), 0 = nowhere
     const unsigned sbits = __float_as_uint(ls.y);
@@ -73,7 +79,7 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
       if (rel >= 0 && rel < p.coop_rows) {
         const int64_t br = p.coop_row0 + rel;
         const float2 bls = lse_scale[br];
-        const f16x8 bo = *reinterpret_cast<const f16x8*>(rows + br * D + sub * V);
+        const Row8 bo = *reinterpret_cast<const Row8*>(rows + br * D + sub * V);
         take(bls.x, __uint_as_float(__float_as_uint(bls.y) & 0xff800000u), bo);
       } else {
         stray = 1;
@@ -148,7 +154,15 @@ hipError_t launch_merge(const MergeParams& p, hipStream_t stream) {
   const int per_block = kMergeThreads / (p.head_dim / 8 * split);
   const int grid = (rows + per_block - 1) / per_block;
 #define FCA_MERGE(D_, S_) hipLaunchKernelGGL((fca_merge_kernel<D_, S_>), dim3(grid), dim3(kMergeThreads), 0, stream, p)
-  if (p.head_dim == 256) {
+  if (p.partial_f32) {  // head sizes 64 and 128 (checked with the tensors)
+    if (p.head_dim == 128) {
+      if (split == 4) hipLaunchKernelGGL((fca_merge_kernel<128, 4, true>), dim3(grid), dim3(kMergeThreads), 0, stream, p);
+      else hipLaunchKernelGGL((fca_merge_kernel<128, 1, true>), dim3(grid), dim3(kMergeThreads), 0, stream, p);
+    } else {
+      if (split == 4) hipLaunchKernelGGL((fca_merge_kernel<64, 4, true>), dim3(grid), dim3(kMergeThreads), 0, stream, p);
+      else hipLaunchKernelGGL((fca_merge_kernel<64, 1, true>), dim3(grid), dim3(kMergeThreads), 0, stream, p);
+    }
+  } else if (p.head_dim == 256) {
     if (split == 2) FCA_MERGE(256, 2); else FCA_MERGE(256, 1);
   } else if (p.head_dim == 128) {
     if (split == 4) FCA_MERGE(128, 4); else FCA_MERGE(128, 1);

@@ -174,6 +174,7 @@ def build_forest_metadata(
     row_table: torch.Tensor | None = None,
     row_group: torch.Tensor | None = None,
     kv_reread: bool | None = None,
+    partial_dtype: torch.dtype | None = None,
 ) -> ForestMetadata:
     """Discover the shared-prefix forest of a decode batch on the device.
 
@@ -184,6 +185,8 @@ def build_forest_metadata(
     groups of rows that share their leading blocks (``fca_build_metadata_rows``).
     ``kv_reread`` says whether a launch reads KV blocks again and again (long query runs,
     many tiles per sequence); the default assumes so when groups are declared.
+    ``partial_dtype=torch.float32`` sizes the partial rows for the all-fp32 path (fp32 queries on
+    an fp32 cache); the default is the scaled half-precision rows of the bf16 / fp8 kernels.
 
     ``cascade=False`` turns sharing off: every sequence becomes one private node over its
     whole block-table row, which makes the same kernels a plain paged decode attention.
@@ -219,7 +222,10 @@ def build_forest_metadata(
         rows_per_item=rows_per_item,
         max_levels=max_levels if cascade else 0,
     )
-    same_workspace = out is not None and bytes(out.plan) == bytes(plan)
+    if partial_dtype not in (None, torch.float16, torch.float32):
+        raise ValueError(f"partial_dtype must be torch.float32 or None, got {partial_dtype}")
+    partial_dtype = partial_dtype or torch.float16
+    same_workspace = out is not None and bytes(out.plan) == bytes(plan) and out.partial_out.dtype == partial_dtype
     if same_workspace:
         md = dataclasses.replace(out, block_table=block_table, seq_lens=seq_lens, row_table=row_table, row_group=row_group)
         md.kv_reread = row_group is not None if kv_reread is None else bool(kv_reread)
@@ -227,13 +233,14 @@ def build_forest_metadata(
         layout = _lib.FcaMetaLayout()
         _lib.check(lib.fca_meta_describe(ctypes.byref(plan), ctypes.byref(layout)))
         nm, no, nl = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
-        _lib.check(lib.fca_workspace_bytes(ctypes.byref(plan), ctypes.byref(nm), ctypes.byref(no), ctypes.byref(nl)))
+        kv_dtype = _lib.FCA_F32 if partial_dtype == torch.float32 else _lib.FCA_BF16
+        _lib.check(lib.fca_workspace_bytes_dtype(ctypes.byref(plan), kv_dtype, ctypes.byref(nm), ctypes.byref(no), ctypes.byref(nl)))
         dev = block_table.device
         md = ForestMetadata(
             plan=plan,
             layout=layout,
             meta=torch.zeros(nm.value // 4, dtype=torch.int32, device=dev),
-            partial_out=torch.empty(no.value // 2, dtype=torch.float16, device=dev),
+            partial_out=torch.empty(no.value // (4 if partial_dtype == torch.float32 else 2), dtype=partial_dtype, device=dev),
             # (zeros: a merge that runs before any attention pass has written the buffers then
             # finds plain empty rows, not row scales that point somewhere)
             partial_lse=torch.zeros(nl.value // 4, dtype=torch.float32, device=dev),

@@ -23,18 +23,25 @@ from .forest import ForestMetadata, _stream_ptr
 from .kv_layout import BLOCK_SIZE
 
 
-def _tensors(q, kv_cache, meta: ForestMetadata, scale, k_scale, v_scale) -> _lib.FcaTensors:
+def _tensors(q, kv_cache, meta: ForestMetadata, scale, k_scale, v_scale, f32_ok=False) -> _lib.FcaTensors:
     plan = meta.plan
-    if q.dtype != torch.bfloat16:
-        raise TypeError("q must be bfloat16")
-    if q.shape != (plan.num_seqs, plan.num_q_heads, plan.head_dim) or q.stride(2) != 1:
-        raise ValueError(f"q must be [{plan.num_seqs}, {plan.num_q_heads}, {plan.head_dim}] with contiguous head_dim")
-    if kv_cache.dtype == torch.bfloat16:
+    if q.dtype == torch.float32 or kv_cache.dtype == torch.float32:
+        # the all-fp32 path: fp32 queries on an fp32 cache, fp32 partial rows
+        if q.dtype != kv_cache.dtype:
+            raise TypeError(f"the fp32 path takes q and the KV cache both in float32, got {q.dtype} and {kv_cache.dtype}")
+        if not f32_ok:
+            raise TypeError("float32 tensors run through forest_cascade_decode (and its static variant) only")
+        kv_dtype = _lib.FCA_F32
+    elif q.dtype != torch.bfloat16:
+        raise TypeError("q must be bfloat16 (or float32 with a float32 KV cache)")
+    elif kv_cache.dtype == torch.bfloat16:
         kv_dtype = _lib.FCA_BF16
     elif kv_cache.dtype == torch.float8_e4m3fn:
         kv_dtype = _lib.FCA_FP8_E4M3
     else:
-        raise TypeError(f"unsupported KV cache dtype {kv_cache.dtype} (bfloat16 or float8_e4m3fn)")
+        raise TypeError(f"unsupported KV cache dtype {kv_cache.dtype} (bfloat16, float8_e4m3fn, or float32 with a float32 q)")
+    if q.shape != (plan.num_seqs, plan.num_q_heads, plan.head_dim) or q.stride(2) != 1:
+        raise ValueError(f"q must be [{plan.num_seqs}, {plan.num_q_heads}, {plan.head_dim}] with contiguous head_dim")
     if (
         kv_cache.dim() != 4
         or kv_cache.shape[0] != 2
@@ -69,6 +76,16 @@ def _tensors(q, kv_cache, meta: ForestMetadata, scale, k_scale, v_scale) -> _lib
     )
 
 
+def _check_partials(meta: ForestMetadata, t) -> None:
+    """fp32 tensors write fp32 partial rows: the workspace must have been sized for them."""
+    want = torch.float32 if t.kv_dtype == _lib.FCA_F32 else torch.float16
+    if meta.partial_out.dtype != want:
+        raise ValueError(
+            f"the metadata's partial rows are {meta.partial_out.dtype}, these tensors need {want}: "
+            "build the metadata with partial_dtype=torch.float32 for float32 tensors (and without for the others)"
+        )
+
+
 def _out_args(q, meta, out, out_dtype):
     plan = meta.plan
     if out is None:
@@ -87,10 +104,13 @@ def _out_args(q, meta, out, out_dtype):
 def forest_cascade_decode(
     q, kv_cache, meta: ForestMetadata, scale, k_scale=None, v_scale=None, out=None, return_lse=True, out_dtype=None
 ):
-    """One layer's decode attention.  Returns ``out`` or ``(out, lse)``."""
+    """One layer's decode attention.  Returns ``out`` or ``(out, lse)``.  ``q`` and ``kv_cache``
+    in float32 take the all-fp32 path (fp32 products and partial rows; ``out`` then defaults to
+    float32): the metadata must have been built with ``partial_dtype=torch.float32``."""
     lib = _lib.load_library()
-    t = _tensors(q, kv_cache, meta, scale, k_scale, v_scale)
-    out, code = _out_args(q, meta, out, out_dtype)
+    t = _tensors(q, kv_cache, meta, scale, k_scale, v_scale, f32_ok=True)
+    _check_partials(meta, t)
+    out, code = _out_args(q, meta, out, out_dtype or (torch.float32 if t.kv_dtype == _lib.FCA_F32 else None))
     lse = torch.empty(meta.plan.num_seqs, meta.plan.num_q_heads, dtype=torch.float32, device=q.device) if return_lse else None
     _lib.check(
         lib.fca_decode_step(
@@ -117,7 +137,7 @@ def forest_cascade_decode_static(q, kv_cache, meta: ForestMetadata, scale, k_sca
     Plans whose partial rows exceed ``_lib.FCA_STATIC_SCRATCH_BYTES`` raise.  All calls on
     one GPU share the buffers: keep them in stream order."""
     lib = _lib.load_library()
-    t = _tensors(q, kv_cache, meta, scale, k_scale, v_scale)
+    t = _tensors(q, kv_cache, meta, scale, k_scale, v_scale, f32_ok=True)
     out, code = _out_args(q, meta, out, None)
     if lse is not None and (lse.dtype != torch.float32 or lse.shape != (meta.plan.num_seqs, meta.plan.num_q_heads) or not lse.is_contiguous()):
         raise ValueError("lse must be a contiguous fp32 tensor [num_seqs, num_q_heads]")
@@ -168,6 +188,8 @@ def forest_pass(q, kv_cache, meta: ForestMetadata, scale, k_scale=None, v_scale=
 
 def merge_partials(meta: ForestMetadata, q_like, out=None, return_lse=True, out_dtype=None):
     """Log-sum-exp merge of the partial buffers into ``out`` (and ``lse``)."""
+    if meta.partial_out.dtype != torch.float16:
+        raise TypeError("merge_partials reads the half-precision partial rows of the bf16 / fp8 passes; fp32 rows are merged inside forest_cascade_decode")
     lib = _lib.load_library()
     out, code = _out_args(q_like, meta, out, out_dtype)
     lse = torch.empty(meta.plan.num_seqs, meta.plan.num_q_heads, dtype=torch.float32, device=out.device) if return_lse else None

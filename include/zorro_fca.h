@@ -49,12 +49,17 @@ typedef enum fca_status {
 } fca_status;
 
 /* q is bf16 and the KV cache bf16 or fp8: the products run on the bf16 matrix cores with
- * fp32 accumulation.  An fp32 q or KV cache is refused (FCA_ERR_UNSUPPORTED) by every entry
- * point that takes one; fp32 is available for the outputs only. */
+ * fp32 accumulation.  kv_dtype FCA_F32 is the all-fp32 path of the small fp32 configuration:
+ * q, the KV cache and the partial rows are fp32 and so is every product (vector units; the
+ * chip has no more fp32 rate in its matrix cores), at the precision of the reference's
+ * softmax-in-fp32 attention (arctic_platform/rl/zorro_train/qwen_attention_patcher.py:55-61).
+ * It runs through fca_decode_step and fca_decode_step_static only, at head sizes 64 and 128
+ * with rows_per_item 32; the other entry points that take tensors refuse it, and the cache
+ * writer has no fp32 instance. */
 typedef enum fca_dtype {
   FCA_BF16 = 0,     /* q, out, KV cache */
   FCA_FP8_E4M3 = 1, /* KV cache only (OCP e4m3fn) */
-  FCA_F32 = 2       /* out only */
+  FCA_F32 = 2       /* out; as kv_dtype: q and the KV cache are fp32 */
 } fca_dtype;
 
 /* Shape of one decode batch and the tiling the metadata is built for. */
@@ -72,14 +77,14 @@ typedef struct fca_plan {
 
 /* Tensors of one attention layer. */
 typedef struct fca_tensors {
-  const void* q_dev;           /* bf16 [S, Hq, D], D contiguous */
+  const void* q_dev;           /* bf16 (fp32 when kv_dtype is FCA_F32) [S, Hq, D], D contiguous */
   int64_t q_seq_stride;
   int64_t q_head_stride;
   const void* k_cache_dev;     /* K plane: [num_blocks, Hkv, D/x, 16, x], x = 16 bytes / elem size */
   const void* v_cache_dev;     /* V plane: [num_blocks, Hkv, D, 16] */
   int64_t kv_block_stride;     /* elements between blocks of one plane */
   int64_t kv_head_stride;      /* elements between KV heads of one block */
-  int32_t kv_dtype;            /* FCA_BF16 or FCA_FP8_E4M3 */
+  int32_t kv_dtype;            /* FCA_BF16, FCA_FP8_E4M3, or FCA_F32 (then q is fp32 as well) */
   int32_t kv_reread;           /* 0: a launch reads every KV block about once (decode), loads bypass
                                   the caches; non-zero: blocks are read again and again (query runs
                                   built with fca_build_metadata_rows), loads stay cacheable */
@@ -142,6 +147,10 @@ const char* fca_last_error(void);
  * item, so that it leaves alone what fca_prefix_pass wrote there for the same merge).  Both
  * are opaque to the caller: written by the passes, read by the merge. */
 int fca_workspace_bytes(const fca_plan* plan, size_t* meta_bytes, size_t* partial_out_bytes, size_t* partial_lse_bytes);
+/* The same for a given kv_dtype: with FCA_F32 the partial rows are fp32 (partial_out twice the
+ * bytes); FCA_BF16 and FCA_FP8_E4M3 give what fca_workspace_bytes gives. */
+int fca_workspace_bytes_dtype(const fca_plan* plan, int32_t kv_dtype, size_t* meta_bytes, size_t* partial_out_bytes,
+                              size_t* partial_lse_bytes);
 int fca_meta_describe(const fca_plan* plan, fca_meta_layout* layout);
 
 /* Forest metadata builder: block tables + lengths -> flat node / member / work-item arrays.

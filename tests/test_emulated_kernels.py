@@ -250,6 +250,94 @@ def test_separate_passes_with_shared_items_equal_the_fused_step(emu):
     assert_matches_oracle(res[0][0], res[0][1], ref_out, ref_lse, what="reproducible step")
 
 
+# ---- the all-fp32 path --------------------------------------------------------------------------------
+def _decode_f32(lib, w, chunk, max_levels=4, static=False):
+    """fca_decode_step on fp32 queries and an fp32 cache; returns (metadata, out fp32, lse)."""
+    S, mb = w.block_table.shape
+    plan = make_plan(S, mb, w.num_q_heads, w.num_kv_heads, w.head_dim, chunk_tokens=chunk, rows_per_item=32, max_levels=max_levels)
+    layout = _lib.FcaMetaLayout()
+    _ok(lib, lib.fca_meta_describe(ctypes.byref(plan), ctypes.byref(layout)))
+    nm, no, nl = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    _ok(lib, lib.fca_workspace_bytes_dtype(ctypes.byref(plan), _lib.FCA_F32, ctypes.byref(nm), ctypes.byref(no), ctypes.byref(nl)))
+    half = ctypes.c_size_t()
+    _ok(lib, lib.fca_workspace_bytes(ctypes.byref(plan), None, ctypes.byref(half), None))
+    assert no.value == 2 * half.value
+    meta = guarded(torch.zeros(nm.value // 4, dtype=torch.int32))
+    po = guarded(torch.full((no.value // 4,), float("nan"), dtype=torch.float32))
+    pl = guarded(torch.full((nl.value // 4,), float("nan"), dtype=torch.float32))
+    bt, sl = guarded(w.block_table), guarded(w.seq_lens)
+    q, kv = guarded(w.q), guarded(w.kv_cache)
+    assert q.dtype == torch.float32 and kv.dtype == torch.float32
+    _ok(lib, lib.fca_build_metadata(ctypes.byref(plan), bt.data_ptr(), bt.stride(0), sl.data_ptr(), meta.data_ptr(), None))
+    md = ForestMetadata(plan=plan, layout=layout, meta=meta, partial_out=po, partial_lse=pl, block_table=bt, seq_lens=sl)
+    md.check()
+    t = _lib.FcaTensors(
+        q.data_ptr(), q.stride(0), q.stride(1), kv.data_ptr(), kv.data_ptr() + kv.stride(0) * 4, kv.stride(1), kv.stride(2),
+        _lib.FCA_F32, 0, bt.data_ptr(), bt.stride(0), None, None, float(w.scale), 0, EMU_WORKGROUPS,
+    )
+    out = guarded(torch.full((S, w.num_q_heads, w.head_dim), float("nan"), dtype=torch.float32))
+    lse = guarded(torch.full((S, w.num_q_heads), float("nan"), dtype=torch.float32))
+    if static:
+        _ok(lib, lib.fca_decode_step_static(ctypes.byref(plan), ctypes.byref(t), meta.data_ptr(), out.data_ptr(), out.stride(0), out.stride(1), _lib.FCA_F32, lse.data_ptr(), None))
+    else:
+        _ok(lib, lib.fca_decode_step(ctypes.byref(plan), ctypes.byref(t), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), out.data_ptr(), out.stride(0), out.stride(1), _lib.FCA_F32, lse.data_ptr(), None))
+    assert int(meta[layout.header + 3]) == 0
+    # the other entry points that take tensors have no fp32 path and say so
+    assert lib.fca_forest_pass(ctypes.byref(plan), ctypes.byref(t), meta.data_ptr(), po.data_ptr(), pl.data_ptr(), None) == -2
+    assert b"fca_decode_step" in lib.fca_last_error()
+    return md, out, lse
+
+
+def _assert_fp32_close(out, lse, w, what):
+    """fp32 arithmetic on fp32 inputs against the fp64 oracle on the same inputs: 2e-5."""
+    ref_out, ref_lse = oracle_for(w)
+    err = (out.double() - ref_out).abs()
+    assert bool((err <= 2e-5 + 2e-5 * ref_out.abs()).all()), f"{what}: out max |err| {err.max():.3g}"
+    lerr = (lse.double() - ref_lse).abs().max()
+    assert lerr <= 2e-5, f"{what}: lse max |err| {lerr:.3g}"
+
+
+@pytest.mark.parametrize("chunk", [32, 96, 512])
+def test_fp32_configuration_1(emu, chunk):
+    """The small fp32 configuration as it is defined (fp32 q, K, V): outputs and log-sum-exp to
+    fp32 accuracy, and the committed golden result of the fp64 oracle on the same values."""
+    import numpy as np
+
+    from arctic_platform_amd.workloads import make_config
+
+    w = make_config(1, device="cpu", poison_unused=True)
+    assert w.q.dtype == torch.float32 and w.kv_cache.dtype == torch.float32
+    md, out, lse = _decode_f32(emu, w, chunk)
+    _check_nodes(md, w)
+    _assert_fp32_close(out, lse, w, f"C1 fp32, chunk {chunk}")
+    gold = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "config1.npz"))
+    assert float(np.abs(out.numpy() - gold["out"]).max()) <= 2e-5
+    assert float(np.abs(lse.numpy() - gold["lse"]).max()) <= 2e-5
+
+
+@pytest.mark.parametrize("case", [c for c in CASES if c[0] in (2, 5, 7, 12, 15)], ids=lambda c: f"seed{c[0]}")
+def test_fp32_random_forests(emu, case):
+    """Random forests (several levels, ragged lengths, GQA groups that do not fill a tile) in fp32,
+    head sizes 64 and 128, on caller-owned partial buffers and on the library's own."""
+    seed, hq, hkv, d, kv_dtype, depth, fanout, len_range, leaf_range, chunk, rows = case
+    if d == 256:
+        pytest.skip("the fp32 path has head sizes 64 and 128")
+    seg_len, paths = random_forest(random.Random(seed), depth, fanout, len_range, leaf_range)
+    w = make_forest_workload(
+        "random", seg_len, paths, torch.Generator().manual_seed(seed), num_q_heads=hq, num_kv_heads=hkv, head_dim=d,
+        dtype=torch.float32, device="cpu", poison_unused=True,
+    )
+    md, out, lse = _decode_f32(emu, w, chunk)
+    _check_nodes(md, w)
+    _assert_fp32_close(out, lse, w, f"seed {seed}")
+    _, out2, lse2 = _decode_f32(emu, w, chunk, static=True)
+    assert torch.equal(out2, out) and torch.equal(lse2, lse)
+    # sharing off: the same kernel as a plain paged decode attention
+    md0, out0, lse0 = _decode_f32(emu, w, chunk, max_levels=0)
+    assert md0.header()["shared_items"] == 0
+    _assert_fp32_close(out0, lse0, w, f"seed {seed}, sharing off")
+
+
 @pytest.mark.parametrize("rows,d", [(32, 128), (64, 128), (32, 64), (32, 256)])
 def test_merge_stays_inside_buffers_of_random_bits(emu, rows, d):
     """fca_merge on partial buffers nothing has written: whatever bits they hold, every load stays
