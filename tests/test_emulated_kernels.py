@@ -202,9 +202,9 @@ def test_separate_passes_with_shared_items_equal_the_fused_step(emu):
     enough long items for pairs of waves to attend some together: the launch over the private
     items shares none, so the second partials that the launch over the shared items left are
     still there when the merge follows them."""
-    hq, hkv, d, chunk = 16, 4, 128, 512
+    hq, hkv, d, chunk = 16, 4, 128, 256
     gen = torch.Generator().manual_seed(311)
-    seg_len, paths = two_level_forest(gen, 12, 5, (700, 2500), (230, 900))
+    seg_len, paths = two_level_forest(gen, 10, 4, (400, 1200), (230, 500))
     w = make_forest_workload("two-level", seg_len, paths, gen, num_q_heads=hq, num_kv_heads=hkv, head_dim=d, device="cpu", poison_unused=True)
     md, out, lse = _decode(emu, w, chunk, 32)
     waves = 4 * EMU_WORKGROUPS
