@@ -53,6 +53,8 @@ class FcaSplitPlan(ctypes.Structure):
         ("num_kv_heads", ctypes.c_int32),
         ("head_dim", ctypes.c_int32),
         ("window", ctypes.c_int32),
+        ("dropout_p", ctypes.c_float),
+        ("dropout_seed", ctypes.c_uint32),
     ]
 
 

@@ -466,7 +466,22 @@ int check_split(const fca_split_plan* p) {
                 "their operands through LDS have an instance of that size",
                 p->num_q_heads / p->num_kv_heads);
   if (p->window < 0) return fail(FCA_ERR_INVALID_ARG, "window must be >= 0 (0 = none), got %d", p->window);
+  if (!(p->dropout_p >= 0.f && p->dropout_p < 1.f))
+    return fail(FCA_ERR_INVALID_ARG, "dropout_p must lie in [0, 1), got %g", (double)p->dropout_p);
   return FCA_OK;
+}
+// window, dropout threshold, scale and seed of a plan, as the kernels take them
+void split_options(const fca_split_plan* plan, fca::SplitParams* p) {
+  p->window = plan->window;
+  p->drop_thr = 0, p->drop_scale = 1.f, p->drop_seed = 0;
+  if (plan->dropout_p > 0.f) {
+    const double thr = (double)plan->dropout_p * 4294967296.0;
+    p->drop_thr = thr >= 4294967295.0 ? 4294967295u : thr < 1.0 ? 1u : (uint32_t)thr;
+    p->drop_scale = 1.f / (1.f - plan->dropout_p);
+    p->drop_seed = plan->dropout_seed;
+    // the general instances test a window too: one that no sequence reaches
+    if (p->window == 0) p->window = 0x3fffffff;
+  }
 }
 int check_rows(const char* name, const void* ptr, int64_t stride, int heads, int head_dim) {
   if (!ptr) return fail(FCA_ERR_INVALID_ARG, "%s is NULL", name);
@@ -556,7 +571,7 @@ int fca_split_attention_forward(const fca_split_plan* plan, const void* q_dev, i
   p.num_q_heads = plan->num_q_heads;
   p.num_kv_heads = plan->num_kv_heads;
   p.scale = scale;
-  p.window = plan->window;
+  split_options(plan, &p);
   hipError_t e = fca::launch_split_forward(p, plan->head_dim, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? FCA_OK : hip_fail(e, "split attention forward launch");
 }
@@ -608,7 +623,7 @@ int fca_split_attention_backward(const fca_split_plan* plan, const void* q_dev, 
   p.num_q_heads = hq;
   p.num_kv_heads = hkv;
   p.scale = scale;
-  p.window = plan->window;
+  split_options(plan, &p);
   hipError_t e = fca::launch_split_backward(p, d, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? FCA_OK : hip_fail(e, "split attention backward launch");
 }

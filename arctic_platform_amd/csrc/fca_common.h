@@ -234,10 +234,26 @@ struct SplitParams {
   // small batches: dk and dv are formed per query head (fp32 slices [Hq / Hkv][T][Hkv][D]) and summed afterwards
   int32_t head_split;
   float *dk_part, *dv_part;
-  // > 0: a row sees only the keys fewer than `window` positions before it in its own sequence
-  // (prompt followed by the sample's response); the kernels then have instances of their own
+  // The general instances of the kernels (chosen when a window or dropout is asked for):
+  // window > 0: a row sees only the keys fewer than `window` positions before it in its own
+  // sequence (prompt followed by the sample's response); none = a window no sequence reaches.
   int32_t window;
+  // Attention dropout: the probability of (query head, row, key) is dropped when
+  // split_dropout_hash(...) < drop_thr and scaled by drop_scale = 1 / (1 - p) otherwise.
+  uint32_t drop_thr, drop_seed;
+  float drop_scale;
 };
+// The hash that decides dropout, the same for all four kernels and for the tests' restatement:
+// one 32-bit mix (two multiplications) of a linear combination of the three indices and the seed.
+__host__ __device__ inline uint32_t split_dropout_hash(uint32_t seed, uint32_t head, uint32_t row, uint32_t key) {
+  uint32_t x = seed + head * 0xC2B2AE3Du + row * 0x9E3779B1u + key * 0x85EBCA77u;
+  x ^= x >> 16;
+  x *= 0x7FEB352Du;
+  x ^= x >> 15;
+  x *= 0x846CA68Bu;
+  x ^= x >> 16;
+  return x;
+}
 // A batch with few key tiles leaves most of the chip idle behind its longest walks (a prompt's
 // key tiles are seen by the whole group): then every query head of a KV head gets a workgroup
 // of its own, which shortens the longest walk by Hq / Hkv.

@@ -250,8 +250,10 @@ __global__ __launch_bounds__(kThreads) void split_images_kernel(const __bf16* x,
 // the L1 sees a quarter of the operand traffic.  Without it (query heads per KV head not a
 // multiple of four) every wave fetches its own tiles into two register buffers.  Head size
 // 256 runs one workgroup per CU (its accumulators and query rows alone take 192 registers).
-// WIN: the instances for a sliding window (p.window > 0).  Every pair of tiles is tested element
-// by element there, with the positions of row and key in their own sequence beside the limits.
+// WIN: the general instances, for a sliding window and for attention dropout.  Every pair of
+// tiles is tested element by element there, with the positions of row and key in their own
+// sequence beside the limits, and with dropout every probability draws its fate from a hash of
+// (seed, query head, row, key), so that the four kernels agree on it without a stored mask.
 template <int D, bool BWD, bool SHARED, bool WIN>
 __global__ __launch_bounds__(kThreads, SHARED && D < 256 ? 2 : 1) void split_query_kernel(SplitParams p) {
   constexpr int KS = D / 16, NDB = D / 32, SLOTS = (BWD ? 3 : 2) * KS, PER = SLOTS / kWaves;
@@ -282,6 +284,14 @@ __global__ __launch_bounds__(kThreads, SHARED && D < 256 ? 2 : 1) void split_que
   // the first position this lane's row still sees: keys at positions pos_lo .. its own
   int pos_lo = 0;
   if constexpr (WIN) pos_lo = p.layout[L.pos + r] - p.window + 1;
+  // dropout: the part of the hash argument that belongs to this lane's row and head
+  const uint32_t drop_base = WIN ? p.drop_seed + (uint32_t)hq * 0xC2B2AE3Du + (uint32_t)r * 0x9E3779B1u : 0u;
+  auto kept = [&](int j, int x) {  // register x of key tile j: key 32 j + 8 h + 16 (x / 8) + x % 8
+    const uint32_t key = (uint32_t)(32 * j + 8 * h + 16 * (x >> 3) + (x & 7));
+    uint32_t v = drop_base + key * 0x85EBCA77u;
+    v ^= v >> 16, v *= 0x7FEB352Du, v ^= v >> 15, v *= 0x846CA68Bu, v ^= v >> 16;
+    return v >= p.drop_thr;
+  };
 
   bf16x8 qreg[KS], doreg[BWD ? KS : 1];
 #pragma unroll
@@ -384,8 +394,11 @@ __global__ __launch_bounds__(kThreads, SHARED && D < 256 ? 2 : 1) void split_que
       float sum = 0.f;
 #pragma unroll
       for (int x = 0; x < 16; ++x) {
-        const float e = fast_exp2(__builtin_fmaf(sr[x], sc, -mrow));
-        sum += e;
+        float e = fast_exp2(__builtin_fmaf(sr[x], sc, -mrow));
+        sum += e;  // (the row sum, and with it the log-sum-exp, is that of the probabilities before dropout)
+        if constexpr (WIN) {
+          if (p.drop_thr) e = kept(j, x) ? e * p.drop_scale : 0.f;
+        }
         pb[x >> 3][x & 7] = (__bf16)e;
       }
       lrow += sum;
@@ -398,7 +411,11 @@ __global__ __launch_bounds__(kThreads, SHARED && D < 256 ? 2 : 1) void split_que
 #pragma unroll
       for (int x = 0; x < 16; ++x) {
         const float e = fast_exp2(__builtin_fmaf(sr[x], sc, -lse2));
-        pb[x >> 3][x & 7] = (__bf16)(e * (dp[x] - delta));
+        float d = dp[x];
+        if constexpr (WIN) {
+          if (p.drop_thr) d = kept(j, x) ? d * p.drop_scale : 0.f;  // dP through the dropout of the forward
+        }
+        pb[x >> 3][x & 7] = (__bf16)(e * (d - delta));
       }
     }
 #pragma unroll
@@ -539,6 +556,7 @@ __global__ __launch_bounds__(kThreads, D < 256 ? 2 : 1) void split_key_kernel(Sp
   // the last position that still sees this lane's key
   int pos_hi = 0;
   if constexpr (WIN) pos_hi = p.layout[L.pos + t] + p.window - 1;
+  const uint32_t drop_base = WIN ? p.drop_seed + (uint32_t)t * 0x85EBCA77u : 0u;  // this lane's key in the dropout hash
   const float sc = p.scale * kLog2e;
 
   bf16x8 kreg[KS], vreg[DK ? KS : 1];
@@ -638,7 +656,18 @@ __global__ __launch_bounds__(kThreads, D < 256 ? 2 : 1) void split_key_kernel(Sp
           for (int e4 = 0; e4 < 4; ++e4) {
             const int x = 4 * q4 + e4;
             float e = fast_exp2(__builtin_fmaf(sr[x], sc, -ls[e4]));
-            if constexpr (DK) e *= dp[x] - dl[e4];
+            if constexpr (WIN) {
+              float keep = 1.f;
+              if (p.drop_thr) {  // row 32 i + 8 h + 16 (x / 8) + x % 8 of query head hq0 + g
+                uint32_t v = drop_base + (uint32_t)(hq0 + g) * 0xC2B2AE3Du + (uint32_t)(row0 + 16 * (x >> 3) + (x & 7)) * 0x9E3779B1u;
+                v ^= v >> 16, v *= 0x7FEB352Du, v ^= v >> 15, v *= 0x846CA68Bu, v ^= v >> 16;
+                keep = v >= p.drop_thr ? p.drop_scale : 0.f;
+              }
+              if constexpr (DK) e *= dp[x] * keep - dl[e4];
+              else e *= keep;
+            } else {
+              if constexpr (DK) e *= dp[x] - dl[e4];
+            }
             pb[x >> 3][x & 7] = (__bf16)e;
           }
         }
@@ -726,7 +755,7 @@ hipError_t launch_split_forward(const SplitParams& p, int head_dim, hipStream_t 
     // each do not fit a wave; such plans are refused when they are checked)
     const bool shared = (p.num_q_heads / p.num_kv_heads) % kWaves == 0;
     if (!shared && D == 256) return hipErrorInvalidValue;
-    if (p.window > 0) {
+    if (p.window > 0 || p.drop_thr) {
       if (shared) {
         split_query_kernel<D, false, true, true><<<grid, kThreads, 0, stream>>>(p);
       } else if constexpr (D < 256) {
@@ -760,7 +789,7 @@ hipError_t launch_split_backward(const SplitParams& p, int head_dim, hipStream_t
     if (!shared && D == 256) return hipErrorInvalidValue;
     const int ratio = p.num_q_heads / p.num_kv_heads;
     const unsigned kgrid = (unsigned)((nt + kWaves - 1) / kWaves) * p.num_kv_heads * (p.head_split ? ratio : 1);
-    if (p.window > 0) {
+    if (p.window > 0 || p.drop_thr) {
       if (shared) {
         split_query_kernel<D, true, true, true><<<qgrid, kThreads, 0, stream>>>(p);
       } else if constexpr (D < 256) {

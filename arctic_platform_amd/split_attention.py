@@ -145,20 +145,46 @@ def _check_heads(q, k, v):
         raise ValueError(f"k and v must have one shape and the head size of q, got q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
 
 
-def _plan(q, k, layout):
-    return _lib.FcaSplitPlan(layout.num_tokens, q.shape[1], k.shape[1], q.shape[2], layout.window)
+def _plan(q, k, layout, dropout=0.0, seed=0):
+    dropout = float(dropout or 0.0)
+    if not 0.0 <= dropout < 1.0:
+        raise ValueError(f"attention dropout must lie in [0, 1), got {dropout}")
+    return _lib.FcaSplitPlan(layout.num_tokens, q.shape[1], k.shape[1], q.shape[2], layout.window, dropout, int(seed) & 0xFFFFFFFF)
 
 
-def split_attention_forward(q, k, v, layout: SplitLayout, scale: float, out=None):
+def dropout_keep_mask(seed: int, dropout: float, num_q_heads: int, num_tokens: int) -> torch.Tensor:
+    """The mask the kernels apply for ``dropout`` and ``seed``: bool ``[Hq, T, T]``, entry
+    (h, r, t) true when the probability of row r and key t (places in the deduplicated order)
+    survives in query head h.  The hash of include/zorro_fca.h restated on the host, for
+    callers that want to see or reproduce what a step dropped."""
+    thr = min(int(float(dropout) * 4294967296.0), 4294967295) if dropout > 0 else 0
+    if dropout > 0:
+        thr = max(thr, 1)
+    m = 0xFFFFFFFF
+    h = np.arange(num_q_heads, dtype=np.uint64)[:, None, None]
+    r = np.arange(num_tokens, dtype=np.uint64)[None, :, None]
+    t = np.arange(num_tokens, dtype=np.uint64)[None, None, :]
+    x = ((int(seed) & m) + h * 0xC2B2AE3D + r * 0x9E3779B1 + t * 0x85EBCA77) & m
+    x ^= x >> 16
+    x = (x * 0x7FEB352D) & m
+    x ^= x >> 15
+    x = (x * 0x846CA68B) & m
+    x ^= x >> 16
+    return torch.from_numpy(x >= thr)
+
+
+def split_attention_forward(q, k, v, layout: SplitLayout, scale: float, out=None, dropout: float = 0.0, seed: int = 0):
     """q ``[T, Hq, D]``, k, v ``[T, Hkv, D]`` bf16 in deduplicated order.  Returns
     ``(out [T, Hq, D] bf16, lse fp32 [Hq, 32 * ceil(T / 32)])``; ``lse[:, :T]`` is the
-    natural-log log-sum-exp of every row's scores.  ``out`` may be given to write into."""
+    natural-log log-sum-exp of every row's scores.  ``out`` may be given to write into.
+    ``dropout`` > 0 drops attention probabilities after the softmax (``seed`` decides which;
+    the backward needs the same two values)."""
     t, rows = layout.num_tokens, layout.num_query_rows
     _check_rows("q", q, rows)
     for name, x in (("k", k), ("v", v)):
         _check_rows(name, x, t)
     _check_heads(q, k, v)
-    plan = _plan(q, k, layout)
+    plan = _plan(q, k, layout, dropout, seed)
     if out is None:
         out = torch.empty((rows, q.shape[1], q.shape[2]), dtype=torch.bfloat16, device=q.device)
     else:
@@ -178,9 +204,9 @@ def split_attention_forward(q, k, v, layout: SplitLayout, scale: float, out=None
     return out, lse
 
 
-def split_attention_backward(dout, q, k, v, out, lse, layout: SplitLayout, scale: float):
+def split_attention_backward(dout, q, k, v, out, lse, layout: SplitLayout, scale: float, dropout: float = 0.0, seed: int = 0):
     """Gradients ``(dq, dk, dv)`` of ``split_attention_forward``'s ``out`` with respect to
-    its inputs, for the upstream gradient ``dout``."""
+    its inputs, for the upstream gradient ``dout`` (``dropout`` and ``seed`` as in the forward)."""
     if layout.responses_only:
         raise ValueError("a layout with responses_only serves the forward only")
     t = layout.num_tokens
@@ -189,7 +215,7 @@ def split_attention_backward(dout, q, k, v, out, lse, layout: SplitLayout, scale
     _check_heads(q, k, v)
     if out.shape != q.shape or dout.shape != q.shape:
         raise ValueError("out and dout must have the shape of q")
-    plan = _plan(q, k, layout)
+    plan = _plan(q, k, layout, dropout, seed)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     for name, x in (("dq", dq), ("dk", dk), ("dv", dv)):
         _check_rows(name, x, t)
@@ -208,10 +234,10 @@ def split_attention_backward(dout, q, k, v, out, lse, layout: SplitLayout, scale
 
 class _SplitAttention(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, layout, scale):
-        out, lse = split_attention_forward(q, k, v, layout, scale)
+    def forward(ctx, q, k, v, layout, scale, dropout=0.0, seed=0):
+        out, lse = split_attention_forward(q, k, v, layout, scale, dropout=dropout, seed=seed)
         ctx.save_for_backward(q, k, v, out, lse)
-        ctx.layout, ctx.scale = layout, scale
+        ctx.layout, ctx.scale, ctx.dropout, ctx.seed = layout, scale, dropout, seed
         return out
 
     @staticmethod
@@ -219,18 +245,16 @@ class _SplitAttention(torch.autograd.Function):
         q, k, v, out, lse = ctx.saved_tensors
         if dout.stride(2) != 1 or dout.stride(1) != dout.shape[2]:
             dout = dout.contiguous()
-        dq, dk, dv = split_attention_backward(dout, q, k, v, out, lse, ctx.layout, ctx.scale)
-        return dq, dk, dv, None, None
+        dq, dk, dv = split_attention_backward(dout, q, k, v, out, lse, ctx.layout, ctx.scale, ctx.dropout, ctx.seed)
+        return dq, dk, dv, None, None, None, None
 
 
 def _check_call_arguments(dropout, sliding_window, layout):
     """The trainer hands both to its attention calls on every step
     (qwen_attention_patcher.py:1204-1206, :1224-1226).  The window is a property of the layout
-    (its walks are cut to it), so the call's value must be the one the layout was made for.
-    Attention dropout is 0 outside training and in every recipe of the reference; the kernels
-    have none, and another value is refused rather than silently ignored."""
-    if dropout is not None and float(dropout) != 0.0:
-        raise NotImplementedError(f"attention dropout {dropout} is not supported by the split attention kernels (only 0.0)")
+    (its walks are cut to it), so the call's value must be the one the layout was made for."""
+    if dropout is not None and not 0.0 <= float(dropout) < 1.0:
+        raise ValueError(f"attention dropout must lie in [0, 1), got {dropout}")
     want = 0 if sliding_window is None else int(sliding_window)
     if want != layout.window:
         raise ValueError(
@@ -239,15 +263,21 @@ def _check_call_arguments(dropout, sliding_window, layout):
         )
 
 
-def split_attention(q, k, v, layout: SplitLayout, scale: float, dropout: float = 0.0, sliding_window=None):
+def split_attention(q, k, v, layout: SplitLayout, scale: float, dropout: float = 0.0, sliding_window=None, seed=None):
     """Differentiable split attention: ``out [T, Hq, D]`` in deduplicated order.  ``dropout``
-    and ``sliding_window`` are the arguments of the trainer's attention calls: dropout must be
-    0.0, the window the one ``layout`` was made for."""
+    and ``sliding_window`` are the arguments of the trainer's attention calls
+    (``0.0 if not module.training else module.attention_dropout``; the window must be the one
+    ``layout`` was made for).  With dropout, ``seed`` decides which probabilities fall (drawn
+    from torch's CPU generator when not given, so ``torch.manual_seed`` makes a run repeatable);
+    the backward reuses it."""
     _check_call_arguments(dropout, sliding_window, layout)
-    return _SplitAttention.apply(q, k, v, layout, scale)
+    dropout = float(dropout or 0.0)
+    if dropout > 0.0 and seed is None:
+        seed = int(torch.randint(0, 2**31 - 1, (1,)).item())
+    return _SplitAttention.apply(q, k, v, layout, scale, dropout, int(seed or 0))
 
 
-def split_attention_padded(q, k, v, valid, layout: SplitLayout, scale: float, dropout: float = 0.0, sliding_window=None):
+def split_attention_padded(q, k, v, valid, layout: SplitLayout, scale: float, dropout: float = 0.0, sliding_window=None, seed=None):
     """The same attention for a deduplicated batch that still carries its padding (the
     trainer's padded variant, qwen_attention_patcher.py:881-1040, which masks the padding inside
     its two attention calls): ``q``, ``k``, ``v`` are ``[T_padded, H, D]``, ``valid`` a bool
@@ -258,5 +288,5 @@ def split_attention_padded(q, k, v, valid, layout: SplitLayout, scale: float, dr
     index = torch.nonzero(valid, as_tuple=False).squeeze(-1)
     if index.numel() != layout.num_tokens:
         raise ValueError(f"{index.numel()} valid tokens, the layout counts {layout.num_tokens}")
-    out = split_attention(q.index_select(0, index), k.index_select(0, index), v.index_select(0, index), layout, scale, dropout, sliding_window)
+    out = split_attention(q.index_select(0, index), k.index_select(0, index), v.index_select(0, index), layout, scale, dropout, sliding_window, seed)
     return torch.zeros_like(q).index_copy(0, index, out)

@@ -302,14 +302,25 @@ int fca_gather_kv(void* key_dev, void* value_dev, int64_t token_stride, int64_t 
  * counted in the sample's own sequence (the prompt's tokens, then the response's), i.e.
  * key position > row position - window.  The layout must have been built for a window at
  * least as wide (or for none): its walks leave out the tiles no row sees any more.
- * Attention dropout, the other argument of those calls, has no counterpart here (it is 0
- * outside training and in every recipe of the reference). */
+ * dropout_p > 0 is the dropout both calls receive while training (:1204, :1224): after the
+ * softmax each probability is dropped with that probability and the others are scaled by
+ * 1 / (1 - dropout_p), as the attention interface does (dropout on the attention weights,
+ * then the product with V); the log-sum-exp is that of the undropped scores.  Which
+ * probabilities fall is a function of (dropout_seed, query head, row, key) alone:
+ *   x = seed + head * 0xC2B2AE3D + row * 0x9E3779B1 + key * 0x85EBCA77   (mod 2^32; row and
+ *       key are places in the deduplicated order)
+ *   x ^= x >> 16; x *= 0x7FEB352D; x ^= x >> 15; x *= 0x846CA68B; x ^= x >> 16;
+ *   dropped  <=>  x < floor(dropout_p * 2^32)
+ * so the forward and the three gradients agree without a stored mask, and a caller can
+ * reproduce it.  The backward must be given the plan (seed included) of its forward. */
 typedef struct fca_split_plan {
   int32_t num_tokens; /* T: tokens of the deduplicated batch */
   int32_t num_q_heads;
   int32_t num_kv_heads;
   int32_t head_dim; /* 64, 128 or 256 (256: num_q_heads / num_kv_heads a multiple of 4) */
   int32_t window;   /* 0 = none */
+  float dropout_p;  /* in [0, 1); 0 = none */
+  uint32_t dropout_seed;
 } fca_split_plan;
 
 /* int32 entries of the layout array of a batch of num_tokens tokens. */

@@ -56,10 +56,15 @@ def total_tokens(layout) -> int:
     return sum(int(p) + sum(int(n) for n in rs) for p, rs in layout)
 
 
-def _attend(q, k, v, scale, first_key_offset, window=None):
+def _attend(q, k, v, scale, first_key_offset, window=None, keep=None, dropout=0.0):
     """q [Lq, Hq, D], k/v [Lk, Hkv, D]; query i sees keys 0 .. first_key_offset + i
     (bottom-right aligned causal mask when first_key_offset = Lk - Lq), with ``window`` only
-    the last ``window`` of them.  Returns out and the natural-log log-sum-exp [Lq, Hq]."""
+    the last ``window`` of them.  ``keep`` (bool [Hq, Lq, Lk]) with ``dropout`` = p: the
+    probabilities where it is false are dropped and the others divided by 1 - p, after the
+    softmax and before the product with V, as the eager attention interface applies
+    ``nn.functional.dropout`` to the attention weights (transformers
+    models/qwen3/modeling_qwen3.py:173-207).  Returns out and the natural-log log-sum-exp
+    [Lq, Hq] (of the scores, untouched by dropout)."""
     lq, hq, _ = q.shape
     lk, hkv, _ = k.shape
     rep = hq // hkv
@@ -73,24 +78,33 @@ def _attend(q, k, v, scale, first_key_offset, window=None):
         s = s.masked_fill(keys <= rows + first_key_offset - int(window), -math.inf)
     lse = torch.logsumexp(s, dim=-1)
     p = torch.exp(s - lse[..., None])
+    if keep is not None:
+        p = p * keep.to(p.dtype) / (1.0 - dropout)
     return torch.einsum("hqk,khd->qhd", p, vv), lse.transpose(0, 1)
 
 
-def split_attention(q, k, v, layout, scale, dtype=torch.float64, window=None):
+def split_attention(q, k, v, layout, scale, dtype=torch.float64, window=None, keep=None, dropout=0.0):
     """q [T, Hq, D], k/v [T, Hkv, D] in deduplicated order.  Returns (out [T, Hq, D],
-    lse [T, Hq]) in ``dtype``.  Differentiable."""
+    lse [T, Hq]) in ``dtype``.  Differentiable.  ``keep``: bool [Hq, T, T] over places in the
+    deduplicated order (row, key), the dropout mask of attention dropout ``dropout``."""
     q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+
+    def sub(rows, keys):  # the mask of a call: its rows against its key sequence
+        return None if keep is None else keep[:, rows][:, :, keys]
+
     outs, lses = [], []
     prompt_of = {}
     for g, kind, start, n in segments(layout):
         if kind == "p":
             prompt_of[g] = (start, n)
-            o, l = _attend(q[start : start + n], k[start : start + n], v[start : start + n], scale, 0, window)
+            own = torch.arange(start, start + n)
+            o, l = _attend(q[start : start + n], k[start : start + n], v[start : start + n], scale, 0, window, sub(own, own), dropout)
         else:
             ps, pn = prompt_of[g]
             kk = torch.cat([k[ps : ps + pn], k[start : start + n]])
             vv = torch.cat([v[ps : ps + pn], v[start : start + n]])
-            o, l = _attend(q[start : start + n], kk, vv, scale, pn, window)
+            own = torch.arange(start, start + n)
+            o, l = _attend(q[start : start + n], kk, vv, scale, pn, window, sub(own, torch.cat([torch.arange(ps, ps + pn), own])), dropout)
         outs.append(o)
         lses.append(l)
     return torch.cat(outs), torch.cat(lses)

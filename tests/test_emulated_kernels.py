@@ -642,11 +642,10 @@ def test_split_attention_forward_and_backward(emu, heads, late):
     _split_cases(emu, heads, late, None)
 
 
-@pytest.mark.parametrize("late", [False, True], ids=["loads-land-at-once", "loads-land-at-their-wait"])
 @pytest.mark.parametrize(
-    "heads,window",
-    [((8, 2, 128), 1), ((8, 2, 128), 45), ((8, 2, 128), 200), ((6, 2, 64), 7), ((6, 2, 64), 32), ((4, 1, 256), 45)],
-    ids=lambda x: "Hq%d-Hkv%d-D%d" % x if isinstance(x, tuple) else f"w{x}",
+    "heads,window,late",
+    [((8, 2, 128), 1, False), ((8, 2, 128), 45, True), ((8, 2, 128), 200, False), ((6, 2, 64), 7, True), ((6, 2, 64), 32, False), ((4, 1, 256), 45, True)],
+    ids=lambda x: "Hq%d-Hkv%d-D%d" % x if isinstance(x, tuple) else f"{x}",
 )
 def test_split_attention_with_a_sliding_window(emu, heads, window, late):
     """The instances for a sliding window: a row sees the last ``window`` positions of its own
@@ -655,8 +654,19 @@ def test_split_attention_with_a_sliding_window(emu, heads, window, late):
     _split_cases(emu, heads, late, window)
 
 
-def _split_cases(emu, heads, late, window):
-    from arctic_platform_amd.split_attention import SplitLayout
+@pytest.mark.parametrize(
+    "heads,window,dropout,late",
+    [((8, 2, 128), None, 0.1, True), ((6, 2, 64), None, 0.5, False), ((8, 2, 128), 45, 0.25, False), ((4, 1, 256), None, 0.3, True)],
+    ids=lambda x: "Hq%d-Hkv%d-D%d" % x if isinstance(x, tuple) else f"{x}",
+)
+def test_split_attention_with_attention_dropout(emu, heads, window, dropout, late):
+    """Attention dropout in the general instances: the four kernels draw the fate of a probability
+    from the same hash of (seed, query head, row, key), which the host restates for the oracle."""
+    _split_cases(emu, heads, late, window, dropout)
+
+
+def _split_cases(emu, heads, late, window, dropout=0.0):
+    from arctic_platform_amd.split_attention import SplitLayout, dropout_keep_mask
 
     hq, hkv, d = heads
     emu.emu_set_dma_late(1 if late else 0)
@@ -669,7 +679,8 @@ def _split_cases(emu, heads, late, window):
         scale = d**-0.5
         lay = guarded(torch.from_numpy(SplitLayout(layout, device="cpu", sliding_window=window).host))
         nt = (t + 31) // 32
-        plan = _lib.FcaSplitPlan(t, hq, hkv, d, window or 0)
+        plan = _lib.FcaSplitPlan(t, hq, hkv, d, window or 0, dropout, 4000 + ci)
+        keep = dropout_keep_mask(4000 + ci, dropout, hq, t) if dropout > 0 else None
         fwd, bwd = ctypes.c_size_t(), ctypes.c_size_t()
         _ok(emu, emu.fca_split_workspace_bytes(ctypes.byref(plan), ctypes.byref(fwd), ctypes.byref(bwd)))
         ws_f, ws_b = guarded(torch.zeros(fwd.value, dtype=torch.uint8)), guarded(torch.zeros(bwd.value, dtype=torch.uint8))
@@ -683,7 +694,7 @@ def _split_cases(emu, heads, late, window):
             ),
         )
         q64, k64, v64 = (x.double().requires_grad_() for x in (q, k, v))
-        ro, rl = oracle_split(q64, k64, v64, layout, scale, window=window)
+        ro, rl = oracle_split(q64, k64, v64, layout, scale, window=window, keep=keep, dropout=dropout)
         _close("out", out, ro, 2e-2 / max(1.0, float(ro.detach().abs().max())))
         torch.testing.assert_close(lse[:, :t].T.double(), rl.detach(), rtol=1e-3, atol=1e-3)
         dout = guarded(torch.randn(t, hq, d, generator=torch.Generator().manual_seed(ci + 1)).bfloat16())

@@ -37,7 +37,9 @@ def _functions(asm):
 
 
 def test_attention_kernels_use_no_scratch(hipcc, tmp_path):
-    for src, count in (("fca_attend32.hip", 8), ("fca_attend.hip", 12)):
+    # (the fp32 kernel keeps 32 rows of running maxima, sums and accumulators in registers,
+    # and the merge its partial rows: in scratch they would be memory traffic per token)
+    for src, count in (("fca_attend32.hip", 8), ("fca_attend.hip", 12), ("fca_attend_f32.hip", 2), ("fca_merge.hip", 11)):
         res = subprocess.run(
             [hipcc, *FLAGS, "-c", "-Rpass-analysis=kernel-resource-usage", os.path.join(CSRC, src), "-o", str(tmp_path / "o.o")],
             capture_output=True, text=True, cwd=CSRC,

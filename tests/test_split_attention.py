@@ -13,6 +13,7 @@ import torch
 from arctic_platform_amd import _lib
 from arctic_platform_amd.split_attention import (
     SplitLayout,
+    dropout_keep_mask,
     split_attention,
     split_attention_padded,
     split_attention_backward,
@@ -145,6 +146,47 @@ def test_oracle_with_a_sliding_window(window):
         assert torch.equal(vis, visible(layout))
 
 
+def test_oracle_with_attention_dropout():
+    """Dropout on the attention weights (after the softmax, before the product with V), the
+    way the eager interface the reference resolves applies it.  Pinned by what needs no
+    second implementation: nothing dropped = no dropout at all; a constant V gives back the
+    surviving probability mass over 1 - p; over many seeds the mean output tends to the
+    undropped one; the log-sum-exp does not move; and the mask itself drops a share p,
+    with no visible tie between neighbouring heads, rows or keys."""
+    layout = LAYOUTS[0]
+    hq, t = 4, total_tokens(layout)
+    q, k, v = _inputs(layout, hq, 2, 8, 17)
+    plain_out, plain_lse = oracle_split(q, k, v, layout, 0.3)
+    everything = torch.ones(hq, t, t, dtype=torch.bool)
+    out, lse = oracle_split(q, k, v, layout, 0.3, keep=everything, dropout=0.0)
+    assert torch.equal(out, plain_out) and torch.equal(lse, plain_lse)
+    p = 0.25
+    keep = dropout_keep_mask(99, p, hq, t)
+    vc = torch.ones_like(v) * 0.5
+    out, lse = oracle_split(q, k, vc, layout, 0.3, keep=keep, dropout=p)
+    assert torch.equal(lse, plain_lse)
+    vis = visible(layout)
+    s = (torch.einsum("qhd,khd->hqk", q, k.repeat_interleave(2, 1)) * 0.3).masked_fill(~vis[None], -math.inf)
+    mass = (torch.softmax(s, -1) * keep).sum(-1) / (1 - p)  # [Hq, T]
+    torch.testing.assert_close(out, 0.5 * mass.T[:, :, None].expand(-1, -1, 8), rtol=1e-12, atol=1e-12)
+    mean = torch.zeros_like(plain_out)
+    seeds = 400
+    for seed in range(seeds):
+        mean += oracle_split(q, k, v, layout, 0.3, keep=dropout_keep_mask(seed, p, hq, t), dropout=p)[0]
+    # a row that sees n keys has variance ~ p / (1 - p) * sum(prob^2 v^2) per seed
+    assert float((mean / seeds - plain_out).abs().max()) < 0.25
+    assert float((mean / seeds - plain_out).abs().mean()) < 0.03
+    # the mask: share dropped, and no tie between neighbours along any of its three axes
+    big = dropout_keep_mask(7, p, 8, 300).float()
+    assert abs(float(big.mean()) - (1 - p)) < 3 * math.sqrt(p * (1 - p) / big.numel()) + 1e-4
+    centred = big - big.mean()
+    for a, b in ((centred[1:], centred[:-1]), (centred[:, 1:], centred[:, :-1]), (centred[:, :, 1:], centred[:, :, :-1])):
+        corr = float((a * b).mean() / centred.var())
+        assert abs(corr) < 0.01, corr
+    assert not torch.equal(dropout_keep_mask(7, p, 2, 64), dropout_keep_mask(8, p, 2, 64))
+    assert bool(dropout_keep_mask(7, 0.0, 2, 64).all())
+
+
 # ---- the layout array (host code of the library) -------------------------------------------------
 @pytest.mark.parametrize("window", [None, 1, 9, 32, 50, 200])
 def test_layout_array_against_brute_force(window):
@@ -242,17 +284,19 @@ def test_layout_for_response_rows_only():
     assert (full.kv_lim() == L.kv_lim()).all()
 
 
-def test_dropout_is_refused_and_the_window_must_be_the_layouts():
-    """The trainer passes both on every call (qwen_attention_patcher.py:1204-1206).  Dropout
-    other than 0 raises before a tensor is looked at; so does a window that is not the one the
-    layout was made for (its walks are cut to it)."""
+def test_dropout_range_and_the_window_must_be_the_layouts():
+    """The trainer passes both on every call (qwen_attention_patcher.py:1204-1206).  A dropout
+    outside [0, 1) raises before a tensor is looked at; so does a window that is not the one
+    the layout was made for (its walks are cut to it)."""
     from arctic_platform_amd.split_attention import split_attention, split_attention_padded
 
     plain = SplitLayout([(4, [3])], device="cpu")
     windowed = SplitLayout([(4, [3])], device="cpu", sliding_window=128)
     for fn, args in ((split_attention, (None, None, None)), (split_attention_padded, (None, None, None, None))):
-        with pytest.raises(NotImplementedError, match="dropout"):
-            fn(*args, plain, 1.0, dropout=0.1)
+        with pytest.raises(ValueError, match="dropout"):
+            fn(*args, plain, 1.0, dropout=1.0)
+        with pytest.raises(ValueError, match="dropout"):
+            fn(*args, plain, 1.0, dropout=-0.1)
         with pytest.raises(ValueError, match="sliding_window"):
             fn(*args, plain, 1.0, sliding_window=4096)
         with pytest.raises(ValueError, match="sliding_window"):
@@ -320,7 +364,7 @@ def _close(name, got, ref, scale_tol):
     assert bool((err <= bound).all()), f"{name}: max |err| {err.max():.4g}, largest reference {ref.abs().max():.4g}"
 
 
-def _run_case(layout, hq, hkv, d, seed, strided=False, q_gain=1.0, window=None):
+def _run_case(layout, hq, hkv, d, seed, strided=False, q_gain=1.0, window=None, dropout=0.0):
     q, k, v = _inputs(layout, hq, hkv, d, seed, torch.bfloat16)
     q = (q.float() * q_gain).bfloat16()
     t = q.shape[0]
@@ -335,14 +379,15 @@ def _run_case(layout, hq, hkv, d, seed, strided=False, q_gain=1.0, window=None):
         assert t == 1 or qd.stride(0) == (hq + 2 * hkv) * d
     else:
         qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
-    out, lse = split_attention_forward(qd, kd, vd, L, scale)
+    out, lse = split_attention_forward(qd, kd, vd, L, scale, dropout=dropout, seed=seed + 5)
     q64, k64, v64 = (x.double().requires_grad_() for x in (q, k, v))
-    ro, rl = oracle_split(q64, k64, v64, layout, scale, window=window)
+    keep = dropout_keep_mask(seed + 5, dropout, hq, t) if dropout > 0 else None
+    ro, rl = oracle_split(q64, k64, v64, layout, scale, window=window, keep=keep, dropout=dropout)
     _close("out", out, ro, 2e-2 / max(1.0, float(ro.detach().abs().max())))
     torch.testing.assert_close(lse[:, :t].T.cpu().double(), rl.detach(), rtol=1e-3, atol=1e-3)
     dout = torch.randn(t, hq, d, generator=torch.Generator().manual_seed(seed + 1)).bfloat16()
     ro.backward(dout.double())
-    dq, dk, dv = split_attention_backward(dout.cuda(), qd, kd, vd, out, lse, L, scale)
+    dq, dk, dv = split_attention_backward(dout.cuda(), qd, kd, vd, out, lse, L, scale, dropout=dropout, seed=seed + 5)
     _close("dq", dq, q64.grad, 1e-2)
     _close("dk", dk, k64.grad, 1e-2)
     _close("dv", dv, v64.grad, 1e-2)
@@ -364,6 +409,45 @@ def test_sliding_window_matches_the_oracle(heads, window):
     their operands through LDS and the per-wave ones."""
     for layout in LAYOUTS:
         _run_case(layout, *heads, seed=51, window=window)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dropout,window", [(0.1, None), (0.5, None), (0.25, 40)])
+@pytest.mark.parametrize("heads", [(8, 2, 128), (6, 2, 64), (4, 4, 128)])
+def test_attention_dropout_matches_the_oracle(heads, dropout, window):
+    """Attention dropout (the trainer's calls pass module.attention_dropout while training,
+    qwen_attention_patcher.py:1204, :1224): forward and the three gradients against the oracle
+    under the same mask, which the host restates from the seed; alone and with a window."""
+    for layout in LAYOUTS:
+        _run_case(layout, *heads, seed=71, window=window, dropout=dropout)
+
+
+@pytest.mark.gpu
+def test_attention_dropout_through_autograd_repeats_under_a_seed():
+    layout = [(70, [40, 33]), (20, [50])]
+    hq, hkv, d = 8, 2, 128
+    q, k, v = (x.cuda().requires_grad_() for x in _inputs(layout, hq, hkv, d, 81, torch.bfloat16))
+    L = SplitLayout(layout)
+    torch.manual_seed(5)
+    a = split_attention(q, k, v, L, d**-0.5, dropout=0.2)
+    torch.manual_seed(5)
+    b = split_attention(q, k, v, L, d**-0.5, dropout=0.2)
+    c = split_attention(q, k, v, L, d**-0.5, dropout=0.2)
+    assert torch.equal(a, b) and not torch.equal(a, c)
+    a.float().sum().backward()
+    assert all(bool(torch.isfinite(x.grad.float()).all()) for x in (q, k, v))
+    # the forward's seed reaches the backward: an explicit seed against the oracle
+    q.grad = k.grad = v.grad = None
+    out = split_attention(q, k, v, L, d**-0.5, dropout=0.2, seed=1234)
+    w = torch.randn(out.shape, generator=torch.Generator().manual_seed(82)).bfloat16()
+    (out.float() * w.cuda().float()).sum().backward()
+    q64, k64, v64 = (x.detach().cpu().double().requires_grad_() for x in (q, k, v))
+    keep = dropout_keep_mask(1234, 0.2, hq, total_tokens(layout))
+    ro, _ = oracle_split(q64, k64, v64, layout, d**-0.5, keep=keep, dropout=0.2)
+    (ro * w.double()).sum().backward()
+    _close("out", out, ro, 2e-2 / max(1.0, float(ro.detach().abs().max())))
+    for name, got, ref in (("dq", q.grad, q64.grad), ("dk", k.grad, k64.grad), ("dv", v.grad, v64.grad)):
+        _close(name, got, ref, 1e-2)
 
 
 @pytest.mark.gpu
