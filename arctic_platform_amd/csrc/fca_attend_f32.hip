@@ -36,14 +36,19 @@ __device__ inline float wave_sum(float v) {
 
 constexpr int kStepTokens = 64;  // tokens per step: one per lane
 constexpr int kMaxRows = 32;     // query rows of an item (rows_per_item = 32)
+// Two waves to a workgroup, two workgroups to a CU: every wave still has a SIMD and its whole
+// register file to itself, and a workgroup's LDS (the query rows and the probabilities of its
+// waves: 48 KB at head size 128) stays below 64 KB.
+constexpr int kF32Waves = 2;
+constexpr int kF32Threads = 64 * kF32Waves;
 
 }  // namespace
 
 template <int D>
-__global__ __launch_bounds__(kThreads, 1) void fca_attend_f32_kernel(AttendParams p) {
+__global__ __launch_bounds__(kF32Threads, 1) void fca_attend_f32_kernel(AttendParams p) {
   constexpr int CPL = D / 64;  // channels per lane in the value product
-  __shared__ __attribute__((aligned(16))) float q_lds[kWaves][kMaxRows][D];
-  __shared__ __attribute__((aligned(16))) float p_lds[kWaves][kMaxRows][kStepTokens];
+  __shared__ __attribute__((aligned(16))) float q_lds[kF32Waves][kMaxRows][D];
+  __shared__ __attribute__((aligned(16))) float p_lds[kF32Waves][kMaxRows][kStepTokens];
 
   const int32_t* hdr = p.meta + p.off_header;
   const int total = hdr[H_ITEMS], shared = hdr[H_SHARED_ITEMS];
@@ -53,14 +58,14 @@ __global__ __launch_bounds__(kThreads, 1) void fca_attend_f32_kernel(AttendParam
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int G = p.group, Hkv = p.num_kv_heads;
-  const int nwaves = (int)gridDim.x * kWaves;
+  const int nwaves = (int)gridDim.x * kF32Waves;
   const float* qbase = static_cast<const float*>(p.q);
   float* pout = static_cast<float*>(p.partial_out);
   const float sc = p.scale * kLog2e;
   float(*qw)[D] = q_lds[wave];
   float(*pw)[kStepTokens] = p_lds[wave];
 
-  for (int t = (int)blockIdx.x * kWaves + wave; t < ntickets; t += nwaves) {
+  for (int t = (int)blockIdx.x * kF32Waves + wave; t < ntickets; t += nwaves) {
     const int it = t / Hkv, kvh = t - it * Hkv;
     const int32_t* rec = p.meta + p.off_items + (int64_t)(first + it) * kItemInts;
     const int rep = __builtin_amdgcn_readfirstlane(rec[0]);
@@ -196,13 +201,14 @@ hipError_t launch_attend_f32(const AttendParams& p, const fca_plan& plan, int ma
     int cus = 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0) grid = cus;
   }
+  grid *= 2;  // two workgroups of two waves per CU
   if (max_workgroups > 0 && max_workgroups < grid) grid = max_workgroups;
-  if ((int64_t)grid * kWaves > max_tickets) grid = (int)((max_tickets + kWaves - 1) / kWaves);
+  if ((int64_t)grid * kF32Waves > max_tickets) grid = (int)((max_tickets + kF32Waves - 1) / kF32Waves);
   if (grid < 1) grid = 1;
   if (plan.head_dim == 128) {
-    fca_attend_f32_kernel<128><<<dim3(grid), kThreads, 0, stream>>>(p);
+    fca_attend_f32_kernel<128><<<dim3(grid), kF32Threads, 0, stream>>>(p);
   } else if (plan.head_dim == 64) {
-    fca_attend_f32_kernel<64><<<dim3(grid), kThreads, 0, stream>>>(p);
+    fca_attend_f32_kernel<64><<<dim3(grid), kF32Threads, 0, stream>>>(p);
   } else {
     return hipErrorInvalidValue;
   }

@@ -97,8 +97,9 @@ typedef struct fca_tensors {
   int32_t reproducible;        /* non-zero: no work item is attended by two waves together, so where an
                                   item is cut, and with it the last bit of a few outputs, never depends
                                   on timing: two launches on the same inputs give the same bits */
-  int32_t max_workgroups;      /* > 0: the attention launch uses at most this many workgroups (of four
-                                  waves), leaving the rest of the GPU to work on other streams; 0: all */
+  int32_t max_workgroups;      /* > 0: the attention launch uses at most this many workgroups (four waves
+                                  each; two in the fp32 path), leaving the rest of the GPU to work on
+                                  other streams; 0: all */
 } fca_tensors;
 
 /* Offsets (in int32 units) of the arrays inside a built metadata workspace, for
