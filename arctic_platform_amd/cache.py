@@ -24,19 +24,23 @@ def gather_kv(kv_cache, slot_mapping, head_dim, k_scale=None, v_scale=None, out=
     hkv = kv_cache.shape[2]
     t = slot_mapping.shape[0]
     if out is None:
-        out = tuple(torch.empty(t, hkv, head_dim, dtype=torch.bfloat16, device=kv_cache.device) for _ in range(2))
+        rows_dtype = torch.float32 if kv_cache.dtype == torch.float32 else torch.bfloat16
+        out = tuple(torch.empty(t, hkv, head_dim, dtype=rows_dtype, device=kv_cache.device) for _ in range(2))
     _cache_rows(True, out[0], out[1], kv_cache, slot_mapping, k_scale, v_scale)
     return out
 
 
 def append_kv(key, value, kv_cache, slot_mapping, k_scale=None, v_scale=None) -> None:
-    """key, value: bf16 ``[T, Hkv, D]``; slot_mapping: int64 ``[T]``; kv_cache as in kv_layout."""
+    """key, value: bf16 ``[T, Hkv, D]`` (float32 for a float32 cache); slot_mapping: int64 ``[T]``;
+    kv_cache as in kv_layout."""
     _cache_rows(False, key, value, kv_cache, slot_mapping, k_scale, v_scale)
 
 
 def _cache_rows(gather, key, value, kv_cache, slot_mapping, k_scale, v_scale) -> None:
-    if key.dtype != torch.bfloat16 or value.dtype != torch.bfloat16 or key.shape != value.shape or key.dim() != 3:
-        raise TypeError("key and value must be bfloat16 tensors of the same shape [tokens, kv_heads, head_dim]")
+    f32 = kv_cache.dtype == torch.float32
+    rows_dtype = torch.float32 if f32 else torch.bfloat16
+    if key.dtype != rows_dtype or value.dtype != rows_dtype or key.shape != value.shape or key.dim() != 3:
+        raise TypeError(f"key and value must be {rows_dtype} tensors of the same shape [tokens, kv_heads, head_dim] for a {kv_cache.dtype} cache")
     if key.stride() != value.stride() or key.stride(2) != 1:
         raise ValueError("key and value must share strides and have a contiguous head_dim")
     t, hkv, d = key.shape
@@ -54,6 +58,8 @@ def _cache_rows(gather, key, value, kv_cache, slot_mapping, k_scale, v_scale) ->
         code = _lib.FCA_BF16
     elif kv_cache.dtype == torch.float8_e4m3fn:
         code = _lib.FCA_FP8_E4M3
+    elif f32:
+        code = _lib.FCA_F32  # the all-fp32 path: fp32 rows, fp32 cache
     else:
         raise TypeError(f"unsupported KV cache dtype {kv_cache.dtype}")
     if not (key.is_cuda and kv_cache.is_cuda and slot_mapping.is_cuda):

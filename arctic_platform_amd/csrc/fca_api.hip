@@ -375,12 +375,12 @@ static int cache_rows(bool gather, const void* key_dev, const void* value_dev, i
   if (num_tokens < 0 || num_kv_heads < 1) return fail(FCA_ERR_INVALID_ARG, "num_tokens must be >= 0 and num_kv_heads >= 1");
   if (head_dim != 64 && head_dim != 128 && head_dim != 256)
     return fail(FCA_ERR_UNSUPPORTED, "head_dim %d is not supported (64, 128 or 256)", head_dim);
-  if (kv_dtype != FCA_BF16 && kv_dtype != FCA_FP8_E4M3)
-    return fail(FCA_ERR_UNSUPPORTED, "kv_dtype %d is not supported (bf16 or fp8 e4m3)", kv_dtype);
+  if (kv_dtype != FCA_BF16 && kv_dtype != FCA_FP8_E4M3 && kv_dtype != FCA_F32)
+    return fail(FCA_ERR_UNSUPPORTED, "kv_dtype %d is not supported (bf16, fp8 e4m3, or fp32 with fp32 rows)", kv_dtype);
   if (num_tokens == 0) return FCA_OK;
   if (!key_dev || !value_dev || !slot_mapping_dev || !k_cache_dev || !v_cache_dev)
     return fail(FCA_ERR_INVALID_ARG, "key, value, slot_mapping and the cache planes must be non-NULL");
-  const int esz = kv_dtype == FCA_FP8_E4M3 ? 1 : 2;
+  const int esz = kv_elem_bytes(kv_dtype);
   if ((reinterpret_cast<uintptr_t>(key_dev) & 15) || (reinterpret_cast<uintptr_t>(value_dev) & 15) || token_stride % 8 ||
       head_stride % 8)
     return fail(FCA_ERR_INVALID_ARG, "key and value must be 16-byte aligned with strides that are multiples of 8 elements");

@@ -205,9 +205,56 @@ __global__ __launch_bounds__(256) void fca_gather_kernel(AppendParams p) {
   }
 }
 
+// fp32 rows and an fp32 cache (the all-fp32 path): one thread per (token, KV head, four
+// channels).  The K tile keeps four channels of a token together ([D / 4][16 tokens][4]), so
+// that side is one 16-byte access; the V tile ([D][16 tokens]) takes one element per channel.
+// A small-configuration path: no staging through LDS.
+template <bool GATHER>
+__global__ __launch_bounds__(256) void fca_cache_f32_kernel(AppendParams p) {
+  const int groups = p.head_dim / 4;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)p.num_tokens * p.num_kv_heads * groups) return;
+  const int g = (int)(idx % groups);
+  const int h = (int)(idx / groups % p.num_kv_heads);
+  const int64_t t = idx / groups / p.num_kv_heads;
+  const int64_t slot = p.slot_mapping[t];
+  const int64_t row = t * p.token_stride + (int64_t)h * p.head_stride + 4 * g;
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  f4* krow = reinterpret_cast<f4*>(reinterpret_cast<float*>(const_cast<void*>(p.key)) + row);
+  f4* vrow = reinterpret_cast<f4*>(reinterpret_cast<float*>(const_cast<void*>(p.value)) + row);
+  if (slot < 0) {  // padding: nothing to write; the way back gives zeros
+    if (GATHER) *krow = f4{0.f, 0.f, 0.f, 0.f}, *vrow = f4{0.f, 0.f, 0.f, 0.f};
+    return;
+  }
+  const int64_t blk = slot / kBlock;
+  const int off = (int)(slot - blk * kBlock);
+  const int64_t tile = blk * p.cache_block_stride + (int64_t)h * p.cache_head_stride;  // elements
+  f4* kc = reinterpret_cast<f4*>(reinterpret_cast<float*>(p.k_cache) + tile + ((int64_t)g * kBlock + off) * 4);
+  float* vc = reinterpret_cast<float*>(p.v_cache) + tile + (int64_t)(4 * g) * kBlock + off;
+  if (GATHER) {
+    *krow = *kc;
+    *vrow = f4{vc[0], vc[kBlock], vc[2 * kBlock], vc[3 * kBlock]};
+  } else {
+    *kc = *krow;
+    const f4 v = *vrow;
+    vc[0] = v[0], vc[kBlock] = v[1], vc[2 * kBlock] = v[2], vc[3 * kBlock] = v[3];
+  }
+}
+
+static hipError_t launch_cache_f32(const AppendParams& p, bool gather, hipStream_t stream) {
+  const int64_t threads = (int64_t)p.num_tokens * p.num_kv_heads * (p.head_dim / 4);
+  const unsigned grid = (unsigned)((threads + 255) / 256);
+  if (gather)
+    hipLaunchKernelGGL(fca_cache_f32_kernel<true>, dim3(grid), dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL(fca_cache_f32_kernel<false>, dim3(grid), dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+
 hipError_t launch_gather(const AppendParams& p, int kv_dtype, hipStream_t stream) {
   const bool fp8 = kv_dtype == FCA_FP8_E4M3;
   if (p.num_tokens == 0) return hipSuccess;
+  if (kv_dtype == FCA_F32) return launch_cache_f32(p, true, stream);
   const int grid = (p.num_tokens + kGroup - 1) / kGroup * p.num_kv_heads;
   if (fp8)
     hipLaunchKernelGGL(fca_gather_kernel<true>, dim3(grid), dim3(256), 0, stream, p);
@@ -219,6 +266,7 @@ hipError_t launch_gather(const AppendParams& p, int kv_dtype, hipStream_t stream
 hipError_t launch_append(const AppendParams& p, int kv_dtype, hipStream_t stream) {
   const bool fp8 = kv_dtype == FCA_FP8_E4M3;
   if (p.num_tokens == 0) return hipSuccess;
+  if (kv_dtype == FCA_F32) return launch_cache_f32(p, false, stream);
   const int grid = (p.num_tokens + kGroup - 1) / kGroup * p.num_kv_heads;
   if (fp8)
     hipLaunchKernelGGL(fca_append_kernel<true>, dim3(grid), dim3(256), 0, stream, p);

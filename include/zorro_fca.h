@@ -54,8 +54,8 @@ typedef enum fca_status {
  * chip has no more fp32 rate in its matrix cores), at the precision of the reference's
  * softmax-in-fp32 attention (arctic_platform/rl/zorro_train/qwen_attention_patcher.py:55-61).
  * It runs through fca_decode_step and fca_decode_step_static only, at head sizes 64 and 128
- * with rows_per_item 32; the other entry points that take tensors refuse it, and the cache
- * writer has no fp32 instance. */
+ * with rows_per_item 32; the separate passes and the merge refuse it.  fca_append_kv and
+ * fca_gather_kv with kv_dtype FCA_F32 move fp32 rows to and from an fp32 cache. */
 typedef enum fca_dtype {
   FCA_BF16 = 0,     /* q, out, KV cache */
   FCA_FP8_E4M3 = 1, /* KV cache only (OCP e4m3fn) */
@@ -269,7 +269,7 @@ int fca_decode_step_static(const fca_plan* plan, const fca_tensors* t, void* met
                            void* stream);
 
 /* KV-cache append, the step before decode attention in every layer: scatter the new
- * tokens' K and V (bf16 [T, Hkv, D]) into the cache tiles at slot = block * 16 + offset
+ * tokens' K and V (bf16 [T, Hkv, D]; fp32 when kv_dtype is FCA_F32) into the cache tiles at slot = block * 16 + offset
  * (negative slot = padding, skipped), quantising to fp8 e4m3 with per-KV-head scales
  * (stored = clamp(x / scale, +-448) rounded to nearest even) when kv_dtype says so.
  * Replaces the external engine's cache-write op on this layout; in-tree the reference only

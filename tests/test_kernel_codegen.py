@@ -39,14 +39,19 @@ def _functions(asm):
 def test_attention_kernels_use_no_scratch(hipcc, tmp_path):
     # (the fp32 kernel keeps 32 rows of running maxima, sums and accumulators in registers,
     # and the merge its partial rows: in scratch they would be memory traffic per token)
-    for src, count in (("fca_attend32.hip", 8), ("fca_attend.hip", 12), ("fca_attend_f32.hip", 2), ("fca_merge.hip", 11)):
-        res = subprocess.run(
-            [hipcc, *FLAGS, "-c", "-Rpass-analysis=kernel-resource-usage", os.path.join(CSRC, src), "-o", str(tmp_path / "o.o")],
-            capture_output=True, text=True, cwd=CSRC,
+    sources = (("fca_attend32.hip", 8), ("fca_attend.hip", 12), ("fca_attend_f32.hip", 2), ("fca_merge.hip", 11))
+    jobs = [
+        subprocess.Popen(
+            [hipcc, *FLAGS, "-c", "-Rpass-analysis=kernel-resource-usage", os.path.join(CSRC, src), "-o", str(tmp_path / (src + ".o"))],
+            stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, cwd=CSRC,
         )
-        assert res.returncode == 0, res.stderr[-2000:]
-        names = re.findall(r"Function Name: (\S+)", res.stderr)
-        sizes = [int(n) for n in re.findall(r"ScratchSize \[bytes/lane\]: (\d+)", res.stderr)]
+        for src, _ in sources
+    ]
+    for (src, count), job in zip(sources, jobs):
+        _, stderr = job.communicate()
+        assert job.returncode == 0, stderr[-2000:]
+        names = re.findall(r"Function Name: (\S+)", stderr)
+        sizes = [int(n) for n in re.findall(r"ScratchSize \[bytes/lane\]: (\d+)", stderr)]
         assert len(names) == len(sizes) == count, (src, names)
         for name, size in zip(names, sizes):
             if "ILi256E" in name:

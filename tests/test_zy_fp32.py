@@ -92,6 +92,31 @@ def test_random_forests_in_fp32(gpu, seed, hq, hkv, d, depth, fanout, shared, le
     assert torch.equal(out2, out) and torch.equal(lse2, lse)
 
 
+def test_fp32_cache_writer_and_reader(gpu):
+    """fp32 rows into an fp32 cache and back (bit-exact against the CPU restatement's plain loops),
+    and a decode step over what was written."""
+    from arctic_platform_amd.cache import append_kv, gather_kv
+    from arctic_platform_amd.kv_layout import kv_cache_shape
+    from oracle.cache import append_kv_reference
+
+    gen = torch.Generator().manual_seed(3)
+    hkv, d, nblocks = 2, 64, 9
+    slots = list(range(21, 75)) + [3, 130, -1, 100]
+    key = torch.randn(len(slots), hkv, d, generator=gen)
+    value = torch.randn(len(slots), hkv, d, generator=gen)
+    slot_mapping = torch.tensor(slots, dtype=torch.int64)
+    cache = torch.zeros(kv_cache_shape(nblocks, 16, hkv, d), dtype=torch.float32, device=gpu)
+    append_kv(key.to(gpu), value.to(gpu), cache, slot_mapping.to(gpu))
+    want = append_kv_reference(torch.zeros(kv_cache_shape(nblocks, 16, hkv, d)), key, value, slot_mapping)
+    assert torch.equal(cache.cpu(), want)
+    back_k, back_v = gather_kv(cache, slot_mapping.to(gpu), d)
+    live = torch.tensor([s >= 0 for s in slots])
+    assert back_k.dtype == torch.float32 and torch.equal(back_k.cpu()[live], key[live]) and torch.equal(back_v.cpu()[live], value[live])
+    assert not back_k.cpu()[~live].any() and not back_v.cpu()[~live].any()
+    with pytest.raises(TypeError, match="float32"):
+        append_kv(key.to(gpu).bfloat16(), value.to(gpu).bfloat16(), cache, slot_mapping.to(gpu))
+
+
 def test_fp32_tensors_are_refused_where_there_is_no_fp32_path(gpu):
     from arctic_platform_amd import ops
     from arctic_platform_amd.forest import build_forest_metadata
