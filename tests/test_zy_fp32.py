@@ -93,8 +93,7 @@ def test_random_forests_in_fp32(gpu, seed, hq, hkv, d, depth, fanout, shared, le
 
 
 def test_fp32_cache_writer_and_reader(gpu):
-    """fp32 rows into an fp32 cache and back (bit-exact against the CPU restatement's plain loops),
-    and a decode step over what was written."""
+    """fp32 rows into an fp32 cache and back, bit-exact against the CPU restatement's plain loops."""
     from arctic_platform_amd.cache import append_kv, gather_kv
     from arctic_platform_amd.kv_layout import kv_cache_shape
     from oracle.cache import append_kv_reference
