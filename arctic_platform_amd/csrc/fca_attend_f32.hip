@@ -17,6 +17,8 @@
 //            probabilities from LDS, again one address for all lanes.
 // Items are dealt round-robin over the waves; nothing here draws from the work counter of
 // the metadata header, which therefore stays zero.
+#include <hip/hip_ext.h>
+
 #include "fca_attend_common.h"
 
 namespace fca {
@@ -205,13 +207,20 @@ hipError_t launch_attend_f32(const AttendParams& p, const fca_plan& plan, int ma
   if (max_workgroups > 0 && max_workgroups < grid) grid = max_workgroups;
   if ((int64_t)grid * kF32Waves > max_tickets) grid = (int)((max_tickets + kF32Waves - 1) / kF32Waves);
   if (grid < 1) grid = 1;
+  // (a pending pair of timing events is this launch's, as for the other attention kernels)
+  hipEvent_t ev_start, ev_stop;
+  take_attend_timing(&ev_start, &ev_stop);
+#define FCA_LAUNCH_F32(D_) \
+  if (ev_start) hipExtLaunchKernelGGL((fca_attend_f32_kernel<D_>), dim3(grid), dim3(kF32Threads), 0, stream, ev_start, ev_stop, 0, p); \
+  else hipLaunchKernelGGL((fca_attend_f32_kernel<D_>), dim3(grid), dim3(kF32Threads), 0, stream, p)
   if (plan.head_dim == 128) {
-    fca_attend_f32_kernel<128><<<dim3(grid), kF32Threads, 0, stream>>>(p);
+    FCA_LAUNCH_F32(128);
   } else if (plan.head_dim == 64) {
-    fca_attend_f32_kernel<64><<<dim3(grid), kF32Threads, 0, stream>>>(p);
+    FCA_LAUNCH_F32(64);
   } else {
     return hipErrorInvalidValue;
   }
+#undef FCA_LAUNCH_F32
   return hipGetLastError();
 }
 
