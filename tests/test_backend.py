@@ -41,6 +41,21 @@ def test_config_string_and_rejections():
     meta = CommonAttentionMetadata(None, None, None, None, num_reqs=4, max_query_len=0)
     with pytest.raises(ValueError, match="max_query_len"):
         builder.build(0, meta)
+    assert builder.reproducible is False
+    assert ForestCascadeMetadataBuilder(32, 8, 128, device="cpu", forest_cascade_attn_configs='{"reproducible": true}').reproducible is True
+
+
+def test_query_runs_need_the_token_count_from_the_host():
+    """A step with query runs sizes its row arrays by the number of query tokens; that number comes
+    from the host side (num_actual_tokens, or the engine's host copy of query_start_loc), never from
+    reading the device tensor back."""
+    builder = ForestCascadeMetadataBuilder(32, 8, 128, device="cpu")
+    starts = torch.tensor([0, 3, 5], dtype=torch.int32)
+    lens = torch.tensor([40, 50], dtype=torch.int32)
+    table = torch.zeros(2, 8, dtype=torch.int32)
+    meta = CommonAttentionMetadata(starts, lens, table, torch.zeros(5, dtype=torch.int64), num_reqs=2, max_query_len=3)
+    with pytest.raises(ValueError, match="num_actual_tokens"):
+        builder.build(0, meta)
 
 
 def test_workspace_cache_is_bounded():
