@@ -20,6 +20,8 @@ __all__ = [
     "SplitLayout",
     "split_attention_forward",
     "split_attention_backward",
+    "reconstruct_sequences",
+    "deduplicate_sequences",
 ]
 
 
@@ -44,6 +46,10 @@ def __getattr__(name):
         import importlib
 
         return getattr(importlib.import_module(".split_attention", __name__), name)
+    if name in ("reconstruct_sequences", "deduplicate_sequences"):
+        from . import reconstruct
+
+        return getattr(reconstruct, name)
     if name == "append_kv":
         from . import cache
 

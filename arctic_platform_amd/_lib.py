@@ -43,6 +43,8 @@ EXPORTS = (
     "fca_split_workspace_bytes",
     "fca_split_attention_forward",
     "fca_split_attention_backward",
+    "fca_gather_rows",
+    "fca_sum_rows",
 )
 
 
@@ -186,6 +188,8 @@ def declare_signatures(lib: ctypes.CDLL) -> ctypes.CDLL:
     lib.fca_split_attention_backward.argtypes = (
         [P(FcaSplitPlan)] + [VP, I64] * 5 + [VP, VP, F32, VP] + [VP, I64] * 3 + [VP]
     )
+    lib.fca_gather_rows.argtypes = [VP, I64, VP, I64, I64, VP, I64, VP]
+    lib.fca_sum_rows.argtypes = [VP, I64, VP, VP, I64, I64, I32, VP, I64, VP]
     for name in EXPORTS:
         if name not in ("fca_version", "fca_last_error"):
             getattr(lib, name).restype = ctypes.c_int

@@ -629,3 +629,42 @@ int fca_split_attention_backward(const fca_split_plan* plan, const void* q_dev, 
 }
 
 }  // extern "C"
+
+// ---- rows of a deduplicated tensor to whole samples and back -----------------------------
+extern "C" {
+
+int fca_gather_rows(const void* src_dev, int64_t src_stride_bytes, const int32_t* index_dev, int64_t num_rows, int64_t row_bytes,
+                    void* dst_dev, int64_t dst_stride_bytes, void* stream) {
+  if (num_rows < 0 || row_bytes < 0) return fail(FCA_ERR_INVALID_ARG, "num_rows and row_bytes must be >= 0");
+  if (num_rows == 0 || row_bytes == 0) return FCA_OK;
+  if (num_rows > 0x7fffffffLL) return fail(FCA_ERR_UNSUPPORTED, "more than 2^31 - 1 rows");
+  if (!src_dev || !index_dev || !dst_dev) return fail(FCA_ERR_INVALID_ARG, "src, index and dst must be non-NULL");
+  if (row_bytes % 16 || src_stride_bytes % 16 || dst_stride_bytes % 16 || (reinterpret_cast<uintptr_t>(src_dev) & 15) ||
+      (reinterpret_cast<uintptr_t>(dst_dev) & 15))
+    return fail(FCA_ERR_INVALID_ARG, "rows must be 16-byte aligned: pointers, strides and row_bytes multiples of 16");
+  if (src_stride_bytes < row_bytes || dst_stride_bytes < row_bytes)
+    return fail(FCA_ERR_INVALID_ARG, "row strides must be at least row_bytes");
+  hipError_t e = fca::launch_gather_rows(src_dev, src_stride_bytes, index_dev, num_rows, row_bytes, dst_dev, dst_stride_bytes,
+                                         static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? FCA_OK : hip_fail(e, "row gather launch");
+}
+
+int fca_sum_rows(const void* src_dev, int64_t src_stride_bytes, const int32_t* offsets_dev, const int32_t* rows_dev,
+                 int64_t num_dst_rows, int64_t channels, int32_t dtype, void* dst_dev, int64_t dst_stride_bytes, void* stream) {
+  if (num_dst_rows < 0 || channels < 0) return fail(FCA_ERR_INVALID_ARG, "num_dst_rows and channels must be >= 0");
+  if (dtype != FCA_BF16 && dtype != FCA_F32) return fail(FCA_ERR_UNSUPPORTED, "dtype %d is not supported (bf16 or f32)", dtype);
+  if (num_dst_rows == 0 || channels == 0) return FCA_OK;
+  if (num_dst_rows > 0x7fffffffLL) return fail(FCA_ERR_UNSUPPORTED, "more than 2^31 - 1 rows");
+  if (!src_dev || !offsets_dev || !rows_dev || !dst_dev) return fail(FCA_ERR_INVALID_ARG, "src, offsets, rows and dst must be non-NULL");
+  const int64_t row_bytes = channels * (dtype == FCA_F32 ? 4 : 2);
+  if (channels % 8 || src_stride_bytes % 16 || dst_stride_bytes % 16 || (reinterpret_cast<uintptr_t>(src_dev) & 15) ||
+      (reinterpret_cast<uintptr_t>(dst_dev) & 15))
+    return fail(FCA_ERR_INVALID_ARG, "channels must be a multiple of 8 and rows 16-byte aligned");
+  if (src_stride_bytes < row_bytes || dst_stride_bytes < row_bytes)
+    return fail(FCA_ERR_INVALID_ARG, "row strides must be at least one row");
+  hipError_t e = fca::launch_sum_rows(src_dev, src_stride_bytes, offsets_dev, rows_dev, num_dst_rows, channels, dtype == FCA_F32,
+                                      dst_dev, dst_stride_bytes, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? FCA_OK : hip_fail(e, "row sum launch");
+}
+
+}  // extern "C"

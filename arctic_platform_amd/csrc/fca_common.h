@@ -296,5 +296,9 @@ hipError_t launch_attend_f32(const AttendParams& p, const fca_plan& plan, int ma
 hipError_t launch_attend32(const AttendParams& p, const fca_plan& plan, int kv_dtype, int grid, hipStream_t stream);
 hipError_t launch_merge(const MergeParams& p, hipStream_t stream);
 hipError_t launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
+hipError_t launch_gather_rows(const void* src, int64_t src_stride, const int32_t* index, int64_t num_rows, int64_t row_bytes,
+                              void* dst, int64_t dst_stride, hipStream_t stream);  // strides in bytes
+hipError_t launch_sum_rows(const void* src, int64_t src_stride, const int32_t* offsets, const int32_t* rows, int64_t num_dst_rows,
+                           int64_t channels, bool f32, void* dst, int64_t dst_stride, hipStream_t stream);
 
 }  // namespace fca

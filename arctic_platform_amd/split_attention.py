@@ -63,6 +63,8 @@ class SplitLayout:
         )
         self.device = torch.device(device)
         self.dev = torch.from_numpy(self.host).to(self.device) if self.device.type == "cuda" else None
+        # original batch index of every sample, group by group (None: numbered in layout order)
+        self.sample_ids = None
         self._scratch = {} if scratch_pool is None else scratch_pool
 
     @classmethod
@@ -78,14 +80,16 @@ class SplitLayout:
         prompt's count from the group's first sample, one response count per sample in group order."""
 
         def valid(seg):
-            return int(seg.get("num_valid_tokens", seg["end"] - seg["start"]))
+            return int(seg["num_valid_tokens"] if "num_valid_tokens" in seg else seg["end"] - seg["start"])
 
         segs = {(s["group_idx"], s["type"], s["original_idx"]): s for s in reconstruction_info["segment_info"]}
         groups = []
         for g, members in enumerate(reconstruction_info["prompt_groups"]):
             prompt = valid(segs[(g, "prompt", members[0])])
             groups.append((prompt, [valid(segs[(g, "response", m)]) for m in members]))
-        return cls(groups, device=device, sliding_window=sliding_window)
+        layout = cls(groups, device=device, sliding_window=sliding_window)
+        layout.sample_ids = [[int(m) for m in members] for members in reconstruction_info["prompt_groups"]]
+        return layout
 
     # views of the layout array (tests, inspection)
     def kv_lim(self):

@@ -357,6 +357,24 @@ int fca_split_attention_backward(const fca_split_plan* plan, const void* q_dev, 
                                  int64_t dq_stride, void* dk_dev, int64_t dk_stride, void* dv_dev, int64_t dv_stride,
                                  void* stream);
 
+/* ---- whole samples from a deduplicated tensor, and back ---------------------------------
+ * dst[i] = src[index[i]] for rows of row_bytes bytes (a multiple of 16; strides in bytes,
+ * multiples of 16; index < 0 gives a row of zeros).  With the index of every sample's prompt
+ * rows followed by its response rows this is ZoRRoTrain.reconstruct_sequences in its packed
+ * form (arctic_platform/rl/zorro_train/zorro_train.py:1071-1159, and the row-per-program
+ * Triton kernel at :160-235); with the index of each group's first sample's prompt rows and
+ * every sample's response rows it is deduplicate_sequences (:1162-1179).  The index arrays
+ * are made on the host once per batch. */
+int fca_gather_rows(const void* src_dev, int64_t src_stride_bytes, const int32_t* index_dev, int64_t num_rows, int64_t row_bytes,
+                    void* dst_dev, int64_t dst_stride_bytes, void* stream);
+/* The transpose of a gather, for its gradient: dst[j] = sum over k in [offsets[j],
+ * offsets[j + 1]) of src[rows[k]], channels (a multiple of 8) of bf16 or fp32 per row, added
+ * up in fp32 in the order given (no atomics: the result does not depend on timing).  The
+ * gradient of a reconstructed tensor with respect to the deduplicated one: a prompt row sums
+ * the rows of its copies in all samples of its group. */
+int fca_sum_rows(const void* src_dev, int64_t src_stride_bytes, const int32_t* offsets_dev, const int32_t* rows_dev,
+                 int64_t num_dst_rows, int64_t channels, int32_t dtype, void* dst_dev, int64_t dst_stride_bytes, void* stream);
+
 /* Plain device-to-device copy with 16-byte loads and stores.  No counterpart in the
  * reference: it is the known-size yardstick for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE
  * readings of the kernels above. */

@@ -123,6 +123,44 @@ def reconstruct(x, layout):
     return samples
 
 
+def reconstruct_packed(x, layout, sample_ids=None):
+    """Deduplicated rows -> every sample's prompt rows followed by its response rows, samples in
+    the order of their batch indices, one packed tensor (the loops of
+    ``ZoRRoTrain._reconstruct_sequences_packed``, zorro_train.py:1071-1159).  ``sample_ids[g]``:
+    batch indices of group g's samples in layout order (default: numbered in layout order)."""
+    per_sample = reconstruct(x, layout)
+    if sample_ids is None:
+        order = list(range(len(per_sample)))
+    else:
+        flat = [s for ids in sample_ids for s in ids]
+        order = sorted(range(len(flat)), key=lambda k: flat[k])
+    return torch.cat([per_sample[k] for k in order]) if per_sample else x[:0]
+
+
+def deduplicate_packed(full, layout, sample_ids=None):
+    """The way back (``ZoRRoTrain.deduplicate_sequences`` for an unpadded batch, zorro_train.py:
+    1162-1179 and the packed variant behind it): a group's prompt rows from its first sample,
+    every response from its own sample.  A group without samples gets zero prompt rows."""
+    lens = [p + r for p, rs in layout for r in rs]
+    flat = list(range(len(lens))) if sample_ids is None else [s for ids in sample_ids for s in ids]
+    # where every sample starts in the packed tensor (samples lie in batch order)
+    by_batch = sorted(range(len(flat)), key=lambda k: flat[k])
+    start, at = {}, 0
+    for k in by_batch:
+        start[k] = at
+        at += lens[k]
+    out, k = [], 0
+    for p, rs in layout:
+        if rs:
+            out.append(full[start[k] : start[k] + p])
+        else:
+            out.append(torch.zeros((p,) + tuple(full.shape[1:]), dtype=full.dtype))
+        for r in rs:
+            out.append(full[start[k] + p : start[k] + p + r])
+            k += 1
+    return torch.cat(out) if out else full[:0]
+
+
 def full_attention_of_samples(q, k, v, layout, scale, dtype=torch.float64, window=None):
     """Every sample's whole sequence attended causally on its own, from the deduplicated
     tensors; returns per sample (out, lse) of prompt + response rows."""

@@ -617,6 +617,44 @@ def test_cache_append_and_gather(emu, kv_dtype, d):
         assert ((back_k.float() - key.float()).abs()[live] <= step).all()
 
 
+# ---- whole samples from a deduplicated tensor and back ----------------------------------------------
+@pytest.mark.parametrize("dtype,channels", [(torch.bfloat16, 64), (torch.float32, 8), (torch.bfloat16, 2560)])
+def test_row_gather_and_row_sum(emu, dtype, channels):
+    """fca_gather_rows with the index of a reconstruction and of a deduplication (negative entries give
+    zero rows; strided sources), and fca_sum_rows as the gradient of a reconstruction, against plain
+    indexing.  Guard pages sit behind every buffer."""
+    from arctic_platform_amd.reconstruct import SampleIndex
+    from arctic_platform_amd.split_attention import SplitLayout
+    from oracle.split_attention import deduplicate_packed, reconstruct_packed
+
+    layout, ids = [(40, [20, 33, 7]), (7, [5]), (3, [])], [[3, 0, 2], [1], []]
+    ix = SampleIndex(SplitLayout(layout, device="cpu"), ids)
+    t, esz = ix.num_dedup, torch.empty((), dtype=dtype).element_size()
+    gen = torch.Generator().manual_seed(channels)
+    wide = guarded((torch.randn(t, 2 * channels, generator=gen) * 10).to(dtype))
+    x = wide[:, channels:]  # every second half row: a strided source
+    full = guarded(torch.full((ix.num_full, channels), float("nan")).to(dtype))
+    index = guarded(torch.from_numpy(ix.full_from))
+    _ok(emu, emu.fca_gather_rows(x.data_ptr(), x.stride(0) * esz, index.data_ptr(), ix.num_full, channels * esz, full.data_ptr(), full.stride(0) * esz, None))
+    assert torch.equal(full, reconstruct_packed(x, layout, ids))
+    back = guarded(torch.full((t, channels), float("nan")).to(dtype))
+    index2 = guarded(torch.from_numpy(ix.dedup_from))
+    _ok(emu, emu.fca_gather_rows(full.data_ptr(), full.stride(0) * esz, index2.data_ptr(), t, channels * esz, back.data_ptr(), back.stride(0) * esz, None))
+    assert torch.equal(back, deduplicate_packed(full, layout, ids))
+    assert not back[-3:].any()  # the prompt of the group without samples
+    # the gradient of the reconstruction: every deduplicated row sums its copies
+    grad_full = guarded(torch.randn(ix.num_full, channels, generator=gen).to(dtype))
+    grad = guarded(torch.full((t, channels), float("nan")).to(dtype))
+    offs, rows = guarded(torch.from_numpy(ix.copies_offsets)), guarded(torch.from_numpy(ix.copies_rows))
+    code = _lib.FCA_F32 if dtype == torch.float32 else _lib.FCA_BF16
+    _ok(emu, emu.fca_sum_rows(grad_full.data_ptr(), grad_full.stride(0) * esz, offs.data_ptr(), rows.data_ptr(), t, channels, code, grad.data_ptr(), grad.stride(0) * esz, None))
+    want = torch.zeros(t, channels, dtype=torch.float64).index_add_(0, torch.from_numpy(ix.full_from).long(), grad_full.double())
+    torch.testing.assert_close(grad.double(), want, rtol=1e-2 if dtype == torch.bfloat16 else 1e-6, atol=1e-2 if dtype == torch.bfloat16 else 1e-6)
+    # argument checks
+    assert emu.fca_gather_rows(x.data_ptr(), x.stride(0) * esz, index.data_ptr(), ix.num_full, channels * esz - 8, full.data_ptr(), full.stride(0) * esz, None) == -1
+    assert emu.fca_sum_rows(grad_full.data_ptr(), grad_full.stride(0) * esz, offs.data_ptr(), rows.data_ptr(), t, channels, _lib.FCA_FP8_E4M3, grad.data_ptr(), grad.stride(0) * esz, None) == -2
+
+
 # ---- split attention of the trainer --------------------------------------------------------------
 def _close(name, got, ref, scale_tol):
     got, ref = got.detach().double(), ref.detach().double()
