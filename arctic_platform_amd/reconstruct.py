@@ -108,7 +108,10 @@ def _rows(x, tokens, what):
         raise ValueError(f"{what} must be [T, ...] or [1, T, ...] with T = {tokens}, got {tuple(x.shape)}")
     if not x2.is_cuda:
         raise RuntimeError(f"rows are gathered on the GPU; {what} must be a device tensor")
-    x2 = x2.reshape(tokens, -1) if x2.is_contiguous() else x2.contiguous().reshape(tokens, -1)
+    width = 1
+    for n in x2.shape[1:]:
+        width *= int(n)
+    x2 = (x2 if x2.is_contiguous() else x2.contiguous()).reshape(tokens, width)  # (an explicit width: no rows is a legal batch)
     if (x2.shape[1] * x2.element_size()) % 16 or x2.data_ptr() % 16:
         raise ValueError(f"a row of {what} must be a multiple of 16 bytes and 16-byte aligned")
     return x2, batched
