@@ -118,6 +118,8 @@ def _rows(x, tokens, what):
 
 
 def _gather(src, index, num_rows):
+    if src.shape[0] == 0:  # nothing to take rows from: every index is "none"
+        return torch.zeros((num_rows, src.shape[1]), dtype=src.dtype, device=src.device)
     out = torch.empty((num_rows, src.shape[1]), dtype=src.dtype, device=src.device)
     _lib.check(
         _lib.load_library().fca_gather_rows(
