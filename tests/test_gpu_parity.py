@@ -293,3 +293,27 @@ def test_items_shared_by_pairs_of_waves(gpu, index, workgroups, chunk):
     torch.cuda.synchronize()
     assert_matches_oracle(out2, lse2, ref_out, ref_lse, what="second launch")
     assert int(ctr.abs().max()) == 0
+
+
+def test_reproducible_launches_share_no_item_and_repeat_bit_for_bit(gpu):
+    """fca_tensors.reproducible: on a batch and grid where the default launch lets pairs of waves
+    attend their last items together, no second partial is written, two launches agree in every
+    bit, and the result is the oracle's."""
+    from arctic_platform_amd.ops import forest_cascade_decode
+
+    w = make_config(2, device=gpu, shrink=4, poison_unused=True)
+    md, out, lse = _run(w, max_workgroups=8, reproducible=True, chunk_tokens=512)
+    rows = md.plan.num_seqs * md.layout.max_partials * w.num_q_heads
+    md.partial_lse.view(-1, 2)[rows:].fill_(float("nan"))
+    out2, lse2 = forest_cascade_decode(w.q, w.kv_cache, md, w.scale, w.k_scale, w.v_scale)
+    torch.cuda.synchronize()
+    assert torch.equal(out2.view(torch.int16), out.view(torch.int16)) and torch.equal(lse2.view(torch.int32), lse.view(torch.int32))
+    assert bool(torch.isnan(md.partial_lse.view(-1, 2)[rows:]).all()), "a second partial was written"
+    ref_out, ref_lse = oracle_for(w)
+    assert_matches_oracle(out, lse, ref_out, ref_lse, what="reproducible launch")
+    # the same batch with sharing: second partials appear
+    md.reproducible = False
+    forest_cascade_decode(w.q, w.kv_cache, md, w.scale, w.k_scale, w.v_scale)
+    torch.cuda.synchronize()
+    assert bool((~torch.isnan(md.partial_lse.view(-1, 2)[rows:, 0])).any())
+
