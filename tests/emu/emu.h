@@ -76,6 +76,7 @@ struct Block {
 inline Block* B = nullptr;
 inline Fiber* F = nullptr;
 inline bool dma_late = false;  // direct-to-LDS loads land at the wait that covers them instead of at once
+inline unsigned long long streamed_bytes = 0;  // bytes requested by non-temporal loads (the kernels stream their KV tiles with them)
 inline long n_progress = 0;  // rendezvous completed and fibers finished (deadlock detection)
 
 inline void yield() {
@@ -453,5 +454,5 @@ inline int cvt_pk_fp8_f32(float a, float b, int old, bool hi) {
 // (a wave runs in lockstep on the GPU; here its lanes run one after the other, so wherever lanes read what
 // other lanes of the wave wrote, the scheduling barrier that marks the place has to be a real rendezvous)
 #define __builtin_amdgcn_wave_barrier() ((void)emu::wave_exchange("", 0))
-#define __builtin_nontemporal_load(p) (*(p))
+#define __builtin_nontemporal_load(p) (emu::streamed_bytes += sizeof(*(p)), *(p))
 #define __builtin_nontemporal_store(v, p) (*(p) = (v))

@@ -3,3 +3,11 @@
 
 // 1: a direct-to-LDS load lands when a wait covers it (the latest the hardware allows); 0: at once.
 extern "C" void emu_set_dma_late(int on) { emu::dma_late = on != 0; }
+
+// Bytes requested by non-temporal loads since the last call (the streaming kernels read their KV tiles,
+// and the merge its partial rows, with such loads).
+extern "C" unsigned long long emu_take_streamed_bytes() {
+  const unsigned long long n = emu::streamed_bytes;
+  emu::streamed_bytes = 0;
+  return n;
+}
