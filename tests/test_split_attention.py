@@ -401,75 +401,6 @@ def test_forward_and_backward_match_the_oracle(layout, heads):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("window", [1, 20, 32, 100, 4096])
-@pytest.mark.parametrize("heads", [(8, 2, 128), (6, 2, 64), (4, 4, 128)])
-def test_sliding_window_matches_the_oracle(heads, window):
-    """The window of the trainer's attention calls (qwen_attention_patcher.py:1206, :1226):
-    shorter than a tile, a tile, across tiles, longer than every sample; the kernels that share
-    their operands through LDS and the per-wave ones."""
-    for layout in LAYOUTS:
-        _run_case(layout, *heads, seed=51, window=window)
-
-
-@pytest.mark.gpu
-@pytest.mark.parametrize("dropout,window", [(0.1, None), (0.5, None), (0.25, 40)])
-@pytest.mark.parametrize("heads", [(8, 2, 128), (6, 2, 64), (4, 4, 128)])
-def test_attention_dropout_matches_the_oracle(heads, dropout, window):
-    """Attention dropout (the trainer's calls pass module.attention_dropout while training,
-    qwen_attention_patcher.py:1204, :1224): forward and the three gradients against the oracle
-    under the same mask, which the host restates from the seed; alone and with a window."""
-    for layout in LAYOUTS:
-        _run_case(layout, *heads, seed=71, window=window, dropout=dropout)
-
-
-@pytest.mark.gpu
-def test_attention_dropout_through_autograd_repeats_under_a_seed():
-    layout = [(70, [40, 33]), (20, [50])]
-    hq, hkv, d = 8, 2, 128
-    q, k, v = (x.cuda().requires_grad_() for x in _inputs(layout, hq, hkv, d, 81, torch.bfloat16))
-    L = SplitLayout(layout)
-    torch.manual_seed(5)
-    a = split_attention(q, k, v, L, d**-0.5, dropout=0.2)
-    torch.manual_seed(5)
-    b = split_attention(q, k, v, L, d**-0.5, dropout=0.2)
-    c = split_attention(q, k, v, L, d**-0.5, dropout=0.2)
-    assert torch.equal(a, b) and not torch.equal(a, c)
-    a.float().sum().backward()
-    assert all(bool(torch.isfinite(x.grad.float()).all()) for x in (q, k, v))
-    # the forward's seed reaches the backward: an explicit seed against the oracle
-    q.grad = k.grad = v.grad = None
-    out = split_attention(q, k, v, L, d**-0.5, dropout=0.2, seed=1234)
-    w = torch.randn(out.shape, generator=torch.Generator().manual_seed(82)).bfloat16()
-    (out.float() * w.cuda().float()).sum().backward()
-    q64, k64, v64 = (x.detach().cpu().double().requires_grad_() for x in (q, k, v))
-    keep = dropout_keep_mask(1234, 0.2, hq, total_tokens(layout))
-    ro, _ = oracle_split(q64, k64, v64, layout, d**-0.5, keep=keep, dropout=0.2)
-    (ro * w.double()).sum().backward()
-    _close("out", out, ro, 2e-2 / max(1.0, float(ro.detach().abs().max())))
-    for name, got, ref in (("dq", q.grad, q64.grad), ("dk", k.grad, k64.grad), ("dv", v.grad, v64.grad)):
-        _close(name, got, ref, 1e-2)
-
-
-@pytest.mark.gpu
-def test_sliding_window_through_autograd_and_on_long_responses():
-    """Long responses over a long prompt with a window much shorter than either (most tiles of
-    the walks are left out), through the autograd function with the window passed on the call."""
-    layout = [(700, [400, 260]), (300, [500])]
-    hq, hkv, d, window = 8, 2, 128, 128
-    q, k, v = (x.cuda().requires_grad_() for x in _inputs(layout, hq, hkv, d, 61, torch.bfloat16))
-    L = SplitLayout(layout, sliding_window=window)
-    out = split_attention(q, k, v, L, d**-0.5, dropout=0.0, sliding_window=window)
-    w = torch.randn(out.shape, generator=torch.Generator().manual_seed(62)).bfloat16()
-    (out.float() * w.cuda().float()).sum().backward()
-    q64, k64, v64 = (x.detach().cpu().double().requires_grad_() for x in (q, k, v))
-    ro, _ = oracle_split(q64, k64, v64, layout, d**-0.5, window=window)
-    (ro * w.double()).sum().backward()
-    _close("out", out, ro, 2e-2 / max(1.0, float(ro.detach().abs().max())))
-    for name, got, ref in (("dq", q.grad, q64.grad), ("dk", k.grad, k64.grad), ("dv", v.grad, v64.grad)):
-        _close(name, got, ref, 1e-2)
-
-
-@pytest.mark.gpu
 def test_random_layouts_match_the_oracle():
     rng = random.Random(99)
     done = 0
