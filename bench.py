@@ -521,7 +521,7 @@ def main():
     fp32 = w.q.dtype == torch.float32
     # distinct copies at distinct addresses: same values, so every copy gives the same result
     caches = [w.kv_cache] + [w.kv_cache.clone() for _ in range(max(1, args.kv_copies) - 1)]
-    chunk = args.chunk or 1024
+    chunk = args.chunk or (512 if w.head_dim == 256 else 1024)  # the adapter's defaults
     rows = args.rows or (64 if args.config == 3 else 32)
     kw = dict(num_q_heads=w.num_q_heads, num_kv_heads=w.num_kv_heads, head_dim=w.head_dim, chunk_tokens=chunk, rows_per_item=rows)
     if args.kv_reread:

@@ -23,6 +23,15 @@ def test_backend_surface():
     assert b.get_impl_cls() is ForestCascadeAttentionImpl and b.get_builder_cls() is ForestCascadeMetadataBuilder
 
 
+def test_default_chunk_follows_the_head_size():
+    """1024-token chunks; 512 at head size 256, whose work list is short (two KV heads) and whose
+    kernel holds one tile buffer; a configured value wins."""
+    cls = ForestCascadeAttentionBackend.get_builder_cls()
+    assert cls(32, 8, 128, device="cpu").chunk_tokens == 1024
+    assert cls(16, 2, 256, device="cpu").chunk_tokens == 512
+    assert cls(16, 2, 256, device="cpu", forest_cascade_attn_configs='{"chunk_tokens": 2048}').chunk_tokens == 2048
+
+
 def test_config_string_and_rejections():
     assert parse_forest_cascade_configs("{}") == {} and parse_forest_cascade_configs(None) == {}
     assert parse_forest_cascade_configs('{"chunk_tokens": 512}') == {"chunk_tokens": 512}
