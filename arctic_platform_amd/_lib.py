@@ -92,6 +92,7 @@ class FcaTensors(ctypes.Structure):
         ("softmax_scale", ctypes.c_float),
         ("reproducible", ctypes.c_int32),
         ("max_workgroups", ctypes.c_int32),
+        ("tile_buffers", ctypes.c_int32),
     ]
 
 

@@ -78,11 +78,12 @@ def parse_forest_cascade_configs(value) -> dict:
     query rows than one row tile holds, e.g. more than rows_per_item / (Hq / Hkv) samples per
     prompt; false: stream; absent: decided per step from the query lengths), reproducible
     (true: no work item is cut between two waves at a point that depends on timing, so equal
-    inputs give equal bits, at a few per cent of the speed)."""
+    inputs give equal bits, at a few per cent of the speed), fp8_tile_buffers (3: attention on an
+    fp8 cache at head size 128 keeps three tiles in flight per wave instead of two)."""
     if value is None or value == "":
         return {}
     cfg = json.loads(value) if isinstance(value, str) else dict(value)
-    unknown = set(cfg) - {"chunk_tokens", "rows_per_item", "max_levels", "enable", "rebuild_every", "kv_reread", "reproducible"}
+    unknown = set(cfg) - {"chunk_tokens", "rows_per_item", "max_levels", "enable", "rebuild_every", "kv_reread", "reproducible", "fp8_tile_buffers"}
     if unknown:
         raise ValueError(f"unknown forest_cascade_attn_configs keys: {sorted(unknown)}")
     return cfg
@@ -157,6 +158,9 @@ class ForestCascadeMetadataBuilder:
         self.kv_reread = None if cfg.get("kv_reread") is None else bool(cfg["kv_reread"])
         # the same bits from every launch on the same inputs (no item attended by two waves together)
         self.reproducible = bool(cfg.get("reproducible", False))
+        self.fp8_tile_buffers = int(cfg.get("fp8_tile_buffers", 0))
+        if self.fp8_tile_buffers not in (0, 3):
+            raise ValueError(f"fp8_tile_buffers must be 0 or 3, got {self.fp8_tile_buffers}")
         group = num_q_heads // num_kv_heads
         self.rows_per_item = int(cfg.get("rows_per_item", 64 if group > 32 else 32))
         # several query tokens per sequence multiply the rows of every shared node: unless the
@@ -310,6 +314,7 @@ class ForestCascadeMetadataBuilder:
         )
         if forest is not None:  # (a test double of the builder returns none)
             forest.reproducible = self.reproducible
+            forest.fp8_tile_buffers = self.fp8_tile_buffers
         self._keep(key, forest)
         return ForestCascadeMetadata(forest=forest, slot_mapping=m.slot_mapping[:num_tokens], num_decode_tokens=num_tokens)
 

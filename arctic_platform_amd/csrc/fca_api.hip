@@ -82,6 +82,11 @@ int check_tensors(const fca_plan* p, const fca_tensors* t, bool f32_ok = false) 
     return fail(FCA_ERR_INVALID_ARG, "block_table_stride %lld is smaller than max_blocks %d",
                 (long long)t->block_table_stride, p->max_blocks);
   if (t->max_workgroups < 0) return fail(FCA_ERR_INVALID_ARG, "max_workgroups must be >= 0, got %d", t->max_workgroups);
+  if (t->tile_buffers != 0 &&
+      !(t->tile_buffers == 3 && t->kv_dtype == FCA_FP8_E4M3 && p->head_dim == 128 && p->rows_per_item == 32))
+    return fail(FCA_ERR_UNSUPPORTED,
+                "tile_buffers %d: 0, or 3 for an fp8 cache at head_dim 128 with rows_per_item 32 (got kv_dtype %d, head_dim %d, rows_per_item %d)",
+                t->tile_buffers, t->kv_dtype, p->head_dim, p->rows_per_item);
   return FCA_OK;
 }
 
@@ -132,7 +137,7 @@ int run_attend(const fca_plan* p, const fca_tensors* t, void* meta, void* po, fl
   const fca::AttendParams a = attend_params(p, t, meta, po, pl, select);
   hipError_t e = t->kv_dtype == FCA_F32
                      ? fca::launch_attend_f32(a, *p, t->max_workgroups, static_cast<hipStream_t>(stream))
-                     : fca::launch_attend(a, *p, t->kv_dtype, t->max_workgroups, static_cast<hipStream_t>(stream));
+                     : fca::launch_attend(a, *p, t->kv_dtype, t->max_workgroups, t->tile_buffers, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? FCA_OK : hip_fail(e, "attention pass launch");
 }
 

@@ -450,7 +450,7 @@ static int cached_cu_count() {
   return cus;
 }
 
-hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, int max_workgroups, hipStream_t stream) {
+hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, int max_workgroups, int tile_buffers, hipStream_t stream) {
   const bool fp8 = kv_dtype == FCA_FP8_E4M3;
   const int nrt = plan.rows_per_item / 32;
   // Four independent waves per workgroup.  At head size 128 a wave uses the whole register
@@ -466,7 +466,7 @@ hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dty
   if (max_workgroups > 0 && max_workgroups < grid) grid = max_workgroups;
   if ((int64_t)grid * kWaves > max_tickets) grid = (int)((max_tickets + kWaves - 1) / kWaves);
   if (grid < 1) grid = 1;
-  if (nrt == 1 && plan.head_dim != 256) return launch_attend32(p, plan, kv_dtype, grid, stream);
+  if (nrt == 1 && plan.head_dim != 256) return launch_attend32(p, plan, kv_dtype, tile_buffers, grid, stream);
   // With sharing on, a launch reads every KV block once: stream it past the caches.  With
   // sharing off, sequences of a group read the same blocks again and again and the
   // memory-side cache serves the repeats, so the loads stay ordinary; likewise when query

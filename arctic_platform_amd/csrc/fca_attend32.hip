@@ -7,9 +7,13 @@
 // following items -- query rows of item k+1, block ids and member sequences of item k+2,
 // record of item k+3, ticket of item k+4 -- so every step reads what the step before it
 // fetched one whole item earlier, and nothing is ever waited for at the place it was
-// requested.  With the next item's block ids at hand, the two tile buffers are refilled
-// with the next item's first tiles as soon as the current item's last tiles have been
-// consumed, exactly as they are refilled inside an item.
+// requested.  Tiles are attended in groups of as many as there are tile buffers (NB: two; three
+// in the instance for fp8 at head size 128 that a caller can ask for, whose tiles are half the
+// size).  Where an expression differs between the two it is picked by NB at compile time with
+// the two-buffer form spelt as it always was: the two-buffer instances are the kernels that
+// have been measured, and they compile to the same instructions as before NB existed.  With the next item's block ids
+// at hand, the buffers are refilled with the next item's first tiles as soon as the current
+// item's last tiles have been consumed, exactly as they are refilled inside an item.
 //
 // The last item of a wave is shared with a wave of another XCD.  XCDs stream at different
 // speeds (the slowest takes about a sixth longer per tile than the fastest, and which is
@@ -17,8 +21,8 @@
 // ahead of use, the draws come too early to tell a fast wave from a slow one.  So the
 // largest items of the list are set aside, one per pair of waves (grids of a multiple of
 // eight workgroups): both waves of a pair take
-// the item as their last, one from its first pair of tiles upwards, the other from its last
-// pair downwards, each claiming the next pair of tiles from a counter of the pair until the
+// the item as their last, one from its first group of tiles upwards, the other from its last
+// group downwards, each claiming the next group of tiles from a counter of the pair until the
 // claims meet.  Whichever wave arrives earlier or streams faster takes more of the item,
 // and each wave writes a partial of its own (the second one into rows set aside behind the
 // ordinary partial rows; the first one's row scale carries the second one's address).
@@ -35,7 +39,7 @@
 
 namespace fca {
 
-template <int D, bool FP8, bool STREAM>
+template <int D, bool FP8, bool STREAM, int NB = 2>
 __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_attend32_kernel(AttendParams p) {
   constexpr int KS = D / 16;   // MFMA steps of the score product
   constexpr int NDB = D / 32;  // 32-channel blocks of the output
@@ -59,6 +63,10 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
   // row m of the stacked query tile is (member m / G, head m % G)
   const int row_member = m / G;
   const int row_head = m - row_member * G;
+  // Query head of this lane's row under KV head kvh, for the three-buffer instance.  The sum is
+  // formed in 32 bits, unsigned, at every use: written as a 64-bit sum the lane's share of it is
+  // hoisted out of the item loop as a 64-bit register pair, and that instance has none to spare.
+  auto q_head_of = [&](int kvh_) -> unsigned { return (unsigned)(kvh_ * G) + (unsigned)row_head; };
   // MFMA row m carries the token whose index has bits 2 and 3 of m swapped: the score
   // accumulator then holds, per lane half, tokens 8h..8h+7 of each block in register order.
   const int tok_of_m = (m & 3) | ((m & 4) << 1) | ((m & 8) >> 1);
@@ -159,7 +167,7 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
   auto load_q = [&](bf16x8 (&q)[KS], int seq, int mcnt, int kvh) {
     const bool live = row_member < mcnt;
     const __bf16* qp = reinterpret_cast<const __bf16*>(p.q) + (int64_t)seq * p.q_seq_stride +
-                       (int64_t)(kvh * G + row_head) * p.q_head_stride;
+                       (NB == 3 ? (int64_t)q_head_of(kvh) : (int64_t)(kvh * G + row_head)) * p.q_head_stride;
 #pragma unroll
     for (int i = 0; i < KS; ++i) {
       // channel offset of MFMA step i for this lane half: the K tile hands a lane 16 bytes
@@ -215,21 +223,33 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
     if constexpr (FP8) {
       const float* kp = p.k_scale ? p.k_scale + head : reinterpret_cast<const float*>(p.q);
       const float* vp = p.v_scale ? p.v_scale + head : reinterpret_cast<const float*>(p.q);
-      const float k = kp[opaque_zero], v = vp[opaque_zero];
-      ks = p.k_scale ? k : 1.f;
-      vs = p.v_scale ? v : 1.f;
+      if constexpr (NB == 3) {
+        // scalar loads: their results live in scalar registers, which this instance has to
+        // spare, and their counter is not the one the tile loads are waited for by
+        const float k = *kp, v = *vp;
+        ks = p.k_scale ? k : 1.f;
+        vs = p.v_scale ? v : 1.f;
+      } else {
+        const float k = kp[opaque_zero], v = vp[opaque_zero];
+        ks = p.k_scale ? k : 1.f;
+        vs = p.v_scale ? v : 1.f;
+      }
     }
   };
   float k_scale = 1.f, v_scale = 1.f, next_k_scale = 1.f, next_v_scale = 1.f;
   load_scales(kvh, k_scale, v_scale);
-  KT kb0, kb1;
-  VT vb0, vb1;
+  // Tile buffers: two, or three where the registers allow it (an fp8 tile is half the size of a
+  // bf16 one, and with two of them in flight the kernel runs at the latency of memory rather
+  // than at its rate).  Tiles are attended in groups of NB; buffer b holds tile b of a group.
+  KT kb0, kb1, kb2;
+  VT vb0, vb1, vb2;
   {
     const int len = __builtin_amdgcn_readfirstlane(r0.z);
     const int nb = (len + kBlock - 1) / kBlock;
     const int lt = (len + kTile - 1) / kTile - 1;
     load_tile(kb0, vb0, my_blk, nb, kvh, 0);
     load_tile(kb1, vb1, my_blk, nb, kvh, min(1, lt));
+    if constexpr (NB == 3) load_tile(kb2, vb2, my_blk, nb, kvh, min(2, lt));
   }
 
   // ---- state of the item being attended
@@ -391,29 +411,34 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
     const int ntiles = (tok_len + kTile - 1) / kTile;
     const int nfull = (tok_len - (sees > 0 ? 1 : 0)) / kTile;  // tiles without masking; at most one masked tile follows
     const int last = ntiles - 1;
-    const int npairs = (ntiles + 1) >> 1;
+    const int ngroups = NB == 2 ? (ntiles + 1) >> 1 : (ntiles + NB - 1) / NB;
     // partial row this lane's query row is written to, -1 for a dead row
     const int64_t prow = row_member < mcnt
-                             ? ((int64_t)seq * p.max_partials + ord) * p.num_q_heads + kvh * G + row_head
+                             ? (NB == 3 ? ((int64_t)seq * p.max_partials + ord) * p.num_q_heads + (int64_t)q_head_of(kvh)
+                                        : ((int64_t)seq * p.max_partials + ord) * p.num_q_heads + kvh * G + row_head)
                              : -1;
     const int a_len = __builtin_amdgcn_readfirstlane(a0.z);
     const int a_nblk = (a_len + kBlock - 1) / kBlock;
     const int a_last = (a_len + kTile - 1) / kTile - 1;
-    // first tiles of the next item: its first pair, or, for the wave that takes its pair's
-    // item from the back, its last pair
-    const bool a_from_back = COOP && coop_back && ta < coop && a_last >= 2 * kCoopMinPairs - 2;
-    const int a_t0 = a_from_back ? (a_last & ~1) : 0;
+    // first tiles of the next item: its first group, or, for the wave that takes its pair's
+    // item from the back, its last group
+    const bool a_from_back = COOP && coop_back && ta < coop && (NB == 2 ? a_last >= 2 * kCoopMinPairs - 2 : (a_last + NB) / NB >= kCoopMinPairs);
+    const int a_t0 = a_from_back ? (NB == 2 ? (a_last & ~1) : NB * ((a_last + NB) / NB - 1)) : 0;
     const int a_t1 = min(a_t0 + 1, a_last);
 
-    // ---- all pairs of tiles but the last: both tiles full, refills from this item.
-    // Buffer 0 holds tile ti, buffer 1 tile ti + 1; a refill past the end (odd tile count)
+    // ---- all groups of tiles but the last: every tile full, refills from this item.
+    // Buffer b holds tile ti + b; a refill past the end (a last group that is not full)
     // repeats the last tile so that the number of loads in flight never varies.
-    for (int pr = 0; pr < npairs - 1; ++pr) {
-      const int ti = 2 * pr;
+    for (int gr = 0; gr < ngroups - 1; ++gr) {
+      const int ti = NB * gr;
       compute_tile(it, kb0, vb0, ti, std::false_type{});
-      load_tile(kb0, vb0, my_blk, nblk, kvh, ti + 2);
+      load_tile(kb0, vb0, my_blk, nblk, kvh, ti + NB);
       compute_tile(it, kb1, vb1, ti + 1, std::false_type{});
-      load_tile(kb1, vb1, my_blk, nblk, kvh, min(ti + 3, last));
+      load_tile(kb1, vb1, my_blk, nblk, kvh, min(ti + NB + 1, last));
+      if constexpr (NB == 3) {
+        compute_tile(it, kb2, vb2, ti + 2, std::false_type{});
+        load_tile(kb2, vb2, my_blk, nblk, kvh, min(ti + NB + 2, last));
+      }
     }
 
     // ---- one step for each of the items ahead
@@ -427,9 +452,9 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
     load_q(nq, a_seq, a1.x, akvh);
     load_scales(akvh, next_k_scale, next_v_scale);
 
-    // ---- the last pair: refills come from the next item (of a ticket past the end: from
+    // ---- the last group: refills come from the next item (of a ticket past the end: from
     // the last record of the list, loads nobody uses)
-    const int ti = 2 * (npairs - 1);
+    const int ti = NB * (ngroups - 1);
     if (ti < nfull)
       compute_tile(it, kb0, vb0, ti, std::false_type{});
     else
@@ -440,10 +465,21 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
     else if (ti + 1 <= last)
       compute_tile(it, kb1, vb1, ti + 1, std::true_type{});
 
-    // Write the partial (before the second refill: stores count as outstanding memory
+    if constexpr (NB == 3) {
+      load_tile(kb1, vb1, a_blk, a_nblk, akvh, a_t1);
+      if (ti + 2 < nfull)
+        compute_tile(it, kb2, vb2, ti + 2, std::false_type{});
+      else if (ti + 2 <= last)
+        compute_tile(it, kb2, vb2, ti + 2, std::true_type{});
+    }
+
+    // Write the partial (before the last refill: stores count as outstanding memory
     // operations too, and behind the refill they would be waited for together with it).
     write_partial(it, prow, mcnt * G, 0);
-    load_tile(kb1, vb1, a_blk, a_nblk, akvh, a_t1);
+    if constexpr (NB == 3)
+      load_tile(kb2, vb2, a_blk, a_nblk, akvh, min(a_t0 + 2, a_last));
+    else
+      load_tile(kb1, vb1, a_blk, a_nblk, akvh, a_t1);
 
     // ---- move on
     if (ta >= ntickets) break;
@@ -464,14 +500,14 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
     }
   }
 
-  // ---- the item shared with the other wave of the pair, the last one of both.  Pairs of
+  // ---- the item shared with the other wave of the pair, the last one of both.  Groups of
   // tiles are claimed from a counter of the pair: bits 0-9 count the claims from the front,
-  // bits 10-19 those from the back; the first two pairs at either end are granted without a
+  // bits 10-19 those from the back; the first two groups at either end are granted without a
   // claim.  A claim is good while the counts do not meet.  A wave that is through replaces its
   // own count by a marker (+2^20 from the front, -2^20 from the back) that makes every later
   // claim of the other wave fail, so that after both the counter is zero again for the next
-  // launch.  Claims run two pairs ahead of the arithmetic, refills one pair ahead, so a claim
-  // has a whole pair of tiles to come back.  An item of fewer than four pairs is attended by
+  // launch.  Claims run two groups ahead of the arithmetic, refills one group ahead, so a claim
+  // has a whole group of tiles to come back.  An item of fewer than four groups is attended by
   // its front wave alone.
   if (COOP && to_pair_item) {
     Item it;
@@ -483,11 +519,12 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
     const int ntiles = (tok_len + kTile - 1) / kTile;
     const int nfull = (tok_len - (sees > 0 ? 1 : 0)) / kTile;
     const int last = ntiles - 1;
-    const int npairs = (ntiles + 1) >> 1;
-    const bool shared_item = npairs >= kCoopMinPairs;
+    const int ngroups = NB == 2 ? (ntiles + 1) >> 1 : (ntiles + NB - 1) / NB;
+    const bool shared_item = ngroups >= kCoopMinPairs;
     if (shared_item || !coop_back) {
       const bool from_back = shared_item && coop_back;
-      const int64_t front_row = ((int64_t)seq * p.max_partials + ord) * p.num_q_heads + kvh * G + row_head;
+      const int64_t front_row = NB == 3 ? ((int64_t)seq * p.max_partials + ord) * p.num_q_heads + (int64_t)q_head_of(kvh)
+                                        : ((int64_t)seq * p.max_partials + ord) * p.num_q_heads + kvh * G + row_head;
       const int64_t back_row = p.coop_row0 + (int64_t)pair_id * 32 + m;
       const int64_t prow = row_member < mcnt ? (from_back ? back_row : front_row) : -1;
       // the front partial says where the back partial of the same query row is
@@ -499,13 +536,13 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
         if (lane == 0) claim_v = atomicAdd(ctr + opaque_zero, by);
         added += by;
       };
-      // the pair of tiles after `cur`, or -1 when there is none left for this wave
+      // the group of tiles after `cur`, or -1 when there is none left for this wave
       auto next_pair = [&](int cur) -> int {
-        if (!shared_item) return cur + 1 < npairs ? cur + 1 : -1;
+        if (!shared_item) return cur + 1 < ngroups ? cur + 1 : -1;
         const int old = __builtin_amdgcn_readfirstlane(claim_v);
         const int f = old & 1023, b = (old >> 10) & 1023;
-        if ((old >> 20) != 0 || 4 + f + b >= npairs) return -1;
-        return coop_back ? npairs - 3 - b : 2 + f;
+        if ((old >> 20) != 0 || 4 + f + b >= ngroups) return -1;
+        return coop_back ? ngroups - 3 - b : 2 + f;
       };
       auto compute_any = [&](const KT& kt, const VT& vt, int ti) {
         if (ti > last) return;
@@ -514,15 +551,19 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
         else
           compute_tile(it, kt, vt, ti, std::true_type{});
       };
-      int cur = from_back ? npairs - 1 : 0;
-      int nxt = from_back ? npairs - 2 : (npairs > 1 ? 1 : -1);  // granted
+      int cur = from_back ? ngroups - 1 : 0;
+      int nxt = from_back ? ngroups - 2 : (ngroups > 1 ? 1 : -1);  // granted
       issue_claim(inc);
       for (;;) {
         const int refill = nxt >= 0 ? nxt : cur;  // (past the end: loads nobody uses, as above)
-        compute_any(kb0, vb0, 2 * cur);
-        load_tile(kb0, vb0, my_blk, nblk, kvh, 2 * refill);
-        compute_any(kb1, vb1, 2 * cur + 1);
-        load_tile(kb1, vb1, my_blk, nblk, kvh, min(2 * refill + 1, last));
+        compute_any(kb0, vb0, NB * cur);
+        load_tile(kb0, vb0, my_blk, nblk, kvh, NB * refill);
+        compute_any(kb1, vb1, NB * cur + 1);
+        load_tile(kb1, vb1, my_blk, nblk, kvh, min(NB * refill + 1, last));
+        if constexpr (NB == 3) {
+          compute_any(kb2, vb2, NB * cur + 2);
+          load_tile(kb2, vb2, my_blk, nblk, kvh, min(NB * refill + 2, last));
+        }
         if (nxt < 0) break;
         cur = nxt;
         nxt = next_pair(cur);
@@ -536,7 +577,7 @@ __global__ __launch_bounds__(kThreads, workgroups_per_cu(D, FP8, 32)) void fca_a
   __builtin_amdgcn_s_waitcnt(0);
 }
 
-hipError_t launch_attend32(const AttendParams& p, const fca_plan& plan, int kv_dtype, int grid, hipStream_t stream) {
+hipError_t launch_attend32(const AttendParams& p, const fca_plan& plan, int kv_dtype, int tile_buffers, int grid, hipStream_t stream) {
   const bool fp8 = kv_dtype == FCA_FP8_E4M3;
   // With sharing on, a launch reads every KV block once: stream it past the caches.  With
   // sharing off, sequences of a group read the same blocks again and again and the
@@ -545,15 +586,17 @@ hipError_t launch_attend32(const AttendParams& p, const fca_plan& plan, int kv_d
   const bool stream_kv = plan.max_levels > 0 && !p.kv_reread;
   hipEvent_t ev_start, ev_stop;
   take_attend_timing(&ev_start, &ev_stop);
-#define FCA_LAUNCH(D_, F_, S_) \
-  if (ev_start) hipExtLaunchKernelGGL((fca_attend32_kernel<D_, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, ev_start, ev_stop, 0, p); \
-  else hipLaunchKernelGGL((fca_attend32_kernel<D_, F_, S_>), dim3(grid), dim3(kThreads), 0, stream, p)
-#define FCA_PICK(D_, F_) \
-  if (stream_kv) { FCA_LAUNCH(D_, F_, true); } else { FCA_LAUNCH(D_, F_, false); }
-  if (plan.head_dim == 128) {
-    if (fp8) { FCA_PICK(128, true); } else { FCA_PICK(128, false); }
+#define FCA_LAUNCH(D_, F_, S_, N_) \
+  if (ev_start) hipExtLaunchKernelGGL((fca_attend32_kernel<D_, F_, S_, N_>), dim3(grid), dim3(kThreads), 0, stream, ev_start, ev_stop, 0, p); \
+  else hipLaunchKernelGGL((fca_attend32_kernel<D_, F_, S_, N_>), dim3(grid), dim3(kThreads), 0, stream, p)
+#define FCA_PICK(D_, F_, N_) \
+  if (stream_kv) { FCA_LAUNCH(D_, F_, true, N_); } else { FCA_LAUNCH(D_, F_, false, N_); }
+  if (tile_buffers == 3) {  // fp8 at head size 128 only (checked with the tensors)
+    FCA_PICK(128, true, 3);
+  } else if (plan.head_dim == 128) {
+    if (fp8) { FCA_PICK(128, true, 2); } else { FCA_PICK(128, false, 2); }
   } else {
-    if (fp8) { FCA_PICK(64, true); } else { FCA_PICK(64, false); }
+    if (fp8) { FCA_PICK(64, true, 2); } else { FCA_PICK(64, false, 2); }
   }
 #undef FCA_PICK
 #undef FCA_LAUNCH

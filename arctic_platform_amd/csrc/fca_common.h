@@ -21,7 +21,7 @@ constexpr int kHeaderInts = 16;
 // A launch over the private items alone (fca_suffix_pass) shares no item: it would write the
 // same 32 rows per pair as the launch over the shared items that precedes the same merge.
 constexpr int kCoopMaxPairs = 1024;
-constexpr int kCoopMinPairs = 4;  // pairs of 32-token tiles an item needs to be shared
+constexpr int kCoopMinPairs = 4;  // groups of tiles (pairs; threes with three tile buffers) an item needs to be shared
 
 enum HeaderSlot {
   H_ITEMS = 0,
@@ -288,12 +288,12 @@ hipError_t launch_rows(const int32_t* query_start_loc, const int32_t* seq_lens, 
 hipError_t launch_append(const AppendParams& p, int kv_dtype, hipStream_t stream);
 hipError_t launch_gather(const AppendParams& p, int kv_dtype, hipStream_t stream);  // key / value are written
 // max_workgroups > 0 caps the grid
-hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, int max_workgroups, hipStream_t stream);
+hipError_t launch_attend(const AttendParams& p, const fca_plan& plan, int kv_dtype, int max_workgroups, int tile_buffers, hipStream_t stream);
 // Events the next attention launch of this thread records its begin and end in (NULL: none).
 void set_attend_timing(hipEvent_t start, hipEvent_t stop);
 void take_attend_timing(hipEvent_t* start, hipEvent_t* stop);
 hipError_t launch_attend_f32(const AttendParams& p, const fca_plan& plan, int max_workgroups, hipStream_t stream);
-hipError_t launch_attend32(const AttendParams& p, const fca_plan& plan, int kv_dtype, int grid, hipStream_t stream);
+hipError_t launch_attend32(const AttendParams& p, const fca_plan& plan, int kv_dtype, int tile_buffers, int grid, hipStream_t stream);
 hipError_t launch_merge(const MergeParams& p, hipStream_t stream);
 hipError_t launch_copy(const void* src, void* dst, size_t bytes, hipStream_t stream);
 hipError_t launch_gather_rows(const void* src, int64_t src_stride, const int32_t* index, int64_t num_rows, int64_t row_bytes,

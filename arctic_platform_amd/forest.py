@@ -46,6 +46,10 @@ class ForestMetadata:
     reproducible: bool = False
     # Cap of the attention grid in workgroups, 0 = the whole GPU (fca_tensors.max_workgroups).
     max_workgroups: int = 0
+    # Register tile buffers per wave for attention on an fp8 cache: 0 = the kernel's own (two), 3 =
+    # three where that instance exists (head size 128, 32-row items; fca_tensors.tile_buffers).
+    # Calls on a bf16 cache, or with another head size or tile height, are not affected.
+    fp8_tile_buffers: int = 0
 
     # ---- inspection (synchronises; not for the decode loop) -------------------------
     def header(self) -> dict:

@@ -73,6 +73,7 @@ def _tensors(q, kv_cache, meta: ForestMetadata, scale, k_scale, v_scale, f32_ok=
         float(scale),
         1 if meta.reproducible else 0,
         int(meta.max_workgroups),
+        int(meta.fp8_tile_buffers) if kv_dtype == _lib.FCA_FP8_E4M3 and plan.head_dim == 128 and plan.rows_per_item == 32 else 0,
     )
 
 

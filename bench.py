@@ -44,6 +44,7 @@ def parse_args():
     ap.add_argument("--kv-copies", type=int, default=4, help="distinct KV caches cycled over the layers")
     ap.add_argument("--chunk", type=int, default=0, help="split-K chunk in tokens (0 = default of the configuration)")
     ap.add_argument("--rows", type=int, default=0, help="query rows per work item, 32 or 64 (0 = default)")
+    ap.add_argument("--fp8-tile-buffers", type=int, default=0, choices=(0, 3), help="3: the attention kernel of an fp8 cache (--config 5) keeps three register tile buffers per wave instead of two")
     ap.add_argument("--kv-reread", action="store_true", help="keep the KV loads cacheable instead of streaming them (worth a try where a shared node fills more than one row tile, e.g. --config 3 --rows 32: its row tiles then read the same blocks at nearly the same time)")
     ap.add_argument("--time-every", type=int, default=0, help="time the attention launch of every n-th step with events (0 = every second step of a short run, about 24 launches of a long one; -1 = none; under rocprofv3 no launch is timed whatever this says)")
     ap.add_argument("--cpu-seqs", type=int, default=512, help="sequences in the CPU baseline sample (0 = skip)")
@@ -531,6 +532,7 @@ def main():
     out = torch.empty_like(w.q)
 
     md = build_forest_metadata(w.block_table, w.seq_lens, **kw)
+    md.fp8_tile_buffers = args.fp8_tile_buffers
     torch.cuda.synchronize()
     md.check()
     hdr = md.header()
@@ -651,6 +653,7 @@ def main():
             "kv_cache_copies": len(caches),
             "chunk_tokens": chunk,
             "rows_per_item": rows,
+            "fp8_tile_buffers": args.fp8_tile_buffers or None,
             "work_items": hdr["items"],
             "shared_nodes": hdr["shared_nodes"],
         },

@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define FCA_VERSION 104
+#define FCA_VERSION 105
 #define FCA_BLOCK_SIZE 16
 #define FCA_MAX_LEVELS 8
 
@@ -100,6 +100,11 @@ typedef struct fca_tensors {
   int32_t max_workgroups;      /* > 0: the attention launch uses at most this many workgroups (four waves
                                   each; two in the fp32 path), leaving the rest of the GPU to work on
                                   other streams; 0: all */
+  int32_t tile_buffers;        /* 0: the kernel's own choice (two register tile buffers per wave in the
+                                  32-row kernel).  3: three, for fp8 caches at head_dim 128 with
+                                  rows_per_item 32 only (an fp8 tile is half the bytes of a bf16 one, so
+                                  two of them keep half as many bytes in flight): tiles are attended in
+                                  groups of three.  Any other value, or 3 elsewhere: FCA_ERR_UNSUPPORTED */
 } fca_tensors;
 
 /* Offsets (in int32 units) of the arrays inside a built metadata workspace, for

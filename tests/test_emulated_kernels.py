@@ -79,7 +79,7 @@ SHARED_LAST_ITEMS = [
 ]
 
 
-def _decode(lib, w, chunk, rows, max_levels=4):
+def _decode(lib, w, chunk, rows, max_levels=4, tile_buffers=0, reproducible=0):
     S, mb = w.block_table.shape
     plan = make_plan(S, mb, w.num_q_heads, w.num_kv_heads, w.head_dim, chunk_tokens=chunk, rows_per_item=rows, max_levels=max_levels)
     layout = _lib.FcaMetaLayout()
@@ -101,7 +101,8 @@ def _decode(lib, w, chunk, rows, max_levels=4):
     t = _lib.FcaTensors(
         q.data_ptr(), q.stride(0), q.stride(1), kv.data_ptr(), kv.data_ptr() + kv.stride(0) * esz, kv.stride(1), kv.stride(2),
         _lib.FCA_FP8_E4M3 if kv.dtype == torch.float8_e4m3fn else _lib.FCA_BF16, 0, bt.data_ptr(), bt.stride(0),
-        None if ks is None else ks.data_ptr(), None if vs is None else vs.data_ptr(), float(w.scale), 0, EMU_WORKGROUPS,
+        None if ks is None else ks.data_ptr(), None if vs is None else vs.data_ptr(), float(w.scale), reproducible, EMU_WORKGROUPS,
+        tile_buffers,
     )
     out = guarded(torch.full((S, w.num_q_heads, w.head_dim), float("nan")).bfloat16())
     lse = guarded(torch.full((S, w.num_q_heads), float("nan"), dtype=torch.float32))
@@ -116,6 +117,14 @@ def _decode(lib, w, chunk, rows, max_levels=4):
     assert int(meta[layout.header + 3]) == 0
     assert int(meta[layout.coop_ctr : layout.coop_ctr + 1024].abs().sum()) == 0
     return md, out, lse
+
+
+def _second_partials(md):
+    """Partial rows of the launch that point at a second partial, written by the other wave of a
+    pair (the row's stored scale carries the pointer in its mantissa)."""
+    rows = md.plan.num_seqs * md.layout.max_partials * md.plan.num_q_heads
+    scales = md.partial_lse[: 2 * rows].view(torch.int32)[1::2]
+    return int(((scales & 0x007FFFFF) != 0).sum())
 
 
 def _check_nodes(md, w):
@@ -151,8 +160,69 @@ def test_long_items_shared_by_two_waves(emu, case):
     # enough items for the 32-row kernel to set the largest ones aside, one per pair of waves
     if rows == 32:
         assert md.header()["items"] * hkv >= 16 + 3 * 32
+        assert _second_partials(md) > 0  # some pair of waves did meet on its last item
     _check_nodes(md, w)
     assert_matches_oracle(out, lse, *oracle_for(w), what=f"seed {seed}")
+
+
+# ---- three register tile buffers for fp8 tiles at head size 128 (fca_tensors.tile_buffers = 3) -------
+@pytest.mark.parametrize(
+    "seed,hq,hkv,depth,fanout,len_range,leaf_range,chunk",
+    [
+        (17, 24, 4, 3, 4, (1, 150), (1, 100), 128),  # GQA 6: chunks of four tiles, a group and a tile
+        (41, 32, 8, 3, 3, (1, 400), (1, 200), 512),  # items of one to sixteen tiles: every remainder of three
+        (42, 8, 8, 2, 4, (1, 260), (1, 70), 96),  # no GQA: chunks of exactly one group
+        (43, 64, 2, 2, 3, (30, 700), (1, 40), 1024),  # one member per item, items of up to 22 tiles
+    ],
+)
+def test_three_tile_buffers_on_random_forests(emu, seed, hq, hkv, depth, fanout, len_range, leaf_range, chunk):
+    seg_len, paths = random_forest(random.Random(seed), depth, fanout, len_range, leaf_range)
+    w = make_forest_workload(
+        "random", seg_len, paths, torch.Generator().manual_seed(seed), num_q_heads=hq, num_kv_heads=hkv, head_dim=128,
+        kv_dtype=torch.float8_e4m3fn, device="cpu", poison_unused=True,
+    )
+    md, out, lse = _decode(emu, w, chunk, 32, tile_buffers=3)
+    _check_nodes(md, w)
+    assert_matches_oracle(out, lse, *oracle_for(w), what=f"seed {seed}, three tile buffers")
+    # With no item cut between two waves both kernels attend the same tiles in the same order,
+    # whatever buffer a tile travels through: the same bits.
+    _, out3, lse3 = _decode(emu, w, chunk, 32, tile_buffers=3, reproducible=1)
+    _, out2, lse2 = _decode(emu, w, chunk, 32, reproducible=1)
+    assert torch.equal(out3, out2) and torch.equal(lse3, lse2)
+
+
+@pytest.mark.parametrize("seed,samples,prefix_range,suffix_range,chunk", [(101, 5, (700, 2500), (40, 700), 512), (103, 3, (2000, 5000), (300, 1500), 1024)])
+def test_three_tile_buffers_on_items_shared_by_two_waves(emu, seed, samples, prefix_range, suffix_range, chunk):
+    """Last items long enough (four groups of three tiles) are attended by the two waves of a pair from
+    both ends, in groups of three."""
+    gen = torch.Generator().manual_seed(seed)
+    seg_len, paths = two_level_forest(gen, 6, samples, prefix_range, suffix_range)
+    w = make_forest_workload(
+        "two-level", seg_len, paths, gen, num_q_heads=24, num_kv_heads=4, head_dim=128, kv_dtype=torch.float8_e4m3fn, device="cpu",
+        poison_unused=True,
+    )
+    md, out, lse = _decode(emu, w, chunk, 32, tile_buffers=3)
+    assert md.header()["items"] * 4 >= 16 + 3 * 32
+    assert _second_partials(md) > 0  # some pair of waves did meet on its last item
+    _check_nodes(md, w)
+    assert_matches_oracle(out, lse, *oracle_for(w), what=f"seed {seed}, three tile buffers")
+
+
+def test_three_tile_buffers_are_refused_where_there_is_no_such_kernel(emu):
+    gen = torch.Generator().manual_seed(1)
+    seg_len, paths = two_level_forest(gen, 2, 2, (40, 80), (1, 30))
+    for kw, rows in (
+        (dict(head_dim=128, kv_dtype=torch.bfloat16), 32),
+        (dict(head_dim=64, kv_dtype=torch.float8_e4m3fn), 32),
+        (dict(head_dim=128, kv_dtype=torch.float8_e4m3fn), 64),
+        (dict(head_dim=256, kv_dtype=torch.float8_e4m3fn), 32),
+    ):
+        w = make_forest_workload("small", seg_len, paths, gen, num_q_heads=8, num_kv_heads=2, device="cpu", **kw)
+        with pytest.raises(AssertionError, match="tile_buffers 3"):
+            _decode(emu, w, 64, rows, tile_buffers=3)
+    w = make_forest_workload("small", seg_len, paths, gen, num_q_heads=8, num_kv_heads=2, head_dim=128, kv_dtype=torch.float8_e4m3fn, device="cpu")
+    with pytest.raises(AssertionError, match="tile_buffers 2"):
+        _decode(emu, w, 64, 32, tile_buffers=2)
 
 
 def test_entry_points_agree(emu):
@@ -259,8 +329,10 @@ def test_separate_passes_with_shared_items_equal_the_fused_step(emu):
         ("the same with an fp8 cache", lambda g: two_level_forest(g, 4, 8, (1024, 4096), (1, 1024)), torch.float8_e4m3fn, 32, 1.13),
         ("three levels", lambda g: three_level_forest(g, 1024, 4, 8, (2048, 6144), (1, 2048)), torch.bfloat16, 32, 1.14),
         ("a 32k-token prompt, 64-row tiles", lambda g: two_level_forest(g, 1, 16, (32768, 32768), (256, 4096)), torch.bfloat16, 64, 1.06),
+        # three tile buffers: a refill past an item's end repeats up to two tiles, and a wave ends on three
+        ("an fp8 cache, three tile buffers", lambda g: two_level_forest(g, 4, 8, (1024, 4096), (1, 1024)), torch.float8_e4m3fn, 32, 1.22),
     ],
-    ids=["c2-lengths", "c5-lengths", "c4-lengths", "c3-lengths"],
+    ids=["c2-lengths", "c5-lengths", "c4-lengths", "c3-lengths", "c5-lengths-3buf"],
 )
 def test_a_launch_requests_every_kv_block_about_once(emu, name, forest, kv_dtype, rows, bound):
     """The streaming kernels read their KV tiles with non-temporal loads, which the emulation counts:
@@ -276,7 +348,7 @@ def test_a_launch_requests_every_kv_block_about_once(emu, name, forest, kv_dtype
     seg_len, paths = forest(gen)
     w = make_forest_workload(name, seg_len, paths, gen, num_q_heads=8, num_kv_heads=2, head_dim=128, kv_dtype=kv_dtype, device="cpu")
     emu.emu_take_streamed_bytes()
-    md, out, lse = _decode(emu, w, 1024, rows)
+    md, out, lse = _decode(emu, w, 1024, rows, tile_buffers=3 if "three tile buffers" in name else 0)
     requested = emu.emu_take_streamed_bytes()
     merged = sum(md.seq_num_partials()) * w.num_q_heads * (w.head_dim * 2 + 8)  # partial rows and {lse, scale}, read once by the merge
     ratio = (requested - merged) / w.unique_kv_bytes

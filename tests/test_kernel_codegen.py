@@ -39,7 +39,7 @@ def _functions(asm):
 def test_attention_kernels_use_no_scratch(hipcc, tmp_path):
     # (the fp32 kernel keeps 32 rows of running maxima, sums and accumulators in registers,
     # and the merge its partial rows: in scratch they would be memory traffic per token)
-    sources = (("fca_attend32.hip", 8), ("fca_attend.hip", 12), ("fca_attend_f32.hip", 2), ("fca_merge.hip", 11))
+    sources = (("fca_attend32.hip", 10), ("fca_attend.hip", 12), ("fca_attend_f32.hip", 2), ("fca_merge.hip", 11))
     jobs = [
         subprocess.Popen(
             [hipcc, *FLAGS, "-c", "-Rpass-analysis=kernel-resource-usage", os.path.join(CSRC, src), "-o", str(tmp_path / (src + ".o"))],
@@ -67,24 +67,26 @@ def test_tile_loop_of_the_32_row_kernel_keeps_a_tile_in_flight(hipcc, tmp_path):
     res = subprocess.run([hipcc, *FLAGS, "-S", os.path.join(CSRC, "fca_attend32.hip"), "-o", str(out)], capture_output=True, text=True, cwd=CSRC)
     assert res.returncode == 0, res.stderr[-2000:]
     kernels = _functions(out.read_text())
-    # <head size 128, bf16, streaming>: the kernel of the headline configuration
-    name = "_ZN3fca19fca_attend32_kernelILi128ELb0ELb1EEEvNS_12AttendParamsE"
-    assert name in kernels, sorted(kernels)
-    loads_per_tile = 16  # 8 K + 2 x 4 V loads of 16 bytes per lane
-    seen = 0
-    for block in re.split(r"^\.LBB", kernels[name], flags=re.M):
-        header = block.split("\n", 1)[0]
-        if "Depth=2" not in header:  # the tile loop is the only loop nested inside the item loop that holds MFMAs
-            continue
-        if "v_mfma" not in block:
-            continue
-        waits = [int(n) for n in re.findall(r"s_waitcnt vmcnt\((\d+)\)", block)]
-        assert waits, header
-        # every wait inside the loop leaves at least the loads of one whole tile outstanding
-        assert min(waits) >= loads_per_tile, (header, waits)
-        assert len(re.findall(r"global_load_dwordx4", block)) == loads_per_tile, header
-        seen += 1
-    assert seen >= 1
+    # <head size 128, bf16, streaming, two tile buffers>: the kernel of the headline configuration
+    # (8 K + 2 x 4 V loads of 16 bytes per lane and tile; every wait inside the loop leaves at least
+    # the loads of one whole tile outstanding); the fp8 instances: tiles of 8 loads, one of them
+    # outstanding at every wait with two tile buffers, two of them with three
+    for template_args, loads_per_tile, tiles_left in (("ILi128ELb0ELb1ELi2E", 16, 1), ("ILi128ELb1ELb1ELi2E", 8, 1), ("ILi128ELb1ELb1ELi3E", 8, 2)):
+        name = f"_ZN3fca19fca_attend32_kernel{template_args}EEvNS_12AttendParamsE"
+        assert name in kernels, sorted(kernels)
+        seen = 0
+        for block in re.split(r"^\.LBB", kernels[name], flags=re.M):
+            header = block.split("\n", 1)[0]
+            if "Depth=2" not in header:  # the tile loop is the only loop nested inside the item loop that holds MFMAs
+                continue
+            if "v_mfma" not in block:
+                continue
+            waits = [int(n) for n in re.findall(r"s_waitcnt vmcnt\((\d+)\)", block)]
+            assert waits, header
+            assert min(waits) >= tiles_left * loads_per_tile, (name, header, waits)
+            assert len(re.findall(r"global_load_dwordx4", block)) == loads_per_tile, (name, header)
+            seen += 1
+        assert seen >= 1, name
 
 
 def test_split_attention_kernels_use_no_scratch_and_keep_their_ring_in_flight(hipcc, tmp_path):

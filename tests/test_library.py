@@ -26,7 +26,7 @@ def test_exports_every_declared_symbol(lib):
     assert declared == set(_lib.EXPORTS)
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.fca_version() == 104
+    assert lib.fca_version() == 105
 
 
 def test_struct_sizes_match_header():
