@@ -40,50 +40,78 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
   const RowElem* rows = static_cast<const RowElem*>(p.partial_out);
   const float2* lse_scale = reinterpret_cast<const float2*>(p.partial_lse);
 
-  // One online pass (running maximum, rescaled sum): the loads of successive partials do
-  // not depend on each other, so unrolling keeps several of them in flight.
+  // One online pass (running maximum, rescaled sum) over the partials in their order.  The
+  // partials are taken in batches of B: first every load of the batch is issued (the {lse,
+  // scale} pairs and the rows of its partials: none depends on another), then, with the row
+  // scales at hand, the loads of the second partials some of them point at, and only then the
+  // arithmetic, which has no branch in it.  Written as a loop of load-and-accumulate with the
+  // empty partials skipped, the compiler puts every load behind the test of the value loaded
+  // before it, and a row pays two memory round trips per partial, one after the other; this
+  // way it pays two per batch.
+  constexpr int B = F32 ? 4 : (SPLIT == 1 ? 8 : 4);
   float m = -INFINITY, wsum = 0.f;
   int stray = 0;  // a row scale pointed outside the rows set aside for second partials
   float acc[V];
 #pragma unroll
   for (int e = 0; e < V; ++e) acc[e] = 0.f;
+  // (an empty partial, lse = -inf, has weight 0 whatever its output holds, NaN included)
   auto take = [&](float l, float scale, const Row8& o) {
-    if (!(l > -INFINITY)) return;  // empty partial: weight 0, whatever its output holds
+    const bool live = l > -INFINITY;
     const float m_new = fmaxf(m, l);
-    const float keep = __expf(m - m_new);  // exp(-inf) = 0 on the first live partial
-    const float w = __expf(l - m_new);
+    const float keep = m > -INFINITY ? __expf(m - m_new) : 0.f;
+    const float w = live ? __expf(l - m_new) : 0.f;
     wsum = wsum * keep + w;
     const float ws = w * scale;
 #pragma unroll
-    for (int e = 0; e < V; ++e) acc[e] = acc[e] * keep + ws * (float)o[e];
+    for (int e = 0; e < V; ++e) acc[e] = acc[e] * keep + (live ? ws * (float)o[e] : 0.f);
     m = m_new;
   };
-#pragma unroll 4
-  for (int i = share; i < np; i += SPLIT) {
-    const int64_t pr = (base + i) * p.num_q_heads + hq;
-    // (read once: non-temporal, about 1 us per step at the Qwen3-4B shape)
-    typedef float f2v __attribute__((ext_vector_type(2)));
-    const f2v lsv = __builtin_nontemporal_load(reinterpret_cast<const f2v*>(lse_scale + pr));
-    const float2 ls = make_float2(lsv[0], lsv[1]);
-    const Row8 o = __builtin_nontemporal_load(reinterpret_cast<const Row8*>(rows + pr * D + sub * V));
-    // the scale is a power of two; its mantissa bits say where a second partial of the same
-    // chunk is (an item attended by two waves of the attention kernel), 0 = nowhere
-    const unsigned sbits = __float_as_uint(ls.y);
-    const unsigned tag = sbits & 0x007fffffu;
-    take(ls.x, __uint_as_float(sbits & 0xff800000u), o);
-    if (tag) {
-      // tag = 32 * (pair + 1) + row of the tile.  Only a
-      // buffer no attention launch has written (or one written for another plan) holds a tag
-      // that points anywhere else: it is not followed, and the output row leaves as NaN.
-      const int64_t rel = (int64_t)tag - 32;
-      if (rel >= 0 && rel < p.coop_rows) {
-        const int64_t br = p.coop_row0 + rel;
-        const float2 bls = lse_scale[br];
-        const Row8 bo = *reinterpret_cast<const Row8*>(rows + br * D + sub * V);
-        take(bls.x, __uint_as_float(__float_as_uint(bls.y) & 0xff800000u), bo);
-      } else {
-        stray = 1;
+  typedef float f2v __attribute__((ext_vector_type(2)));
+  for (int i0 = share; i0 < np; i0 += B * SPLIT) {
+    f2v ls[B], bls[B];
+    Row8 o[B], bo[B];
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      ls[j] = f2v{-INFINITY, 1.f};
+#pragma unroll
+      for (int e = 0; e < V; ++e) o[j][e] = 0;
+      const int i = i0 + j * SPLIT;
+      if (i < np) {
+        const int64_t pr = (base + i) * p.num_q_heads + hq;
+        // (read once: non-temporal, about 1 us per step at the Qwen3-4B shape)
+        ls[j] = __builtin_nontemporal_load(reinterpret_cast<const f2v*>(lse_scale + pr));
+        o[j] = __builtin_nontemporal_load(reinterpret_cast<const Row8*>(rows + pr * D + sub * V));
       }
+    }
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      bls[j] = f2v{-INFINITY, 1.f};
+#pragma unroll
+      for (int e = 0; e < V; ++e) bo[j][e] = 0;
+      // the scale is a power of two; its mantissa bits say where a second partial of the same
+      // chunk is (an item attended by two waves of the attention kernel), 0 = nowhere:
+      // tag = 32 * (pair + 1) + row of the tile.  Only a buffer no attention launch has
+      // written (or one written for another plan) holds a tag that points anywhere else: it is
+      // not followed, and the output row leaves as NaN.
+      const unsigned tag = __float_as_uint(ls[j][1]) & 0x007fffffu;
+      const int64_t rel = (int64_t)tag - 32;
+      if (tag != 0) {
+        if (rel >= 0 && rel < p.coop_rows) {
+          const int64_t br = p.coop_row0 + rel;
+          bls[j] = *reinterpret_cast<const f2v*>(lse_scale + br);
+          bo[j] = *reinterpret_cast<const Row8*>(rows + br * D + sub * V);
+        } else {
+          stray = 1;
+        }
+      }
+    }
+    // (the arithmetic stays behind the last load of the batch: moved up between the loads of the
+    // second partials it would wait for them one by one)
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      take(ls[j][0], __uint_as_float(__float_as_uint(ls[j][1]) & 0xff800000u), o[j]);
+      take(bls[j][0], __uint_as_float(__float_as_uint(bls[j][1]) & 0xff800000u), bo[j]);
     }
   }
   // combine the shares: the same update with a whole running result in place of one partial
