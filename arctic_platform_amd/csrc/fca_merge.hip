@@ -40,15 +40,20 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
   const RowElem* rows = static_cast<const RowElem*>(p.partial_out);
   const float2* lse_scale = reinterpret_cast<const float2*>(p.partial_lse);
 
-  // One online pass (running maximum, rescaled sum) over the partials in their order.  The
-  // partials are taken in batches of B: first every load of the batch is issued (the {lse,
-  // scale} pairs and the rows of its partials: none depends on another), then, with the row
-  // scales at hand, the loads of the second partials some of them point at, and only then the
-  // arithmetic, which has no branch in it.  Written as a loop of load-and-accumulate with the
-  // empty partials skipped, the compiler puts every load behind the test of the value loaded
-  // before it, and a row pays two memory round trips per partial, one after the other; this
-  // way it pays two per batch.
-  constexpr int B = F32 ? 4 : (SPLIT == 1 ? 8 : 4);
+  // One online pass (running maximum, rescaled sum).  The partials are taken in batches of B:
+  // first every load of the batch is issued, none under a condition (the {lse, scale} pairs,
+  // then the rows: none depends on another), then comes the arithmetic, which has no branch in
+  // it, and only then the second partials that some row scales of the batch point at, again
+  // all loads first.  Written as a loop of load-and-accumulate with the empty partials skipped,
+  // the compiler puts every load behind the test of the value loaded before it, and a row pays
+  // two memory round trips per partial, one after the other; this way it pays one per batch
+  // and one more where the batch has a second partial.  A batch is six partials (a row of the
+  // 512-sequence batch has two to six), four where SPLIT lane groups share a row.  One size only:
+  // with a second, smaller one for the last partials of a row the compiler lifts what the two
+  // have in common, the first load, above the choice between them and waits for it there.  The
+  // kernel stays well below 128 registers, i.e. at least four waves per SIMD: the 4096 waves that
+  // merge 512 sequences of 32 query heads are resident at once.
+  constexpr int B = F32 || SPLIT > 1 ? 4 : 6;
   float m = -INFINITY, wsum = 0.f;
   int stray = 0;  // a row scale pointed outside the rows set aside for second partials
   float acc[V];
@@ -68,50 +73,58 @@ __global__ __launch_bounds__(kMergeThreads) void fca_merge_kernel(MergeParams p)
   };
   typedef float f2v __attribute__((ext_vector_type(2)));
   for (int i0 = share; i0 < np; i0 += B * SPLIT) {
-    f2v ls[B], bls[B];
-    Row8 o[B], bo[B];
+    f2v ls[B];
+    Row8 o[B];
+    // A partial past the row's last one reads the last one again (the same lines, requested a
+    // moment earlier) and gets the weight of an empty partial below.
+    // (read once: non-temporal, about 1 us per step at the Qwen3-4B shape)
 #pragma unroll
     for (int j = 0; j < B; ++j) {
-      ls[j] = f2v{-INFINITY, 1.f};
-#pragma unroll
-      for (int e = 0; e < V; ++e) o[j][e] = 0;
-      const int i = i0 + j * SPLIT;
-      if (i < np) {
-        const int64_t pr = (base + i) * p.num_q_heads + hq;
-        // (read once: non-temporal, about 1 us per step at the Qwen3-4B shape)
-        ls[j] = __builtin_nontemporal_load(reinterpret_cast<const f2v*>(lse_scale + pr));
-        o[j] = __builtin_nontemporal_load(reinterpret_cast<const Row8*>(rows + pr * D + sub * V));
-      }
+      const int64_t pr = (base + min(i0 + j * SPLIT, np - 1)) * p.num_q_heads + hq;
+      ls[j] = __builtin_nontemporal_load(reinterpret_cast<const f2v*>(lse_scale + pr));
     }
 #pragma unroll
     for (int j = 0; j < B; ++j) {
-      bls[j] = f2v{-INFINITY, 1.f};
-#pragma unroll
-      for (int e = 0; e < V; ++e) bo[j][e] = 0;
-      // the scale is a power of two; its mantissa bits say where a second partial of the same
-      // chunk is (an item attended by two waves of the attention kernel), 0 = nowhere:
-      // tag = 32 * (pair + 1) + row of the tile.  Only a buffer no attention launch has
-      // written (or one written for another plan) holds a tag that points anywhere else: it is
-      // not followed, and the output row leaves as NaN.
-      const unsigned tag = __float_as_uint(ls[j][1]) & 0x007fffffu;
-      const int64_t rel = (int64_t)tag - 32;
-      if (tag != 0) {
-        if (rel >= 0 && rel < p.coop_rows) {
-          const int64_t br = p.coop_row0 + rel;
-          bls[j] = *reinterpret_cast<const f2v*>(lse_scale + br);
-          bo[j] = *reinterpret_cast<const Row8*>(rows + br * D + sub * V);
-        } else {
-          stray = 1;
-        }
-      }
+      const int64_t pr = (base + min(i0 + j * SPLIT, np - 1)) * p.num_q_heads + hq;
+      o[j] = __builtin_nontemporal_load(reinterpret_cast<const Row8*>(rows + pr * D + sub * V));
     }
-    // (the arithmetic stays behind the last load of the batch: moved up between the loads of the
-    // second partials it would wait for them one by one)
+    // (nothing that looks at a loaded value moves up between the loads of the batch)
     __builtin_amdgcn_sched_barrier(0);
+    // The scale is a power of two; its mantissa bits say where a second partial of the same
+    // chunk is (an item attended by two waves of the attention kernel), 0 = nowhere:
+    // tag = 32 * (pair + 1) + row of the tile.  Only a buffer no attention launch has written
+    // (or one written for another plan) holds a tag that points anywhere else: it is not
+    // followed, and the output row leaves as NaN.
+    int rel[B];  // row among the second partials, -1 = none
+    bool any = false;
 #pragma unroll
     for (int j = 0; j < B; ++j) {
+      if (i0 + j * SPLIT >= np) ls[j] = f2v{-INFINITY, 1.f};
+      const unsigned tag = __float_as_uint(ls[j][1]) & 0x007fffffu;
+      const bool follow = tag >= 32 && (int64_t)tag - 32 < p.coop_rows;
+      if (tag != 0 && !follow) stray = 1;
+      rel[j] = follow ? (int)tag - 32 : -1;
+      any |= follow;
       take(ls[j][0], __uint_as_float(__float_as_uint(ls[j][1]) & 0xff800000u), o[j]);
-      take(bls[j][0], __uint_as_float(__float_as_uint(bls[j][1]) & 0xff800000u), bo[j]);
+    }
+    // Second partials: about a quarter of the rows of a large batch have one.  Where a batch
+    // has any, all B are loaded (a partial without one reads its own row again, at weight 0: a
+    // row of its own, so that no single line is asked for by every wave) so that these loads too
+    // stand in a row with nothing between them.
+    if (any) {
+      f2v bls[B];
+      Row8 bo[B];
+#pragma unroll
+      for (int j = 0; j < B; ++j) {
+        const int64_t pr = (base + min(i0 + j * SPLIT, np - 1)) * p.num_q_heads + hq;
+        const int64_t br = rel[j] >= 0 ? p.coop_row0 + rel[j] : pr;
+        bls[j] = *reinterpret_cast<const f2v*>(lse_scale + br);
+        bo[j] = *reinterpret_cast<const Row8*>(rows + br * D + sub * V);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < B; ++j)
+        take(rel[j] >= 0 ? bls[j][0] : -INFINITY, __uint_as_float(__float_as_uint(bls[j][1]) & 0xff800000u), bo[j]);
     }
   }
   // combine the shares: the same update with a whole running result in place of one partial

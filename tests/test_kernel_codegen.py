@@ -92,22 +92,29 @@ def test_tile_loop_of_the_32_row_kernel_keeps_a_tile_in_flight(hipcc, tmp_path):
 def test_merge_issues_the_loads_of_a_batch_before_it_waits(hipcc, tmp_path):
     """The merge is a chain of memory round trips with little to hide them behind, so it takes its
     partials in batches: the {lse, scale} pairs and rows of a whole batch are requested back to
-    back, and the first wait on the vector-memory counter stands behind the last of them.  (A loop
-    that loads and accumulates one partial at a time compiles to a wait after every load.)"""
+    back, with no branch and no wait on the vector-memory counter between them, and so are the
+    second partials of a batch.  (A loop that loads and accumulates one partial at a time
+    compiles to a wait after every load.)  And it stays below 128 registers: four waves per
+    SIMD, so the 4096 waves of a 512-sequence batch at 32 query heads are resident at once."""
     out = tmp_path / "merge.s"
     res = subprocess.run([hipcc, *FLAGS, "-S", os.path.join(CSRC, "fca_merge.hip"), "-o", str(out)], capture_output=True, text=True, cwd=CSRC)
     assert res.returncode == 0, res.stderr[-2000:]
-    kernels = {k: v for k, v in _functions(out.read_text()).items() if "fca_merge_kernel" in k}
+    asm = out.read_text()
+    kernels = {k: v for k, v in _functions(asm).items() if "fca_merge_kernel" in k}
     assert len(kernels) == 10, sorted(kernels)
     for name, body in kernels.items():
         split, f32 = re.search(r"ILi\d+ELi(\d)ELb([01])E", name).groups()
-        batch = 4 if f32 == "1" or split != "1" else 8
-        lines = [l.strip() for l in body.splitlines()]
-        streamed = [i for i, l in enumerate(lines) if l.startswith("global_load") and l.split(";")[0].rstrip().endswith(" nt")]
-        # per partial: 8 bytes of {lse, scale} and the lane's 16 bytes of a half-precision row (32 bytes of an fp32 row: two loads)
-        assert len(streamed) == batch * (3 if f32 == "1" else 2), (name, len(streamed))
-        between = lines[streamed[0] : streamed[-1]]
-        assert not [l for l in between if l.startswith("s_waitcnt") and "vmcnt" in l], name
+        batch = 4 if f32 == "1" or split != "1" else 6
+        per_partial = 3 if f32 == "1" else 2  # 8 bytes of {lse, scale}; the lane's 16 bytes of a half-precision row, 32 of an fp32 one
+        lines = [l.split(";")[0].strip() for l in body.splitlines()]
+        streamed = [i for i, l in enumerate(lines) if l.startswith("global_load") and l.endswith(" nt")]
+        second = [i for i, l in enumerate(lines) if l.startswith("global_load_dwordx") and not l.endswith(" nt")]
+        assert len(streamed) == len(second) == batch * per_partial, (name, len(streamed), len(second))
+        for group in (streamed, second):
+            between = lines[group[0] : group[-1]]
+            assert not [l for l in between if (l.startswith("s_waitcnt") and "vmcnt" in l) or l.startswith("s_cbranch")], name
+        vgprs = int(re.search(r"\.amdhsa_kernel " + re.escape(name) + r"\n.*?\.amdhsa_next_free_vgpr (\d+)", asm, flags=re.S).group(1))
+        assert vgprs <= 128, (name, vgprs)
 
 
 def test_split_attention_kernels_use_no_scratch_and_keep_their_ring_in_flight(hipcc, tmp_path):
