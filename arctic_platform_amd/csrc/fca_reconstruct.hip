@@ -42,6 +42,8 @@ __global__ __launch_bounds__(256) void fca_sum_rows_kernel(const char* __restric
   const int64_t j = idx / groups;
   const int g = (int)(idx - j * groups);
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  // (unrolled: the rows of four copies are requested together; the sum keeps its order)
+#pragma unroll 4
   for (int k = offsets[j]; k < offsets[j + 1]; ++k) {
     const char* p = src + (int64_t)rows[k] * src_stride + (int64_t)g * kBytes;
     if constexpr (F32) {
