@@ -308,6 +308,9 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   } else {
     if (tid < kHeaderInts) hdr[tid] = 0;
     if (tid == 0) lds_tokens = 0;
+    // (the error flags set below must not be overtaken by the clearing of the header: other
+    // waves would otherwise be free to flag a bad length before wave 0 has cleared the word)
+    __syncthreads();
     for (int s = tid; s < S; s += kBuildThreads) {
       int len = p.seq_lens[s];
       if (len < 0 || len > p.plan.max_blocks * kBlock) {

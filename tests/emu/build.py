@@ -5,10 +5,12 @@ where the real library takes device pointers.  Test infrastructure only."""
 
 from __future__ import annotations
 
+import hashlib
 import os
 import re
 import shutil
 import subprocess
+import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
@@ -54,29 +56,51 @@ def transform(text: str) -> str:
 
 def build(replace: dict | None = None, tag: str = "emu") -> str:
     """Returns the path of the built library.  ``replace`` maps a file name of ``csrc`` to another
-    source to take in its place."""
+    source to take in its place.  The library is named after a hash of everything that goes into
+    it, is compiled in a directory of its own and moved into place when it is whole: a library
+    that is there is up to date, and processes that build at the same time do not meet."""
     cxx = compiler()
     if cxx is None:
         raise RuntimeError("no clang++ to build the emulation with")
     replace = replace or {}
+    flags = ["-std=c++17", "-O2", "-g", "-fPIC", "-w"]
+    sources = {}
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith(".hip"):
+            with open(replace.get(name, os.path.join(CSRC, name))) as f:
+                sources[name.replace(".hip", ".cpp")] = transform(f.read())
+    digest = hashlib.sha256(" ".join([cxx] + flags).encode())
+    for name, text in sources.items():
+        digest.update(name.encode() + b"\0" + text.encode())
+    for folder in (HERE, os.path.join(HERE, "hip"), CSRC, os.path.join(ROOT, "include")):
+        for name in sorted(os.listdir(folder)):
+            if name.endswith((".h", ".hpp")) or name == "hooks.cpp":
+                with open(os.path.join(folder, name), "rb") as f:
+                    digest.update(name.encode() + b"\0" + f.read())
     out_dir = os.path.join(HERE, "_build_" + tag)
     os.makedirs(out_dir, exist_ok=True)
-    jobs = []
-    for name in sorted(os.listdir(CSRC)):
-        if not name.endswith(".hip"):
-            continue
-        cpp = os.path.join(out_dir, name.replace(".hip", ".cpp"))
-        with open(replace.get(name, os.path.join(CSRC, name))) as f:
-            text = transform(f.read())
-        with open(cpp, "w") as f:
-            f.write(text)
-        obj = cpp[:-4] + ".o"
-        cmd = [cxx, "-std=c++17", "-O2", "-g", "-fPIC", "-w", "-c", f"-I{HERE}", f"-I{CSRC}", f"-I{ROOT}/include", cpp, "-o", obj]
-        jobs.append((subprocess.Popen(cmd), obj))
-    hooks = os.path.join(out_dir, "hooks.o")
-    jobs.append((subprocess.Popen([cxx, "-std=c++17", "-O2", "-fPIC", "-w", "-c", f"-I{HERE}", os.path.join(HERE, "hooks.cpp"), "-o", hooks]), hooks))
-    if any(p.wait() for p, _ in jobs):
-        raise RuntimeError("the emulation build failed to compile")
-    so = os.path.join(out_dir, "libzorro_fca_emu.so")
-    subprocess.run([cxx, "-shared", "-o", so] + [o for _, o in jobs], check=True)
+    so = os.path.join(out_dir, f"libzorro_fca_emu_{digest.hexdigest()[:16]}.so")
+    if os.path.exists(so):
+        return so
+    work = tempfile.mkdtemp(prefix="work_", dir=out_dir)
+    try:
+        jobs = []
+        for name, text in sources.items():
+            cpp = os.path.join(work, name)
+            with open(cpp, "w") as f:
+                f.write(text)
+            obj = cpp[:-4] + ".o"
+            jobs.append((subprocess.Popen([cxx, *flags, "-c", f"-I{HERE}", f"-I{CSRC}", f"-I{ROOT}/include", cpp, "-o", obj]), obj))
+        hooks = os.path.join(work, "hooks.o")
+        jobs.append((subprocess.Popen([cxx, "-std=c++17", "-O2", "-fPIC", "-w", "-c", f"-I{HERE}", os.path.join(HERE, "hooks.cpp"), "-o", hooks]), hooks))
+        if any(p.wait() for p, _ in jobs):
+            raise RuntimeError("the emulation build failed to compile")
+        whole = os.path.join(work, "lib.so")
+        subprocess.run([cxx, "-shared", "-o", whole] + [o for _, o in jobs], check=True)
+        os.replace(whole, so)
+    finally:
+        shutil.rmtree(work, ignore_errors=True)
+    for name in os.listdir(out_dir):  # libraries of earlier states of the sources
+        if name.startswith("libzorro_fca_emu") and os.path.join(out_dir, name) != so:
+            os.unlink(os.path.join(out_dir, name))
     return so

@@ -383,14 +383,18 @@ def _run_case(layout, hq, hkv, d, seed, strided=False, q_gain=1.0, window=None, 
     q64, k64, v64 = (x.double().requires_grad_() for x in (q, k, v))
     keep = dropout_keep_mask(seed + 5, dropout, hq, t) if dropout > 0 else None
     ro, rl = oracle_split(q64, k64, v64, layout, scale, window=window, keep=keep, dropout=dropout)
-    _close("out", out, ro, 2e-2 / max(1.0, float(ro.detach().abs().max())))
+    # Dropout scales the kept probabilities, and with them their gradients, by 1 / (1 - p) before
+    # they are rounded to bf16 for the matrix cores: the rounding noise grows by that factor, and
+    # so do the bounds (found on a single element of one layout that lay 10 % over the plain bound).
+    grow = 1.0 / (1.0 - dropout)
+    _close("out", out, ro, grow * 2e-2 / max(1.0, float(ro.detach().abs().max())))
     torch.testing.assert_close(lse[:, :t].T.cpu().double(), rl.detach(), rtol=1e-3, atol=1e-3)
     dout = torch.randn(t, hq, d, generator=torch.Generator().manual_seed(seed + 1)).bfloat16()
     ro.backward(dout.double())
     dq, dk, dv = split_attention_backward(dout.cuda(), qd, kd, vd, out, lse, L, scale, dropout=dropout, seed=seed + 5)
-    _close("dq", dq, q64.grad, 1e-2)
-    _close("dk", dk, k64.grad, 1e-2)
-    _close("dv", dv, v64.grad, 1e-2)
+    _close("dq", dq, q64.grad, grow * 1e-2)
+    _close("dk", dk, k64.grad, grow * 1e-2)
+    _close("dv", dv, v64.grad, grow * 1e-2)
 
 
 @pytest.mark.gpu

@@ -56,9 +56,10 @@ def test_attention_dropout_through_autograd_repeats_under_a_seed():
     keep = dropout_keep_mask(1234, 0.2, hq, total_tokens(layout))
     ro, _ = oracle_split(q64, k64, v64, layout, d**-0.5, keep=keep, dropout=0.2)
     (ro * w.double()).sum().backward()
-    _close("out", out, ro, 2e-2 / max(1.0, float(ro.detach().abs().max())))
+    grow = 1.0 / (1.0 - 0.2)  # the bounds grow with the scale of the kept probabilities (see _run_case)
+    _close("out", out, ro, grow * 2e-2 / max(1.0, float(ro.detach().abs().max())))
     for name, got, ref in (("dq", q.grad, q64.grad), ("dk", k.grad, k64.grad), ("dv", v.grad, v64.grad)):
-        _close(name, got, ref, 1e-2)
+        _close(name, got, ref, grow * 1e-2)
 
 
 @pytest.mark.gpu
