@@ -40,6 +40,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=720)
     ap.add_argument("--warmup", type=int, default=72)
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1-5 (default 2: the Qwen3-4B decode step); 6 = the forest of 2 with the heads of Qwen3.5 (Hq 16 / Hkv 2 / D 256)")
+    ap.add_argument("--shrink", type=int, default=1, help="the configuration with its group counts and lengths divided by this (to try the script out on a small batch; not a benchmark figure)")
+    ap.add_argument("--device", default="cuda:0", help="device of the tensors (the tests that run this script against the CPU emulation of the kernels pass cpu; the library itself takes device memory only)")
     ap.add_argument("--layers", type=int, default=36, help="attention layers sharing one metadata build")
     ap.add_argument("--kv-copies", type=int, default=4, help="distinct KV caches cycled over the layers")
     ap.add_argument("--chunk", type=int, default=0, help="split-K chunk in tokens (0 = default of the configuration)")
@@ -183,7 +185,7 @@ def main_query_runs(args):
 
     nseq, ql = (int(v) for v in args.query_runs.lower().split("x"))
     ctx, hq, hkv, d = args.context, 32, 8, 128
-    dev = torch.device("cuda:0")
+    dev = torch.device(args.device)
     gen = torch.Generator().manual_seed(4242)
     max_blocks = (ctx + ql + 15) // 16
     table = torch.randperm(nseq * max_blocks, generator=gen).to(torch.int32).view(nseq, max_blocks).to(dev)
@@ -328,7 +330,7 @@ def main_append(args):
 
     nseq, ql = (int(v) for v in args.append.lower().split("x"))
     ctx, hkv, d = args.context, 8, 128
-    dev = torch.device("cuda:0")
+    dev = torch.device(args.device)
     gen = torch.Generator().manual_seed(99)
     max_blocks = (ctx + ql + 15) // 16
     nblocks = nseq * max_blocks
@@ -426,7 +428,7 @@ def main_split_train(args):
         mk = lambda h: torch.randn(t, h, d, generator=gen).to(torch.bfloat16)
         return mk(hq), mk(hkv), mk(hkv), mk(hq)
 
-    dev = torch.device("cuda:0")
+    dev = torch.device(args.device)
     layout = SplitLayout(groups, device=dev)
     q, k, v, dout = (x.to(dev) for x in tensors(groups, 77))
     steps, warmup = min(args.steps, 20), min(args.warmup, 3)
@@ -516,9 +518,9 @@ def main():
     from arctic_platform_amd.forest import build_forest_metadata
     from arctic_platform_amd.workloads import make_config
 
-    dev = torch.device("cuda:0")
+    dev = torch.device(args.device)
     # configuration 1 is defined in fp32 (the CPU-runnable case) and runs on the all-fp32 path
-    w = make_config(args.config, device=dev)
+    w = make_config(args.config, device=dev, shrink=args.shrink)
     fp32 = w.q.dtype == torch.float32
     # distinct copies at distinct addresses: same values, so every copy gives the same result
     caches = [w.kv_cache] + [w.kv_cache.clone() for _ in range(max(1, args.kv_copies) - 1)]
@@ -643,7 +645,7 @@ def main():
         "dtype": "f32" if fp32 else "fp8 KV / bf16 MFMA / f32 accumulate" if args.config == 5 else "bf16 MFMA / f32 accumulate",
         "data": "synthetic",
         "config": {
-            "workload": w.name,
+            "workload": w.name + (f", every count and length divided by {args.shrink}" if args.shrink > 1 else ""),
             "seed": 1000 + args.config,
             "num_seqs": w.num_seqs,
             "unique_kv_bytes": unique_bytes,
@@ -672,7 +674,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(unique_bytes / (kern * 1e-6) / 1e9 / HBM_PEAK_GBS, 4) if kern else None,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, chunk, rows)),
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, chunk, rows)) if args.shrink == 1 else None,
             "launches_timed": len(kern_us),  # 0 under rocprofv3: the trace has the durations
             "launch_us_mean": round(kern, 2) if kern else None,
             "launch_us_min": round(min(kern_us), 2) if kern_us else None,
@@ -680,7 +682,7 @@ def main():
         },
     }
 
-    result["mfma_util"] = MEASURED_MFMA_UTIL.get((args.config, chunk, rows))
+    result["mfma_util"] = MEASURED_MFMA_UTIL.get((args.config, chunk, rows)) if args.shrink == 1 else None
     if split is not None:
         result["split_passes"] = split
 

@@ -55,8 +55,11 @@ def _emulated_device():
 
     arctic_platform_amd.split_attention.SplitLayout.__init__ = layout_on_the_host
     torch.Tensor.is_cuda = property(lambda self: True)
-    torch.Tensor.cuda = lambda self, *args, **kwargs: self
+    torch.Tensor.cuda = lambda self, *args, **kwargs: self.clone()  # (a copy, as the transfer to a device is)
     torch.cuda.synchronize = lambda *args, **kwargs: None
+    import types
+
+    torch.cuda.get_device_properties = lambda device=None: types.SimpleNamespace(multi_processor_count=8, name="CPU emulation")  # (emu.h: 8 CUs)
     return torch.device("cpu")
 
 

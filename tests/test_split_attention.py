@@ -545,7 +545,7 @@ def test_padded_batch_is_gathered_attended_and_scattered():
         assert float(got[~valid.cuda()].abs().max()) == 0.0, name
         _close(name, got[valid.cuda()], ref, 1e-2)
     with pytest.raises(ValueError, match="valid tokens"):
-        split_attention_padded(qd, kd, vd, torch.ones(tp, dtype=torch.bool, device="cuda"), SplitLayout(layout), 0.125)
+        split_attention_padded(qd, kd, vd, torch.ones(tp, dtype=torch.bool).cuda(), SplitLayout(layout), 0.125)
 
 
 @pytest.mark.gpu
