@@ -45,8 +45,11 @@ def test_a_selection_of_the_gpu_tests_passes_on_the_emulation():
     if emu_build.compiler() is None:
         pytest.skip("no clang++ to build the emulation with")
     emu_build.build()  # once, before the workers ask for it
+    import importlib.util
+
+    workers = ["-n", "4"] if importlib.util.find_spec("xdist") else []  # (one process takes about two minutes)
     res = subprocess.run(
-        [sys.executable, "-m", "pytest", *FILES, "-m", "gpu", "--on-emulation", "-x", "-q", "-n", "4", "-p", "no:cacheprovider", "-k", SELECTION],
+        [sys.executable, "-m", "pytest", *FILES, "-m", "gpu", "--on-emulation", "-x", "-q", *workers, "-p", "no:cacheprovider", "-k", SELECTION],
         cwd=ROOT, capture_output=True, text=True, timeout=1500,
     )
     tail = res.stdout[-3000:] + res.stderr[-1000:]
