@@ -30,6 +30,10 @@ def test_default_chunk_follows_the_head_size():
     assert cls(32, 8, 128, device="cpu").chunk_tokens == 1024
     assert cls(16, 2, 256, device="cpu").chunk_tokens == 512
     assert cls(16, 2, 256, device="cpu", forest_cascade_attn_configs='{"chunk_tokens": 2048}').chunk_tokens == 2048
+    assert cls(32, 8, 128, device="cpu").fp8_tile_buffers == 0
+    assert cls(32, 8, 128, device="cpu", forest_cascade_attn_configs='{"fp8_tile_buffers": 3}').fp8_tile_buffers == 3
+    with pytest.raises(ValueError, match="fp8_tile_buffers"):
+        cls(32, 8, 128, device="cpu", forest_cascade_attn_configs='{"fp8_tile_buffers": 2}')
 
 
 def test_config_string_and_rejections():
@@ -167,13 +171,17 @@ def test_lengths_beyond_the_block_table_are_refused_on_the_host():
 def test_decode_loop_through_backend(gpu, index):
     """Three decode steps: every step appends one token per sequence through forward()
     and attends; outputs are checked against the oracle on the cache as written."""
+    decode_loop(gpu, index, '{"chunk_tokens": 128}')
+
+
+def decode_loop(gpu, index, configs):
     from arctic_platform_amd.workloads import make_config
     from tests.helpers import assert_matches_oracle, oracle_for
     import dataclasses
 
     w = make_config(index, device=gpu, shrink=8)
     hq, hkv, d = w.num_q_heads, w.num_kv_heads, w.head_dim
-    builder = ForestCascadeAttentionBackend.get_builder_cls()(hq, hkv, d, device=gpu, forest_cascade_attn_configs='{"chunk_tokens": 128}')
+    builder = ForestCascadeAttentionBackend.get_builder_cls()(hq, hkv, d, device=gpu, forest_cascade_attn_configs=configs)
     impl = ForestCascadeAttentionBackend.get_impl_cls()(hq, d, w.scale, hkv, kv_cache_dtype="fp8" if index == 5 else "auto")
     layer = types.SimpleNamespace(k_scale=w.k_scale, v_scale=w.v_scale)
     # room for growth: spare blocks of the pool become the next private blocks
@@ -216,6 +224,7 @@ def test_decode_loop_through_backend(gpu, index):
         assert_matches_oracle(out.view(w.num_seqs, hq, d), ref_lse.float(), ref_out, ref_lse, what=f"C{index} step {step}")
         assert meta.forest.header()["shared_nodes"] == 8
         assert meta.forest.header()["updates"] == step, "steps after the first are length-only updates"
+    return meta
 
 
 @pytest.mark.gpu

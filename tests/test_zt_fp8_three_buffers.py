@@ -102,3 +102,12 @@ def test_other_caches_and_shapes_are_not_affected(gpu):
     )
     rc = lib.fca_prefix_pass(ctypes.byref(md.plan), ctypes.byref(t), md.meta.data_ptr(), md.partial_out.data_ptr(), md.partial_lse.data_ptr(), None)
     assert rc == -2 and b"tile_buffers 3" in lib.fca_last_error()  # FCA_ERR_UNSUPPORTED
+
+
+def test_decode_loop_through_the_adapter(gpu):
+    """The adapter's ``fp8_tile_buffers`` key reaches the launches of a decode loop on an fp8 cache
+    (three steps, every step appends a token per sequence and attends; checked against the oracle)."""
+    from tests.test_backend import decode_loop
+
+    meta = decode_loop(gpu, 5, '{"chunk_tokens": 256, "fp8_tile_buffers": 3}')
+    assert meta.forest.fp8_tile_buffers == 3
