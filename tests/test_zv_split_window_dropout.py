@@ -79,3 +79,21 @@ def test_sliding_window_through_autograd_and_on_long_responses():
     _close("out", out, ro, 2e-2 / max(1.0, float(ro.detach().abs().max())))
     for name, got, ref in (("dq", q.grad, q64.grad), ("dk", k.grad, k64.grad), ("dv", v.grad, v64.grad)):
         _close(name, got, ref, 1e-2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("window", [1, 20, 64, 300])
+def test_chunks_behind_a_context_under_a_window(window):
+    """A layout of response rows only (a prefill chunk behind a cached context) made with a
+    window: the chunk's rows equal the response rows of the whole computation under that window."""
+    from arctic_platform_amd.split_attention import split_attention_forward
+
+    layout = [(70, [45]), (0, [33]), (200, [64]), (16, [1])]
+    hq, hkv, d = 8, 2, 128
+    scale = d**-0.5
+    q_all, k, v = _inputs(layout, hq, hkv, d, 5, torch.bfloat16)
+    ro, _ = oracle_split(q_all.double(), k.double(), v.double(), layout, scale, window=window)
+    L = SplitLayout(layout, responses_only=True, sliding_window=window)
+    rows = torch.tensor(L.q_index()[: L.num_tokens] >= 0)
+    out, _ = split_attention_forward(q_all[rows].cuda(), k.cuda(), v.cuda(), L, scale)
+    _close("out", out, ro[rows], 2e-2 / max(1.0, float(ro.abs().max())))
