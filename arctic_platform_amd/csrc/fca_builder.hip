@@ -209,6 +209,7 @@ __device__ inline int run_head_lane(unsigned long long key, int lane) {
 __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p) {
   __shared__ int lds_scan[kBuildThreads];
   __shared__ int lds_mismatch;
+  __shared__ int lds_stale;  // the workspace holds no build of this plan (written before a barrier, read after it)
   __shared__ int lds_any;
   __shared__ int lds_listed;
   __shared__ int lds_hist[2 * kSizeBuckets];
@@ -270,9 +271,14 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
   // both are left in the workspace by the build.)
   bool reuse = false;
   if (p.try_update) {
-    if (tid == 0) lds_mismatch = (hdr[H_BUILT] != kBuiltMagic || hdr[H_PLAN_SIG] != plan_sig) ? 1 : 0;
+    if (tid == 0) {
+      lds_stale = (hdr[H_BUILT] != kBuiltMagic || hdr[H_PLAN_SIG] != plan_sig) ? 1 : 0;
+      lds_mismatch = 0;
+    }
     __syncthreads();
-    if (!lds_mismatch) {
+    // (a word of its own: lds_mismatch is raised inside the loop below, and a wave that looked at
+    // it to decide whether to enter the loop would race with the waves already in it)
+    if (!lds_stale) {
       const int gid = tid / kRowLanes, glane = tid % kRowLanes;
       for (int s = gid; s < S; s += kBuildThreads / kRowLanes) {
         const int len = p.seq_lens[s];
@@ -285,7 +291,7 @@ __global__ __launch_bounds__(kBuildThreads) void fca_build_kernel(BuildParams p)
       }
     }
     __syncthreads();
-    reuse = !lds_mismatch;
+    reuse = !lds_stale && !lds_mismatch;
   }
 
   int node_base = 0, member_base = 0, levels = 0;

@@ -76,6 +76,10 @@ struct Block {
 inline Block* B = nullptr;
 inline Fiber* F = nullptr;
 inline bool dma_late = false;  // direct-to-LDS loads land at the wait that covers them instead of at once
+// Order in which the scheduler below takes what the hardware runs at the same time.  Bit 0: the waves of a
+// workgroup from the last to the first in every round; bit 1: the workgroups of a launch from the last to the
+// first.  A kernel must not care: one that does relies on an order the hardware does not promise.
+inline int run_order = 0;
 inline unsigned long long streamed_bytes = 0;  // bytes requested by non-temporal loads (the kernels stream their KV tiles with them)
 inline long n_progress = 0;  // rendezvous completed and fibers finished (deadlock detection)
 
@@ -269,7 +273,8 @@ inline void launch(dim3 grid, dim3 block, K&& kernel) {
   B = &blk;
   for (unsigned bz = 0; bz < grid.z; ++bz)
     for (unsigned by = 0; by < grid.y; ++by)
-      for (unsigned bx = 0; bx < grid.x; ++bx) {
+      for (unsigned bi = 0; bi < grid.x; ++bi) {
+        const unsigned bx = (run_order & 2) ? grid.x - 1 - bi : bi;
         blk.bid = dim3(bx, by, bz);
         blk.waves.assign((nthreads + 63) / 64, WaveSync());
         blk.groups.assign((nthreads + 63) / 64 * 7 * 64, GroupSync());
@@ -290,7 +295,10 @@ inline void launch(dim3 grid, dim3 block, K&& kernel) {
         while (left > 0) {
           const long before = n_progress;
           left = 0;
-          for (int t = 0; t < nthreads; ++t) {
+          const int nw = (nthreads + 63) / 64;
+          for (int i = 0; i < nw * 64; ++i) {
+            const int t = ((run_order & 1) ? nw - 1 - i / 64 : i / 64) * 64 + i % 64;
+            if (t >= nthreads) continue;
             Fiber& f = blk.fibers[t];
             if (f.done) continue;
             F = &f;

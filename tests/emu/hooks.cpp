@@ -11,3 +11,6 @@ extern "C" unsigned long long emu_take_streamed_bytes() {
   emu::streamed_bytes = 0;
   return n;
 }
+
+// Bit 0: waves of a workgroup run from the last to the first; bit 1: workgroups of a launch likewise.
+extern "C" void emu_set_run_order(int order) { emu::run_order = order; }
