@@ -78,7 +78,8 @@ inline Fiber* F = nullptr;
 inline bool dma_late = false;  // direct-to-LDS loads land at the wait that covers them instead of at once
 // Order in which the scheduler below takes what the hardware runs at the same time.  Bit 0: the waves of a
 // workgroup from the last to the first in every round; bit 1: the workgroups of a launch from the last to the
-// first.  A kernel must not care: one that does relies on an order the hardware does not promise.
+// first; bit 2: the lanes of a wave from the last to the first between two rendezvous.  A kernel must not
+// care: one that does relies on an order the hardware does not promise.
 inline int run_order = 0;
 inline unsigned long long streamed_bytes = 0;  // bytes requested by non-temporal loads (the kernels stream their KV tiles with them)
 inline long n_progress = 0;  // rendezvous completed and fibers finished (deadlock detection)
@@ -297,7 +298,7 @@ inline void launch(dim3 grid, dim3 block, K&& kernel) {
           left = 0;
           const int nw = (nthreads + 63) / 64;
           for (int i = 0; i < nw * 64; ++i) {
-            const int t = ((run_order & 1) ? nw - 1 - i / 64 : i / 64) * 64 + i % 64;
+            const int t = ((run_order & 1) ? nw - 1 - i / 64 : i / 64) * 64 + ((run_order & 4) ? 63 - i % 64 : i % 64);
             if (t >= nthreads) continue;
             Fiber& f = blk.fibers[t];
             if (f.done) continue;

@@ -12,5 +12,5 @@ extern "C" unsigned long long emu_take_streamed_bytes() {
   return n;
 }
 
-// Bit 0: waves of a workgroup run from the last to the first; bit 1: workgroups of a launch likewise.
+// Bit 0: waves of a workgroup run from the last to the first; bit 1: workgroups of a launch; bit 2: lanes of a wave.
 extern "C" void emu_set_run_order(int order) { emu::run_order = order; }

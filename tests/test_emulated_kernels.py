@@ -61,8 +61,8 @@ def emu():
     lib = _lib.declare_signatures(ctypes.CDLL(emu_build.build()))
     lib.emu_set_dma_late.argtypes = [ctypes.c_int]
     lib.emu_set_dma_late.restype = None
-    # FCA_EMU_RUN_ORDER = 1, 2 or 3 runs the same tests with the waves of a workgroup, the workgroups of a
-    # launch, or both taken from the last to the first: no kernel may care
+    # FCA_EMU_RUN_ORDER runs the same tests with the waves of a workgroup (bit 0), the workgroups of a launch
+    # (bit 1) or the lanes of a wave (bit 2) taken from the last to the first: no kernel may care
     lib.emu_set_run_order(int(os.environ.get("FCA_EMU_RUN_ORDER", "0")))
     yield lib
     lib.emu_set_dma_late(0)
