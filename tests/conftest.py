@@ -44,6 +44,7 @@ def _emulated_device():
         pytest.skip("no clang++ to build the emulation with")
     lib = _lib.declare_signatures(ctypes.CDLL(emu_build.build()))
     lib.emu_set_run_order(int(os.environ.get("FCA_EMU_RUN_ORDER", "0")))  # (see tests/test_emulated_kernels.py)
+    lib.emu_set_host_threads(int(os.environ.get("FCA_EMU_THREADS", "1")))
     _lib.load_library = lambda: lib
     for module in ("cache", "forest", "ops", "reconstruct", "split_attention"):
         setattr(getattr(arctic_platform_amd, module), "_stream_ptr", lambda device: None)

@@ -1,7 +1,9 @@
 // CPU stand-in for the parts of HIP that the kernels of this library use, for tests without a GPU.
 // A workgroup runs as cooperative fibers, one per thread, on one host thread; every cross-lane
 // operation (shuffles, ballots, readfirstlane, MFMA, the wave barrier) and every workgroup barrier
-// is a rendezvous of the lanes concerned; workgroups of a launch run one after the other.  What the
+// is a rendezvous of the lanes concerned; workgroups of a launch run one after the other, or, with
+// emu::host_threads above 1, several at a time on host threads of their own (LDS is per host thread,
+// atomics are the host's), which is how the workgroups of a persistent grid meet on a GPU.  What the
 // kernels see of the GPU's data layouts (the operand and result registers of
 // mfma_f32_32x32x16_bf16, v_permlane32_swap, the fp8 conversions, direct-to-LDS loads) follows
 // the instruction set.  It checks kernel logic: indices, rings, masks, the dealing of work, and,
@@ -9,6 +11,7 @@
 // speed, about the memory model between workgroups, or about what the compiler makes of the code.
 // Test infrastructure only: nothing in the library includes it.
 #pragma once
+#include <sys/mman.h>
 #include <ucontext.h>
 
 #include <cmath>
@@ -16,7 +19,10 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <algorithm>
+#include <atomic>
 #include <functional>
+#include <thread>
 #include <vector>
 
 struct dim3 {
@@ -33,7 +39,7 @@ inline const char* hipGetErrorString(hipError_t) { return "emu"; }
 #define __global__
 #define __device__
 #define __host__
-#define __shared__ static
+#define __shared__ static thread_local
 #define __launch_bounds__(...)
 
 namespace emu {
@@ -55,9 +61,25 @@ struct DmaWrite {
   unsigned char data[16];
   int bytes;
 };
+// a fiber's stack: mapped, not filled, so that only the pages a fiber touches cost anything
+struct Stack {
+  char* base = nullptr;
+  Stack() {
+    void* p = mmap(nullptr, kStack, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+    if (p == MAP_FAILED) abort();
+    base = static_cast<char*>(p);
+  }
+  Stack(const Stack&) = delete;
+  Stack(Stack&& o) noexcept : base(o.base) { o.base = nullptr; }
+  ~Stack() {
+    if (base) munmap(base, kStack);
+  }
+  char* data() { return base; }
+  size_t size() const { return kStack; }
+};
 struct Fiber {
   ucontext_t ctx;
-  std::vector<char> stack;
+  Stack stack;
   dim3 tid;
   int lane = 0, wave = 0;
   bool done = false;
@@ -73,16 +95,17 @@ struct Block {
   ucontext_t sched;
   std::function<void()> body;
 };
-inline Block* B = nullptr;
-inline Fiber* F = nullptr;
+inline thread_local Block* B = nullptr;
+inline thread_local Fiber* F = nullptr;
+inline int host_threads = 1;  // workgroups of a launch that run at the same time
 inline bool dma_late = false;  // direct-to-LDS loads land at the wait that covers them instead of at once
 // Order in which the scheduler below takes what the hardware runs at the same time.  Bit 0: the waves of a
 // workgroup from the last to the first in every round; bit 1: the workgroups of a launch from the last to the
 // first; bit 2: the lanes of a wave from the last to the first between two rendezvous.  A kernel must not
 // care: one that does relies on an order the hardware does not promise.
 inline int run_order = 0;
-inline unsigned long long streamed_bytes = 0;  // bytes requested by non-temporal loads (the kernels stream their KV tiles with them)
-inline long n_progress = 0;  // rendezvous completed and fibers finished (deadlock detection)
+inline std::atomic<unsigned long long> streamed_bytes{0};  // bytes requested by non-temporal loads (the kernels stream their KV tiles with them)
+inline thread_local long n_progress = 0;  // rendezvous completed and fibers finished (deadlock detection)
 
 inline void yield() {
   swapcontext(&F->ctx, &B->sched);
@@ -229,7 +252,7 @@ inline f32x16_t mfma_32x32x16_bf16(bf16x8_t a, bf16x8_t b, f32x16_t c, int, int,
 }
 
 // ---- direct-to-LDS loads -------------------------------------------------------------------
-inline char lds_anchor;  // LDS "addresses" are offsets from here (static storage lies within 2 GiB of it)
+inline thread_local char lds_anchor;  // LDS "addresses" are offsets from here (static storage lies within 2 GiB of it)
 inline unsigned lds_address(const void* p) { return (unsigned)(int)((const char*)p - &lds_anchor); }
 inline void dma_to_lds(const void* src, unsigned slot, int bytes) {
   char* dst = &lds_anchor + (int)slot + F->lane * bytes;
@@ -262,70 +285,83 @@ inline void fiber_entry() {
   for (;;) yield();
 }
 
-template <class K>
-inline void launch(dim3 grid, dim3 block, K&& kernel) {
+// the workgroups of a launch that this host thread takes from `next`, one after the other
+inline void run_blocks(dim3 grid, dim3 block, const std::function<void()>& kernel, std::atomic<unsigned>& next) {
   const int nthreads = block.x * block.y * block.z;
+  const unsigned nblocks = grid.x * grid.y * grid.z;
   Block blk;
   blk.gdim = grid;
   blk.bdim = block;
   blk.body = kernel;
   blk.fibers.resize(nthreads);
-  for (auto& f : blk.fibers) f.stack.resize(kStack);
   B = &blk;
-  for (unsigned bz = 0; bz < grid.z; ++bz)
-    for (unsigned by = 0; by < grid.y; ++by)
-      for (unsigned bi = 0; bi < grid.x; ++bi) {
-        const unsigned bx = (run_order & 2) ? grid.x - 1 - bi : bi;
-        blk.bid = dim3(bx, by, bz);
-        blk.waves.assign((nthreads + 63) / 64, WaveSync());
-        blk.groups.assign((nthreads + 63) / 64 * 7 * 64, GroupSync());
-        blk.b_arrived = 0, blk.b_gen = 0, blk.b_active = nthreads;
-        for (int t = 0; t < nthreads; ++t) {
-          Fiber& f = blk.fibers[t];
-          f.tid = dim3(t % block.x, (t / block.x) % block.y, t / (block.x * block.y));
-          f.lane = t & 63, f.wave = t >> 6, f.done = false;
-          f.dma.clear();
-          ++blk.waves[f.wave].active;
-          getcontext(&f.ctx);
-          f.ctx.uc_stack.ss_sp = f.stack.data();
-          f.ctx.uc_stack.ss_size = f.stack.size();
-          f.ctx.uc_link = &blk.sched;
-          makecontext(&f.ctx, fiber_entry, 0);
-        }
-        int left = nthreads;
-        while (left > 0) {
-          const long before = n_progress;
-          left = 0;
-          const int nw = (nthreads + 63) / 64;
-          for (int i = 0; i < nw * 64; ++i) {
-            const int t = ((run_order & 1) ? nw - 1 - i / 64 : i / 64) * 64 + ((run_order & 4) ? 63 - i % 64 : i % 64);
-            if (t >= nthreads) continue;
-            Fiber& f = blk.fibers[t];
-            if (f.done) continue;
-            F = &f;
-            swapcontext(&blk.sched, &f.ctx);
-            if (!f.done) ++left;
-          }
-          if (left > 0 && n_progress == before) {
-            // a full round in which nobody got anywhere: lanes wait for lanes that went another way
-            fprintf(stderr, "emu: deadlock in block (%u, %u): %d threads wait at rendezvous that cannot complete\n", bx, by, left);
-            for (size_t wv = 0; wv < blk.waves.size(); ++wv)
-              fprintf(stderr, "  wave %zu: arrived %d of %d active\n", wv, blk.waves[wv].arrived, blk.waves[wv].active);
-            fprintf(stderr, "  block barrier: arrived %d of %d\n", blk.b_arrived, blk.b_active);
-            abort();
-          }
-        }
+  for (;;) {
+    const unsigned taken = next.fetch_add(1);
+    if (taken >= nblocks) break;
+    const unsigned bi = (run_order & 2) ? nblocks - 1 - taken : taken;
+    const unsigned bx = bi % grid.x, by = (bi / grid.x) % grid.y, bz = bi / (grid.x * grid.y);
+    blk.bid = dim3(bx, by, bz);
+    blk.waves.assign((nthreads + 63) / 64, WaveSync());
+    blk.groups.assign((nthreads + 63) / 64 * 7 * 64, GroupSync());
+    blk.b_arrived = 0, blk.b_gen = 0, blk.b_active = nthreads;
+    for (int t = 0; t < nthreads; ++t) {
+      Fiber& f = blk.fibers[t];
+      f.tid = dim3(t % block.x, (t / block.x) % block.y, t / (block.x * block.y));
+      f.lane = t & 63, f.wave = t >> 6, f.done = false;
+      f.dma.clear();
+      ++blk.waves[f.wave].active;
+      getcontext(&f.ctx);
+      f.ctx.uc_stack.ss_sp = f.stack.data();
+      f.ctx.uc_stack.ss_size = f.stack.size();
+      f.ctx.uc_link = &blk.sched;
+      makecontext(&f.ctx, fiber_entry, 0);
+    }
+    int left = nthreads;
+    while (left > 0) {
+      const long before = n_progress;
+      left = 0;
+      const int nw = (nthreads + 63) / 64;
+      for (int i = 0; i < nw * 64; ++i) {
+        const int t = ((run_order & 1) ? nw - 1 - i / 64 : i / 64) * 64 + ((run_order & 4) ? 63 - i % 64 : i % 64);
+        if (t >= nthreads) continue;
+        Fiber& f = blk.fibers[t];
+        if (f.done) continue;
+        F = &f;
+        swapcontext(&blk.sched, &f.ctx);
+        if (!f.done) ++left;
       }
+      if (left > 0 && n_progress == before) {
+        // a full round in which nobody got anywhere: lanes wait for lanes that went another way
+        fprintf(stderr, "emu: deadlock in block (%u, %u): %d threads wait at rendezvous that cannot complete\n", bx, by, left);
+        for (size_t wv = 0; wv < blk.waves.size(); ++wv)
+          fprintf(stderr, "  wave %zu: arrived %d of %d active\n", wv, blk.waves[wv].arrived, blk.waves[wv].active);
+        fprintf(stderr, "  block barrier: arrived %d of %d\n", blk.b_arrived, blk.b_active);
+        abort();
+      }
+    }
+  }
   B = nullptr;
   F = nullptr;
+}
+
+template <class K>
+inline void launch(dim3 grid, dim3 block, K&& kernel) {
+  const std::function<void()> body = kernel;
+  const unsigned nblocks = grid.x * grid.y * grid.z;
+  std::atomic<unsigned> next{0};
+  const unsigned helpers = host_threads > 1 ? std::min<unsigned>(host_threads, nblocks) - 1 : 0;
+  std::vector<std::thread> pool;
+  for (unsigned i = 0; i < helpers; ++i) pool.emplace_back([&] { run_blocks(grid, block, body, next); });
+  run_blocks(grid, block, body, next);
+  for (auto& t : pool) t.join();
 }
 
 }  // namespace emu
 
 // device-library functions and builtins that the kernels use
 #define __HIP_MEMORY_SCOPE_AGENT 0
-#define __hip_atomic_store(p, v, order, scope) (*(p) = (v))
-#define __hip_atomic_load(p, order, scope) (*(p))
+#define __hip_atomic_store(p, v, order, scope) __atomic_store_n(p, v, __ATOMIC_SEQ_CST)
+#define __hip_atomic_load(p, order, scope) __atomic_load_n(p, __ATOMIC_SEQ_CST)
 inline unsigned __float_as_uint(float f) { unsigned u; memcpy(&u, &f, 4); return u; }
 inline float __uint_as_float(unsigned u) { float f; memcpy(&f, &u, 4); return f; }
 template <class T> inline T min(T a, T b) { return b < a ? b : a; }
@@ -362,11 +398,23 @@ inline int __popc(unsigned v) { return __builtin_popcount(v); }
 inline int __ffsll(unsigned long long v) { return __builtin_ffsll((long long)v); }
 inline float __expf(float x) { return expf(x); }
 inline float __logf(float x) { return logf(x); }
-template <class T> inline T atomicAdd(T* p, T v) { T o = *p; *p = o + v; return o; }
-template <class T> inline T atomicOr(T* p, T v) { T o = *p; *p = o | v; return o; }
-template <class T> inline T atomicMin(T* p, T v) { T o = *p; if (v < o) *p = v; return o; }
-template <class T> inline T atomicMax(T* p, T v) { T o = *p; if (o < v) *p = v; return o; }
-template <class T> inline T atomicCAS(T* p, T c, T v) { T o = *p; if (o == c) *p = v; return o; }
+// (integers only: the kernels have no other atomics; the host's own, since workgroups may run on several host threads)
+template <class T> inline T atomicAdd(T* p, T v) { return __atomic_fetch_add(p, v, __ATOMIC_SEQ_CST); }
+template <class T> inline T atomicOr(T* p, T v) { return __atomic_fetch_or(p, v, __ATOMIC_SEQ_CST); }
+template <class T> inline T atomicMin(T* p, T v) {
+  T o = __atomic_load_n(p, __ATOMIC_SEQ_CST);
+  while (v < o && !__atomic_compare_exchange_n(p, &o, v, false, __ATOMIC_SEQ_CST, __ATOMIC_SEQ_CST)) {}
+  return o;
+}
+template <class T> inline T atomicMax(T* p, T v) {
+  T o = __atomic_load_n(p, __ATOMIC_SEQ_CST);
+  while (o < v && !__atomic_compare_exchange_n(p, &o, v, false, __ATOMIC_SEQ_CST, __ATOMIC_SEQ_CST)) {}
+  return o;
+}
+template <class T> inline T atomicCAS(T* p, T c, T v) {
+  __atomic_compare_exchange_n(p, &c, v, false, __ATOMIC_SEQ_CST, __ATOMIC_SEQ_CST);
+  return c;
+}
 inline int atomicAdd(int* p, unsigned v) { return atomicAdd<int>(p, (int)v); }
 #define __align__(n) __attribute__((aligned(n)))
 #define HIP_SYMBOL(x) (&x)

@@ -64,8 +64,20 @@ def emu():
     # FCA_EMU_RUN_ORDER runs the same tests with the waves of a workgroup (bit 0), the workgroups of a launch
     # (bit 1) or the lanes of a wave (bit 2) taken from the last to the first: no kernel may care
     lib.emu_set_run_order(int(os.environ.get("FCA_EMU_RUN_ORDER", "0")))
+    # FCA_EMU_THREADS = n runs n workgroups of a launch at the same time on host threads of their own
+    # (default: one after the other, which repeats bit for bit)
+    lib.emu_set_host_threads(int(os.environ.get("FCA_EMU_THREADS", "1")))
     yield lib
     lib.emu_set_dma_late(0)
+
+
+@pytest.fixture(params=[1, 8], ids=["one-after-the-other", "eight-at-a-time"])
+def workgroups_at_a_time(emu, request):
+    """Workgroups of a launch one after the other, or eight at a time on host threads of their own:
+    then the waves of different workgroups really do draw tickets and claim tiles against each other."""
+    emu.emu_set_host_threads(request.param)
+    yield request.param
+    emu.emu_set_host_threads(int(os.environ.get("FCA_EMU_THREADS", "1")))
 
 
 def _ok(lib, rc):
@@ -152,7 +164,7 @@ def test_random_forests_decode(emu, case):
 
 
 @pytest.mark.parametrize("case", SHARED_LAST_ITEMS, ids=lambda c: f"seed{c[0]}")
-def test_long_items_shared_by_two_waves(emu, case):
+def test_long_items_shared_by_two_waves(emu, case, workgroups_at_a_time):
     seed, hq, hkv, d, kv_dtype, samples, prefix_range, suffix_range, chunk, rows = case
     gen = torch.Generator().manual_seed(seed)
     seg_len, paths = two_level_forest(gen, 6, samples, prefix_range, suffix_range)
@@ -166,7 +178,11 @@ def test_long_items_shared_by_two_waves(emu, case):
         assert md.header()["items"] * hkv >= 16 + 3 * 32
         assert _second_partials(md) > 0  # some pair of waves did meet on its last item
     _check_nodes(md, w)
-    assert_matches_oracle(out, lse, *oracle_for(w), what=f"seed {seed}")
+    ref = oracle_for(w)
+    assert_matches_oracle(out, lse, *ref, what=f"seed {seed}")
+    for again in range(4 if workgroups_at_a_time > 1 else 0):  # (where the claims of a pair meet differs from run to run)
+        md, out, lse = _decode(emu, w, chunk, rows)
+        assert_matches_oracle(out, lse, *ref, what=f"seed {seed}, run {again + 2}")
 
 
 # ---- three register tile buffers for fp8 tiles at head size 128 (fca_tensors.tile_buffers = 3) -------
@@ -196,7 +212,7 @@ def test_three_tile_buffers_on_random_forests(emu, seed, hq, hkv, depth, fanout,
 
 
 @pytest.mark.parametrize("seed,samples,prefix_range,suffix_range,chunk", [(101, 5, (700, 2500), (40, 700), 512)])
-def test_three_tile_buffers_on_items_shared_by_two_waves(emu, seed, samples, prefix_range, suffix_range, chunk):
+def test_three_tile_buffers_on_items_shared_by_two_waves(emu, seed, samples, prefix_range, suffix_range, chunk, workgroups_at_a_time):
     """Last items long enough (four groups of three tiles) are attended by the two waves of a pair from
     both ends, in groups of three."""
     gen = torch.Generator().manual_seed(seed)
@@ -209,7 +225,11 @@ def test_three_tile_buffers_on_items_shared_by_two_waves(emu, seed, samples, pre
     assert md.header()["items"] * 4 >= 16 + 3 * 32
     assert _second_partials(md) > 0  # some pair of waves did meet on its last item
     _check_nodes(md, w)
-    assert_matches_oracle(out, lse, *oracle_for(w), what=f"seed {seed}, three tile buffers")
+    ref = oracle_for(w)
+    assert_matches_oracle(out, lse, *ref, what=f"seed {seed}, three tile buffers")
+    for again in range(4 if workgroups_at_a_time > 1 else 0):  # (where the claims of a pair meet differs from run to run)
+        md, out, lse = _decode(emu, w, chunk, 32, tile_buffers=3)
+        assert_matches_oracle(out, lse, *ref, what=f"seed {seed}, three tile buffers, run {again + 2}")
 
 
 def test_three_tile_buffers_are_refused_where_there_is_no_such_kernel(emu):
